@@ -1,0 +1,117 @@
+/* libsglq — C ABI of the MI355X (gfx950) W8A8 quantized-linear kernels.
+ *
+ * Every entry point takes raw device pointers, sizes, strides (in elements) and
+ * a HIP stream (hipStream_t passed as void*; NULL = the null stream).  Nothing
+ * is allocated, retained or synchronised: work is enqueued on the stream and
+ * the call returns.  Return value: 0 on success, otherwise one of the SGLQ_E*
+ * codes; sglq_last_error() then holds a message for the calling thread.
+ *
+ * "Reference" below is sgl-kernel 0.3.3 inside walker-ai/sglang; each entry
+ * point names the torch op it stands in for.
+ */
+#ifndef SGLQ_H
+#define SGLQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SGLQ_OK 0
+#define SGLQ_EINVAL 1      /* bad shape / stride / alignment / null pointer */
+#define SGLQ_EUNSUPPORTED 2 /* valid in the reference but not built here */
+#define SGLQ_ELAUNCH 3     /* hipGetLastError() after the launch was not hipSuccess */
+
+/* element type codes for 16/32-bit floating inputs and outputs */
+#define SGLQ_BF16 0
+#define SGLQ_FP16 1
+#define SGLQ_FP32 2
+#define SGLQ_I32 3 /* raw accumulators (sglq_int8_mm_i32 only) */
+
+const char* sglq_last_error(void);
+int sglq_abi_version(void);
+
+/* Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_fp8
+ * (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217,230-240; schema
+ * sgl-kernel/csrc/common_extension.cc:116-119).  The UE8M0 packed-scale mode
+ * (scale_ue8m0=true) is not built.
+ *
+ * input  [num_tokens, hidden] contiguous, in_dtype in {BF16, FP16, FP32}
+ * output_q  same shape, one e4m3fn byte per element
+ * output_s  fp32; element (row, g) lives at output_s[row*s_stride_row + g*s_stride_col],
+ *           which covers the reference's row-major, column-major and padded
+ *           column-major scale buffers (per_token_group_quant_8bit.cu:54-64,153-156)
+ * group_size in {16, 32, 64, 128}; hidden % group_size == 0. */
+int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                   int64_t num_tokens, int64_t hidden, int group_size,
+                                   int64_t s_stride_row, int64_t s_stride_col, float eps, float fp8_min,
+                                   float fp8_max, void* stream);
+
+/* Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_int8
+ * (per_token_group_quant_8bit.cu:219-228; schema common_extension.cc:121-124):
+ * same arithmetic with an int8 destination, the float-to-int8 cast truncating
+ * toward zero as the C++ cast in per_token_group_quant_8bit.cu:111 does. */
+int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                    int64_t num_tokens, int64_t hidden, int group_size,
+                                    int64_t s_stride_row, int64_t s_stride_col, float eps, float int8_min,
+                                    float int8_max, void* stream);
+
+/* Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
+ * (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:166-227; schema
+ * common_extension.cc:129-130), zero rows giving zero codes as in the
+ * guarded kernel (:57).  hidden % 8 == 0 (:173).  output_s has num_tokens floats. */
+int sglq_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                             int64_t num_tokens, int64_t hidden, void* stream);
+
+/* Replaces the Triton kernel behind per_token_quant_int8
+ * (python/sglang/srt/layers/quantization/int8_kernel.py:20-81); the reference
+ * has no compiled op for it.  row_sum may be NULL; otherwise it receives the
+ * fp32-accumulated row sums in in_dtype (cal_sum=True, :43-45). */
+int sglq_per_token_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,
+                              void* row_sum, int64_t num_tokens, int64_t hidden, void* stream);
+
+/* Replaces torch.ops.sgl_kernel.fp8_blockwise_scaled_mm
+ * (sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:345-423; schema
+ * common_extension.cc:111-114).
+ *   a   e4m3fn [M, K], row stride lda, unit column stride
+ *   b   e4m3fn [K, N] column-major: element (k, n) at b[n*ldb + k]
+ *   sfa fp32 [M, ceil(K/128)]  at sfa[m*sfa_stride_m + kb*sfa_stride_k]
+ *   sfb fp32 [ceil(K/128), ceil(N/128)] at sfb[kb*sfb_stride_k + nb*sfb_stride_n]
+ *   out [M, N] row stride ldo, out_dtype in {BF16, FP16}
+ * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, a and b 16-byte aligned. */
+int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                 int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                 int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                 int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Replaces torch.ops.sgl_kernel.int8_scaled_mm
+ * (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; schema common_extension.cc:101-104).
+ * out = float(acc) * (scales_b[n] * scales_a[m]) + bias[n], acc exact int32.
+ * bias may be NULL and otherwise has out_dtype. */
+int sglq_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
+                        const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
+                        int64_t M, int64_t N, int64_t K, void* stream);
+
+/* The INT32 accumulators of sglq_int8_scaled_mm before its epilogue, written
+ * as int32 [M, N] with row stride ldo.  No counterpart op in the reference;
+ * it exists so the accumulators can be compared bit for bit. */
+int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64_t ldb, int32_t* out, int64_t ldo,
+                     int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Replaces torch.ops.sgl_kernel.fp8_scaled_mm
+ * (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1071-1146; schema common_extension.cc:106-109).
+ * out = scales_a[m] * (scales_b[n] * sum_k a*b) + bias[n], fp32 accumulation. */
+int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
+                       const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
+                       int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Test hook without a reference counterpart: non-zero (default) makes the GEMMs
+ * copy global memory straight into LDS with buffer loads, zero stages the same
+ * bytes through registers.  Both must give identical results. */
+void sglq_debug_set_direct_lds(int on);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGLQ_H */

@@ -1,0 +1,333 @@
+"""CPU oracle for the W8A8 quantized-linear path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in IEEE-754 binary32 arithmetic on the CPU (torch CPU
+tensors, no GPU, no compiled extension), what each operator on the path
+computes in the reference.  Only tests, the smoke check and the benchmark's
+CPU-baseline leg may import it; the shipped operators never do.
+
+Every function cites the reference lines it follows.  Parity status:
+
+* per_token_group_quant_fp8 / per_token_quant_fp8 / per_token_quant_int8:
+  pinned by closed-form constructions (x = code * scale), by an independent
+  bit-level e4m3fn encoder (``e4m3fn_encode_rne``), by the scalar C restatement
+  in ``w8a8_oracle.c`` and by torch's CPU float8 cast (tests/test_oracle.py).
+* int8 accumulators: pinned exactly by float64 matmul and int64 brute force.
+* fp8_blockwise_scaled_mm / fp8_scaled_mm / int8_scaled_mm outputs: pinned by
+  special cases that reduce to plain matmul, one-hot rows and float64 brute
+  force on tiny shapes; compared at rtol/atol 1e-2 because the reference's
+  summation order inside its GEMM library is not defined by its sources.
+
+The reference keeps no golden vectors for this path, so none are checked.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+FP8_E4M3_MAX = 448.0
+FP8 = torch.float8_e4m3fn
+
+
+# ---------------------------------------------------------------------------
+# e4m3fn encoder written from the format definition (1-4-3, bias 7, no inf,
+# S.1111.111 = NaN, max finite 448).  Independent of torch's cast; used to pin it.
+# ---------------------------------------------------------------------------
+def e4m3fn_encode_rne(x: torch.Tensor) -> torch.Tensor:
+    """Round-to-nearest-even fp32 -> e4m3fn bit patterns (uint8).
+
+    Inputs must already be clamped to [-448, 448] (NaN maps to 0x7f)."""
+    x = x.to(torch.float32)
+    bits = x.view(torch.int32)
+    sign = ((bits >> 24) & 0x80).to(torch.int32)
+    ax = x.abs().to(torch.float64)
+    out = torch.zeros_like(bits)
+    # subnormal range of e4m3: multiples of 2^-9 below 2^-6
+    # normal: exponent e in [-6, 8], 3 mantissa bits
+    e = torch.floor(torch.log2(torch.clamp(ax, min=2.0**-30)))
+    e = torch.clamp(e, min=-6.0)
+    # guard against log2 rounding at exact powers of two
+    e = torch.where(ax >= torch.pow(2.0, e + 1), e + 1, e)
+    e = torch.where((ax < torch.pow(2.0, e)) & (e > -6), e - 1, e)
+    quantum = torch.pow(2.0, e - 3)
+    scaled = ax / quantum  # exact: power-of-two scaling in float64
+    fl = torch.floor(scaled)
+    frac = scaled - fl
+    up = (frac > 0.5) | ((frac == 0.5) & (torch.remainder(fl, 2.0) == 1.0))
+    n = (fl + up.to(torch.float64)).to(torch.int64)  # in units of quantum
+    # n in [0, 16]; n == 16 means carry into next binade
+    eb = (e + 7).to(torch.int64)  # biased exponent for normals
+    is_sub = ax < 2.0**-6
+    # subnormals: code = n (n up to 8 -> 8 is the smallest normal, encodes naturally)
+    code_sub = n
+    code_norm = (eb << 3) + (n - 8)  # n-8 in [0, 8]; 8 carries into exponent
+    code = torch.where(is_sub, code_sub, code_norm).to(torch.int32)
+    code = torch.where(torch.isnan(x), torch.full_like(code, 0x7F), code)
+    out = (code | sign).to(torch.uint8)
+    return out
+
+
+def e4m3fn_decode(codes: torch.Tensor) -> torch.Tensor:
+    """uint8 e4m3fn bit patterns -> fp32 values, from the format definition."""
+    c = codes.to(torch.int32)
+    s = torch.where((c & 0x80) != 0, -1.0, 1.0)
+    e = (c >> 3) & 0xF
+    m = (c & 0x7).to(torch.float32)
+    sub = m * 2.0**-9
+    nor = (1.0 + m / 8.0) * torch.pow(2.0, (e - 7).to(torch.float32))
+    v = torch.where(e == 0, sub, nor)
+    v = torch.where((c & 0x7F) == 0x7F, torch.full_like(v, float("nan")), v)
+    return (s * v).to(torch.float32)
+
+
+def _to_fp8(x_clamped: torch.Tensor) -> torch.Tensor:
+    return x_clamped.to(FP8)
+
+
+def round_half_away(x: torch.Tensor) -> torch.Tensor:
+    """Round to nearest integer, ties away from zero (C ``roundf``), exactly.
+
+    ``x - trunc(x)`` is exact in binary floating point, so no double rounding."""
+    t = torch.trunc(x)
+    frac = x - t
+    step = torch.where(frac.abs() >= 0.5, torch.sign(x), torch.zeros_like(x))
+    return t + step
+
+
+# ---------------------------------------------------------------------------
+# a1  per-token-group FP8 quantization
+# ---------------------------------------------------------------------------
+def make_group_scale_buffer(
+    m: int, k: int, group_size: int, column_major_scales: bool, scale_tma_aligned: bool
+) -> torch.Tensor:
+    """Scale buffer layouts accepted by the op
+    (python/sglang/srt/layers/quantization/fp8_kernel.py:300-341)."""
+    g = k // group_size
+    if column_major_scales:
+        if scale_tma_aligned:
+            aligned = (m + 3) // 4 * 4
+            return torch.zeros((g, aligned), dtype=torch.float32).permute(1, 0)[:m, :]
+        return torch.zeros((g, m), dtype=torch.float32).permute(1, 0)
+    return torch.zeros((m, g), dtype=torch.float32)
+
+
+def per_token_group_quant_8bit(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float,
+    min_8bit: float,
+    max_8bit: float,
+    dst: torch.dtype,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:45,72-113.
+
+    absmax starts at eps (:45,80); y_s = absmax / max_8bit (:86, fp32 divide);
+    q = clamp(x / y_s, min, max) (:110, fp32 divide) cast to dst (:111)."""
+    assert x.shape[-1] % group_size == 0
+    xf = x.to(torch.float32).reshape(-1, group_size)
+    amax = torch.clamp(xf.abs().amax(dim=1, keepdim=True), min=torch.tensor(eps, dtype=torch.float32))
+    y_s = amax / torch.tensor(max_8bit, dtype=torch.float32)
+    q = torch.clamp(xf / y_s, min_8bit, max_8bit)
+    if dst == torch.int8:
+        # static_cast<int8_t>(float) truncates toward zero
+        qd = torch.trunc(q).to(torch.int8)
+    else:
+        qd = q.to(dst)
+    return qd.reshape(x.shape), y_s.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+
+
+def per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int = 128,
+    eps: float = 1e-10,
+    fp8_min: float = -FP8_E4M3_MAX,
+    fp8_max: float = FP8_E4M3_MAX,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Wrapper with the caller's defaults (fp8_kernel.py:83-85,344-372).
+    Returns codes [.., K] (e4m3fn) and row-major fp32 scales [.., K/group]."""
+    return per_token_group_quant_8bit(x, group_size, eps, fp8_min, fp8_max, FP8)
+
+
+# ---------------------------------------------------------------------------
+# a2  per-token INT8 quantization
+# ---------------------------------------------------------------------------
+def per_token_quant_int8(x: torch.Tensor, cal_sum: bool = False):
+    """python/sglang/srt/layers/quantization/int8_kernel.py:38-48.
+
+    absmax = max(max|x|, 1e-10) (:39); scale = absmax / 127 (:40);
+    q = round_half_away(x * (127 / absmax)) (:41-42) -> int8."""
+    xf = x.to(torch.float32)
+    amax = torch.clamp(xf.abs().amax(dim=-1, keepdim=True), min=torch.tensor(1e-10, dtype=torch.float32))
+    c127 = torch.tensor(127.0, dtype=torch.float32)
+    scale = amax / c127
+    r = c127 / amax
+    q = round_half_away(xf * r)
+    q = torch.clamp(q, -128, 127).to(torch.int8)
+    if cal_sum:
+        return q, scale, xf.sum(dim=-1).to(x.dtype)
+    return q, scale
+
+
+# ---------------------------------------------------------------------------
+# a3  per-token FP8 quantization
+# ---------------------------------------------------------------------------
+def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:35-71.
+
+    max = max|x| from 0 (:35-47); scale = max / 448 (:52);
+    inv = scale == 0 ? 0 : 1 / scale (:57); q = clamp(x * inv, +-448) (:68-69)."""
+    assert x.dim() == 2
+    xf = x.to(torch.float32)
+    amax = xf.abs().amax(dim=1, keepdim=True)
+    scale = amax / torch.tensor(FP8_E4M3_MAX, dtype=torch.float32)
+    inv = torch.where(scale == 0, torch.zeros_like(scale), 1.0 / scale)
+    q = torch.clamp(xf * inv, -FP8_E4M3_MAX, FP8_E4M3_MAX)
+    return q.to(FP8), scale
+
+
+# ---------------------------------------------------------------------------
+# a4  block-scaled FP8 GEMM
+# ---------------------------------------------------------------------------
+def fp8_blockwise_scaled_mm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scales_a: torch.Tensor,
+    scales_b: torch.Tensor,
+    out_dtype: torch.dtype,
+    acc_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:345-423 (semantics) with
+    the per-K-tile accumulation of python/sglang/test/test_block_fp8.py:274-326:
+
+    D[m,n] = sum_kb (sum_{k in kb} A[m,k] B[k,n]) * SFA[m,kb] * SFB[kb, n//128].
+
+    a [M,K] e4m3fn; b [K,N] e4m3fn (any strides); scales_a [M, ceil(K/128)];
+    scales_b [ceil(K/128), ceil(N/128)]."""
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2
+    kb = (k + 127) // 128
+    af = a.to(acc_dtype)
+    bf = b.to(acc_dtype)
+    sa = scales_a.to(acc_dtype)
+    sb = scales_b.to(acc_dtype)
+    sb_full = sb.repeat_interleave(128, dim=1)[:, :n]  # [kb, N]
+    out = torch.zeros((m, n), dtype=acc_dtype)
+    for i in range(kb):
+        ks = slice(i * 128, min((i + 1) * 128, k))
+        p = af[:, ks] @ bf[ks, :]
+        out += p * (sa[:, i : i + 1] * sb_full[i : i + 1, :])
+    return out.to(out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# a5  INT8 scaled GEMM
+# ---------------------------------------------------------------------------
+def int8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Exact INT32 accumulators of int8 [M,K] x int8 [K,N]
+    (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:38-153, ElementAccumulator int32).
+    float64 is exact here: |acc| <= K * 128^2 < 2^53 for any K < 2^39."""
+    acc = a.to(torch.float64) @ b.to(torch.float64)
+    return acc.to(torch.int64).to(torch.int32)
+
+
+def int8_scaled_mm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scales_a: torch.Tensor,
+    scales_b: torch.Tensor,
+    out_dtype: torch.dtype,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Epilogue order of
+    sgl-kernel/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:278,301:
+    out = float(acc) * (s_b[n] * s_a[m]) + float(bias[n])."""
+    acc = int8_mm_i32(a, b).to(torch.float32)
+    sa = scales_a.reshape(-1, 1).to(torch.float32)
+    sb = scales_b.reshape(1, -1).to(torch.float32)
+    out = acc * (sb * sa)
+    if bias is not None:
+        out = out + bias.to(torch.float32).reshape(1, -1)
+    return out.to(out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# a6  FP8 scaled GEMM (per-row activation scale, per-column weight scale)
+# ---------------------------------------------------------------------------
+def fp8_scaled_mm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scales_a: torch.Tensor,
+    scales_b: torch.Tensor,
+    out_dtype: torch.dtype,
+    bias: Optional[torch.Tensor] = None,
+    acc_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:522-546 (EVT order):
+    out = s_a[m] * (s_b[n] * sum_k A B) + bias[n]."""
+    acc = a.to(acc_dtype) @ b.to(acc_dtype)
+    sa = scales_a.reshape(-1, 1).to(acc_dtype)
+    sb = scales_b.reshape(1, -1).to(acc_dtype)
+    out = sa * (sb * acc)
+    if bias is not None:
+        out = out + bias.to(acc_dtype).reshape(1, -1)
+    return out.to(out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# Weight preparation for the harness (inputs of the measured ops, not outputs)
+# ---------------------------------------------------------------------------
+def block_quant_weight(w: torch.Tensor, block: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-128x128-block e4m3fn quantization of W [N,K]: scale = absmax/448
+    (0 -> 1), q = (w / scale) -> e4m3fn.  Returns q [N,K] and scales
+    [ceil(N/128), ceil(K/128)]  (layout contract of
+    python/sglang/srt/layers/quantization/fp8.py:276-306)."""
+    n, k = w.shape
+    nb, kb = (n + block - 1) // block, (k + block - 1) // block
+    wp = torch.zeros((nb * block, kb * block), dtype=torch.float32)
+    wp[:n, :k] = w.to(torch.float32)
+    t = wp.reshape(nb, block, kb, block).permute(0, 2, 1, 3)
+    amax = t.abs().amax(dim=(2, 3))
+    scale = amax / FP8_E4M3_MAX
+    scale = torch.where(scale == 0, torch.ones_like(scale), scale)
+    q = torch.clamp(t / scale[:, :, None, None], -FP8_E4M3_MAX, FP8_E4M3_MAX)
+    q = q.permute(0, 2, 1, 3).reshape(nb * block, kb * block)[:n, :k].contiguous().to(FP8)
+    return q, scale.contiguous()
+
+
+def per_tensor_quant_weight(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Single fp32 scale for W [N,K] widened to [N,1]
+    (python/sglang/srt/layers/quantization/utils.py:72-92)."""
+    wf = w.to(torch.float32)
+    amax = torch.clamp(wf.abs().amax(), min=1e-12)
+    scale = amax / FP8_E4M3_MAX
+    q = torch.clamp(wf / scale, -FP8_E4M3_MAX, FP8_E4M3_MAX).to(FP8)
+    return q, scale.reshape(1, 1).expand(w.shape[0], 1).contiguous()
+
+
+# ---------------------------------------------------------------------------
+# Synthetic inputs of the benchmark configurations (seeded on the CPU)
+# ---------------------------------------------------------------------------
+def gen_activation(m: int, k: int, seed: int, outliers: bool = False) -> torch.Tensor:
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn((m, k), generator=g, dtype=torch.float32)
+    if outliers:
+        mask = torch.rand((m, k), generator=g) < 0.01
+        a = torch.where(mask, a * 20.0, a)
+    return a.to(torch.bfloat16)
+
+
+def gen_weight(n: int, k: int, seed: int, std: float = 0.02) -> torch.Tensor:
+    g = torch.Generator().manual_seed(seed + 7919)
+    return torch.randn((n, k), generator=g, dtype=torch.float32) * std
+
+
+def gen_int8_weight(k: int, n: int, seed: int):
+    """B int8 [K,N] column-major (stored [N,K]), s_b U[1e-3,1e-2], bias N(0,0.1) bf16."""
+    g = torch.Generator().manual_seed(seed + 7919)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    s_b = torch.rand((n,), generator=g, dtype=torch.float32) * 9e-3 + 1e-3
+    bias = (torch.randn((n,), generator=g, dtype=torch.float32) * 0.1).to(torch.bfloat16)
+    return w.t(), s_b, bias

@@ -1,0 +1,71 @@
+"""ctypes binding of libsglq.so (the C ABI declared in include/sglq.h).
+
+There is no fallback: if the shared object is missing or a symbol cannot be
+resolved, importing the operators raises."""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "libsglq.so"
+
+SGLQ_BF16, SGLQ_FP16, SGLQ_FP32, SGLQ_I32 = 0, 1, 2, 3
+DTYPE_CODE = {torch.bfloat16: SGLQ_BF16, torch.float16: SGLQ_FP16, torch.float32: SGLQ_FP32}
+
+# name -> argtypes; every function returns int.  Mirrors include/sglq.h.
+_GROUP_QUANT = [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_int64, c_float, c_float, c_float, c_void_p]
+_ROWCOL_MM = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]
+SIGNATURES = {
+    "sglq_per_token_group_quant_fp8": _GROUP_QUANT,
+    "sglq_per_token_group_quant_int8": _GROUP_QUANT,
+    "sglq_per_token_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    "sglq_per_token_quant_int8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                     c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
+    "sglq_int8_scaled_mm": _ROWCOL_MM,
+    "sglq_fp8_scaled_mm": _ROWCOL_MM,
+    "sglq_int8_mm_i32": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load libsglq.so once; raise if it is absent (it is built by ``sglang_amd.build``)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build the HIP kernels first (python -m sglang_amd.build). "
+            "There is no non-HIP fallback for these operators."
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    lib.sglq_last_error.restype = c_char_p
+    lib.sglq_last_error.argtypes = []
+    lib.sglq_abi_version.restype = c_int
+    lib.sglq_abi_version.argtypes = []
+    lib.sglq_debug_set_direct_lds.argtypes = [c_int]
+    lib.sglq_debug_set_direct_lds.restype = None
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().sglq_last_error().decode("utf-8", "replace")
+        if rc == 2:
+            raise NotImplementedError(msg or what)
+        raise RuntimeError(msg or f"{what} failed with code {rc}")
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

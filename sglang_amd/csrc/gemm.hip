@@ -1,0 +1,457 @@
+// W8A8 GEMM kernels for gfx950 (CDNA4): C[M,N] = A[M,K] * B[K,N] with A row-major
+// and B column-major, i.e. both operands K-contiguous ("NT").  One template serves
+//   * block-scaled FP8   (per-token-group activation scales x 128x128 weight scales),
+//   * per-row/per-column scaled FP8, and
+//   * per-row/per-column scaled INT8 (exact INT32 accumulators),
+// on v_mfma_f32_16x16x128_f8f6f4 / v_mfma_i32_16x16x64_i8.
+//
+// Layout of the computation.  The MFMA "row" operand is a 16x128-byte slab of the
+// weight (16 values of n), the "column" operand a 16x128-byte slab of the
+// activations (16 values of m), so lane l of a 16x16 result holds
+//     C[m = l % 16][n = 4 * (l / 16) + j],  j = 0..3
+// i.e. four consecutive n for one m: the per-token scale is one register per lane
+// and the epilogue stores 8-byte runs.
+//
+// Tiles of BM x 128 B (activations) and BN x 128 B (weights) are staged in LDS,
+// double buffered.  A row holds eight 16-byte chunks; chunk c of row r is stored
+// at chunk position c ^ swz(r), swz(r) = (r & 7) ^ ((r >> 3) & 1), which makes the
+// 16-byte MFMA operand reads of any 8 or 16 consecutive lanes hit distinct banks.
+// Global -> LDS copies use buffer loads that write LDS directly (each wavefront
+// instruction fills 1 KiB = 8 rows); rows past M/N and chunks past K read as zero
+// through the buffer range check.
+#include <type_traits>
+
+#include "sglq_common.h"
+
+namespace sglq {
+
+constexpr int KIND_FP8_BLOCK = 0;   // a4: sum_kb P_kb * sfa[m,kb] * sfb[kb,n/128]
+constexpr int KIND_FP8_ROWCOL = 1;  // a6: sa[m] * (sb[n] * acc) + bias[n]
+constexpr int KIND_I8_ROWCOL = 2;   // a5: float(acc) * (sb[n] * sa[m]) + bias[n]
+constexpr int KIND_I8_RAW = 3;      // INT32 accumulators
+
+constexpr uint32_t OOB = 0x80000000u;  // offset beyond any buffer this library accepts
+
+struct GemmArgs {
+  const char* a;   // [M, K] bytes, row stride lda
+  const char* b;   // [N, K] bytes, row stride ldb (column-major [K, N])
+  const float* sa; // block: sfa; rowcol: scales_a [M]
+  const float* sb; // block: sfb; rowcol: scales_b [N]
+  const void* bias;
+  void* out;
+  int64_t sa_stride_m, sa_stride_k;  // block scales
+  int64_t sb_stride_k, sb_stride_n;
+  int64_t ldo;
+  uint32_t lda, ldb;
+  uint32_t a_bytes, b_bytes;
+  int M, N, K;
+  int tiles_m, tiles_n;
+};
+
+SGLQ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+
+template <int OUT_DT>
+SGLQ_DEV void store4(void* out, int64_t idx, float v0, float v1, float v2, float v3) {
+  if constexpr (OUT_DT == SGLQ_BF16) {
+    typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+    bf4 o = {(__bf16)v0, (__bf16)v1, (__bf16)v2, (__bf16)v3};
+    *reinterpret_cast<bf4*>(reinterpret_cast<__bf16*>(out) + idx) = o;
+  } else {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    h4 o = {(_Float16)v0, (_Float16)v1, (_Float16)v2, (_Float16)v3};
+    *reinterpret_cast<h4*>(reinterpret_cast<_Float16*>(out) + idx) = o;
+  }
+}
+
+template <int OUT_DT>
+SGLQ_DEV void load_bias4(const void* bias, int n, float (&b)[4]) {
+  if constexpr (OUT_DT == SGLQ_BF16) {
+    const uint16_t* p = reinterpret_cast<const uint16_t*>(bias) + n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = u2f((uint32_t)p[j] << 16);
+  } else {
+    const _Float16* p = reinterpret_cast<const _Float16*>(bias) + n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = (float)p[j];
+  }
+}
+
+// Map the linear block id to an output tile: consecutive ids are dealt round-robin
+// to the 8 XCDs by the dispatcher, so give every XCD one contiguous range of tiles
+// (its L2 then sees a compact set of A rows and B columns), and walk each range in
+// bands of GROUP_M tile-rows.
+SGLQ_DEV void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int q = total >> 3, rem = total & 7;
+  const int xcd = pid & 7, idx = pid >> 3;
+  int tile = xcd * q + (xcd < rem ? xcd : rem) + idx;
+  constexpr int GROUP_M = 8;
+  const int width = GROUP_M * tiles_n;
+  const int group = tile / width;
+  const int first_m = group * GROUP_M;
+  const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_group = tile - group * width;
+  tm = first_m + in_group % gsz;
+  tn = in_group / gsz;
+}
+
+template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT, bool DMA>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const GemmArgs p) {
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;  // per-wave tile
+  constexpr int MI = TM / 16, NI = TN / 16;
+  constexpr int STAGE_BYTES = (BM + BN) * 128;
+  constexpr int NLOAD = (BM + BN) / 8 / NW;  // 1 KiB copies per wave per stage
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  static_assert((BM + BN) % (8 * NW) == 0 && TM % 16 == 0 && TN % 16 == 0, "tile shape");
+  static_assert(KIND != KIND_FP8_BLOCK || (128 % TN == 0), "a wave must stay inside one 128-wide scale block");
+
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
+
+  // ---- global -> LDS copy plan: copy i (of (BM+BN)/8) fills rows 8i..8i+7 of the stage
+  uint32_t src_off[NLOAD];  // byte offset of this lane's 16-byte chunk at k0 = 0
+  int src_k[NLOAD];         // its k offset inside the 128-byte K block
+#pragma unroll
+  for (int j = 0; j < NLOAD; ++j) {
+    const int i = wave + j * NW;
+    const int row = i * 8 + (lane >> 3);  // row inside the stage (A rows first, then B rows)
+    const bool is_a = row < BM;
+    const int rr = is_a ? row : row - BM;
+    const int c = (lane & 7) ^ swz(rr);
+    const int grow = is_a ? (m0 + rr) : (n0 + rr);
+    const bool ok = is_a ? (grow < p.M) : (grow < p.N);
+    src_k[j] = c * 16;
+    src_off[j] = ok ? (uint32_t)grow * (is_a ? p.lda : p.ldb) + c * 16 : OOB;
+  }
+
+  auto issue_loads = [&](int stage, int k0) {
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+      const int i = wave + j * NW;
+      const bool is_a = (i * 8) < BM;  // uniform per wave instruction
+      uint32_t off = (k0 + src_k[j] < p.K) ? src_off[j] + (uint32_t)k0 : OOB;
+      if (src_off[j] == OOB) off = OOB;
+      char* dst = smem + stage * STAGE_BYTES + i * 1024;
+      if constexpr (DMA) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(is_a ? ra : rb, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 off, 0, 0, 0);
+      } else {
+        v4i v = __builtin_amdgcn_raw_buffer_load_b128(is_a ? ra : rb, off, 0, 0);
+        *reinterpret_cast<v4i*>(dst + lane * 16) = v;
+      }
+    }
+  };
+
+  // ---- MFMA operand addresses in LDS
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  const int a_base = (wm * TM) * 128;
+  const int b_base = (BM + wn * TN) * 128;
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+  // ---- block scales: one activation scale per lane per 16-row fragment
+  const int nkb = (p.K + 127) >> 7;
+  float sfa_next[MI];
+  float sfb_next = 0.f;
+  int sfa_row[MI];
+  int nb = 0;
+  if constexpr (KIND == KIND_FP8_BLOCK) {
+    const int nblocks = (p.N + 127) >> 7;
+    nb = (n0 + wn * TN) >> 7;
+    if (nb >= nblocks) nb = nblocks - 1;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      int m = m0 + wm * TM + i * 16 + r16;
+      sfa_row[i] = m < p.M ? m : p.M - 1;
+      sfa_next[i] = p.sa[sfa_row[i] * p.sa_stride_m];
+    }
+    sfb_next = p.sb[nb * p.sb_stride_n];
+  }
+
+  issue_loads(0, 0);
+
+  for (int kb = 0; kb < nkb; ++kb) {
+    const int cur = kb & 1;
+    __builtin_amdgcn_s_waitcnt(0);  // this stage's copies (and prefetched scales) have landed
+    __syncthreads();                // for every wave; and all waves are done reading the other stage
+    if (kb + 1 < nkb) issue_loads(cur ^ 1, (kb + 1) * 128);
+
+    float sc[MI];
+    if constexpr (KIND == KIND_FP8_BLOCK) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sc[i] = sfa_next[i] * sfb_next;
+      if (kb + 1 < nkb) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) sfa_next[i] = p.sa[sfa_row[i] * p.sa_stride_m + (kb + 1) * p.sa_stride_k];
+        sfb_next = p.sb[(kb + 1) * p.sb_stride_k + nb * p.sb_stride_n];
+      }
+    }
+
+    const char* st = smem + cur * STAGE_BYTES;
+    v8i af[MI], bf[NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const char* q = st + a_base + i * 16 * 128;
+      v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+      v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+      af[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const char* q = st + b_base + j * 16 * 128;
+      v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+      v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+      bf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        if constexpr (KIND == KIND_FP8_BLOCK) {
+          const v4f z = {0.f, 0.f, 0.f, 0.f};
+          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i], z, 0, 0, 0, 0, 0, 0);
+          acc[i][j][0] = __builtin_fmaf(part[0], sc[i], acc[i][j][0]);
+          acc[i][j][1] = __builtin_fmaf(part[1], sc[i], acc[i][j][1]);
+          acc[i][j][2] = __builtin_fmaf(part[2], sc[i], acc[i][j][2]);
+          acc[i][j][3] = __builtin_fmaf(part[3], sc[i], acc[i][j][3]);
+        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+        } else {
+          const v4i b0 = {bf[j][0], bf[j][1], bf[j][2], bf[j][3]}, b1 = {bf[j][4], bf[j][5], bf[j][6], bf[j][7]};
+          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]}, a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m0 + wm * TM + i * 16 + r16;
+    if (m >= p.M) continue;
+    float sam = 1.f;
+    if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = p.sa[m];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n0 + wn * TN + j * 16 + g * 4;
+      if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
+      const int64_t idx = (int64_t)m * p.ldo + n;
+      if constexpr (KIND == KIND_I8_RAW) {
+        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = acc[i][j];
+      } else if constexpr (KIND == KIND_FP8_BLOCK) {
+        store4<OUT_DT>(p.out, idx, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      } else {
+        float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
+        const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
+        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbn[e] * sam, bv[e]);
+          else o[e] = __builtin_fmaf(sam, sbn[e] * acc[i][j][e], bv[e]);
+        }
+        store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static bool g_use_dma = true;
+
+template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT>
+static void launch_cfg(GemmArgs& p, hipStream_t st) {
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  dim3 grid((uint32_t)(p.tiles_m * p.tiles_n)), block(WAVES_M * WAVES_N * 64);
+  if (g_use_dma) gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, true><<<grid, block, 0, st>>>(p);
+  else gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, false><<<grid, block, 0, st>>>(p);
+}
+
+template <int KIND, int OUT_DT>
+static void launch_kind(GemmArgs& p, hipStream_t st) {
+  if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, st);
+  else if (p.M <= 64) launch_cfg<KIND, 64, 128, 1, 4, OUT_DT>(p, st);
+  else launch_cfg<KIND, 128, 128, 2, 2, OUT_DT>(p, st);
+}
+
+static int gemm_common_checks(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb,
+                              const void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int out_elem_bytes) {
+  if (M < 0 || N < 0 || K < 0) {
+    set_error("%s: negative dimension", name);
+    return SGLQ_EINVAL;
+  }
+  if (M == 0 || N == 0) return -1;  // nothing to do
+  if (!a || !b || !out) {
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (K == 0 || K % 16 != 0) {
+    set_error("%s: K (%lld) must be a positive multiple of 16", name, (long long)K);
+    return SGLQ_EINVAL;
+  }
+  if (lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K) {
+    set_error("%s: lda/ldb must be multiples of 16 and >= K", name);
+    return SGLQ_EINVAL;
+  }
+  if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15)) {
+    set_error("%s: mat_a and mat_b must be 16-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  if (N % 4 != 0 || ldo % 4 != 0 || ldo < N || (reinterpret_cast<uintptr_t>(out) & (4 * out_elem_bytes - 1))) {
+    set_error("%s: N and ldo must be multiples of 4 and out aligned to 4 elements", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t a_bytes = (M - 1) * lda + K, b_bytes = (N - 1) * ldb + K;
+  if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || M >= (1 << 30) || N >= (1 << 30)) {
+    set_error("%s: operand larger than 2 GiB is not supported", name);
+    return SGLQ_EUNSUPPORTED;
+  }
+  return SGLQ_OK;
+}
+
+static void fill_common(GemmArgs& p, const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
+                        int64_t M, int64_t N, int64_t K) {
+  p = GemmArgs{};
+  p.a = static_cast<const char*>(a);
+  p.b = static_cast<const char*>(b);
+  p.out = out;
+  p.lda = (uint32_t)lda;
+  p.ldb = (uint32_t)ldb;
+  p.ldo = ldo;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.a_bytes = (uint32_t)((M - 1) * lda + K);
+  p.b_bytes = (uint32_t)((N - 1) * ldb + K);
+}
+
+static int finish(const char* name) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", name, hipGetErrorString(e));
+    return SGLQ_ELAUNCH;
+  }
+  return SGLQ_OK;
+}
+
+}  // namespace sglq
+
+using namespace sglq;
+
+// Test hook: choose between direct-to-LDS buffer loads (default) and loads staged
+// through registers.  Both fill LDS identically.
+extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
+
+extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                            int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                            int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  const char* name = "fp8_blockwise_scaled_mm";
+  int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
+  if (rc < 0) return SGLQ_OK;
+  if (rc) return rc;
+  if (!sfa || !sfb) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (out_dtype != SGLQ_BF16 && out_dtype != SGLQ_FP16) {
+    set_error("%s: out_dtype must be Half or BFloat16", name);
+    return SGLQ_EINVAL;
+  }
+  GemmArgs p;
+  fill_common(p, a, lda, b, ldb, out, ldo, M, N, K);
+  p.sa = sfa;
+  p.sb = sfb;
+  p.sa_stride_m = sfa_stride_m;
+  p.sa_stride_k = sfa_stride_k;
+  p.sb_stride_k = sfb_stride_k;
+  p.sb_stride_n = sfb_stride_n;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_BLOCK, SGLQ_BF16>(p, st);
+  else launch_kind<KIND_FP8_BLOCK, SGLQ_FP16>(p, st);
+  return finish(name);
+}
+
+static int rowcol_entry(const char* name, bool fp8, const void* a, int64_t lda, const void* b, int64_t ldb,
+                        const float* scales_a, const float* scales_b, const void* bias, void* out, int64_t ldo,
+                        int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
+  if (rc < 0) return SGLQ_OK;
+  if (rc) return rc;
+  if (!scales_a || !scales_b) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (reinterpret_cast<uintptr_t>(scales_b) & 15) {
+    set_error("%s: scales_b must be 16-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  if (out_dtype != SGLQ_BF16 && out_dtype != SGLQ_FP16) {
+    set_error("%s: out_dtype must be Half or BFloat16", name);
+    return SGLQ_EINVAL;
+  }
+  GemmArgs p;
+  fill_common(p, a, lda, b, ldb, out, ldo, M, N, K);
+  p.sa = scales_a;
+  p.sb = scales_b;
+  p.bias = bias;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (fp8) {
+    if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_ROWCOL, SGLQ_BF16>(p, st);
+    else launch_kind<KIND_FP8_ROWCOL, SGLQ_FP16>(p, st);
+  } else {
+    if (out_dtype == SGLQ_BF16) launch_kind<KIND_I8_ROWCOL, SGLQ_BF16>(p, st);
+    else launch_kind<KIND_I8_ROWCOL, SGLQ_FP16>(p, st);
+  }
+  return finish(name);
+}
+
+extern "C" int sglq_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
+                                   const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
+                                   int64_t M, int64_t N, int64_t K, void* stream) {
+  return rowcol_entry("int8_scaled_mm", false, a, lda, b, ldb, scales_a, scales_b, bias, out, ldo, out_dtype, M, N, K,
+                      stream);
+}
+
+extern "C" int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
+                                  const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
+                                  int64_t M, int64_t N, int64_t K, void* stream) {
+  return rowcol_entry("fp8_scaled_mm", true, a, lda, b, ldb, scales_a, scales_b, bias, out, ldo, out_dtype, M, N, K,
+                      stream);
+}
+
+extern "C" int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64_t ldb, int32_t* out, int64_t ldo,
+                                int64_t M, int64_t N, int64_t K, void* stream) {
+  const char* name = "int8_mm_i32";
+  int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 4);
+  if (rc < 0) return SGLQ_OK;
+  if (rc) return rc;
+  GemmArgs p;
+  fill_common(p, a, lda, b, ldb, out, ldo, M, N, K);
+  launch_kind<KIND_I8_RAW, SGLQ_BF16>(p, static_cast<hipStream_t>(stream));
+  return finish(name);
+}

@@ -1,0 +1,514 @@
+// Activation quantization kernels for gfx950: per-token-group FP8/INT8,
+// per-token FP8 and per-token INT8.  All are HBM-bound: every element is read
+// once with 128-bit loads, kept in registers across the abs-max reduction
+// (DPP inside 16-lane rows), and written once.
+//
+// Arithmetic contract (bit-exact with the reference's definitions):
+//   group  : amax = max(eps, max|x|); s = amax / max8; q = clamp(x / s)     (IEEE divides)
+//   tok fp8: amax = max|x|; s = amax / 448; inv = s == 0 ? 0 : 1/s; q = clamp(x * inv)
+//   tok i8 : amax = max(max|x|, 1e-10); s = amax / 127; q = roundf(x * (127 / amax))
+// The per-element divide of the group kernel is evaluated as a multiply by the
+// correctly rounded reciprocal plus an exact FMA remainder correction, which
+// returns the IEEE quotient (see div_by).  NaN inputs are outside the contract.
+#include "sglq_common.h"
+
+namespace sglq {
+
+// ---------------------------------------------------------------------------
+// 8 consecutive input elements -> 8 floats, plus the bit pattern of their abs-max
+// ---------------------------------------------------------------------------
+template <int DT>
+struct Chunk8;
+
+template <>
+struct Chunk8<SGLQ_BF16> {
+  v4u raw;
+  static constexpr int kBytes = 16;
+  SGLQ_MEM void load(const void* p) { raw = *reinterpret_cast<const v4u*>(p); }
+  SGLQ_MEM uint32_t amax_bits() const {
+    // |bf16| orders like its low 15 bits taken as an integer: packed 16-bit max.
+    v2us m = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t a = raw[i] & 0x7fff7fffu;
+      m = __builtin_elementwise_max(m, __builtin_bit_cast(v2us, a));
+    }
+    uint32_t hi = m.x > m.y ? m.x : m.y;
+    return hi << 16;
+  }
+  SGLQ_MEM float get(int i) const {
+    uint32_t w = raw[i >> 1];
+    return u2f((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+};
+
+template <>
+struct Chunk8<SGLQ_FP16> {
+  v4u raw;
+  static constexpr int kBytes = 16;
+  SGLQ_MEM void load(const void* p) { raw = *reinterpret_cast<const v4u*>(p); }
+  SGLQ_MEM float get(int i) const {
+    uint32_t w = raw[i >> 1];
+    unsigned short h = (i & 1) ? (unsigned short)(w >> 16) : (unsigned short)(w & 0xffffu);
+    return (float)__builtin_bit_cast(_Float16, h);
+  }
+  SGLQ_MEM uint32_t amax_bits() const {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = umax(m, f2u(get(i)) & 0x7fffffffu);
+    return m;
+  }
+};
+
+template <>
+struct Chunk8<SGLQ_FP32> {
+  v4u raw[2];
+  static constexpr int kBytes = 32;
+  SGLQ_MEM void load(const void* p) {
+    raw[0] = reinterpret_cast<const v4u*>(p)[0];
+    raw[1] = reinterpret_cast<const v4u*>(p)[1];
+  }
+  SGLQ_MEM float get(int i) const { return u2f(raw[i >> 2][i & 3]); }
+  SGLQ_MEM uint32_t amax_bits() const {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = umax(m, raw[i >> 2][i & 3] & 0x7fffffffu);
+    return m;
+  }
+};
+
+template <int DT>
+constexpr int elem_bytes() {
+  return DT == SGLQ_FP32 ? 4 : 2;
+}
+
+// 8 quantized floats -> 8 bytes
+struct Fp8Pack {
+  SGLQ_DEV v2u pack(const float (&v)[8]) {
+    v2u o;
+    uint32_t w = cvt_pk_e4m3<false>(v[0], v[1], 0);
+    o.x = cvt_pk_e4m3<true>(v[2], v[3], w);
+    w = cvt_pk_e4m3<false>(v[4], v[5], 0);
+    o.y = cvt_pk_e4m3<true>(v[6], v[7], w);
+    return o;
+  }
+};
+
+struct I8Pack {
+  // inputs are already integral (or to be truncated) and inside [-128, 127]
+  SGLQ_DEV v2u pack(const float (&v)[8]) {
+    v2u o;
+    o.x = ((uint32_t)(int)v[0] & 0xffu) | (((uint32_t)(int)v[1] & 0xffu) << 8) |
+          (((uint32_t)(int)v[2] & 0xffu) << 16) | ((uint32_t)(int)v[3] << 24);
+    o.y = ((uint32_t)(int)v[4] & 0xffu) | (((uint32_t)(int)v[5] & 0xffu) << 8) |
+          (((uint32_t)(int)v[6] & 0xffu) << 16) | ((uint32_t)(int)v[7] << 24);
+    return o;
+  }
+};
+
+// Division of a 32-bit index by a runtime-constant divisor (Granlund-Montgomery).
+struct FastDiv {
+  uint32_t d, magic, shift;
+  void init(uint32_t div) {
+    d = div;
+    uint32_t l = 0;
+    while ((1ull << l) < div) ++l;
+    magic = (uint32_t)(((1ull << 32) * ((1ull << l) - div)) / div + 1);
+    shift = l;
+  }
+  SGLQ_MEM uint32_t div(uint32_t n) const {
+    uint32_t t = __umulhi(magic, n);
+    // shift may be 0 (d == 1): split the shift so that no shift count is negative
+    uint32_t s1 = shift > 0 ? 1u : 0u;
+    return (t + ((n - t) >> s1)) >> (shift - s1);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Per-token-group quantization.  16 elements per lane as two 8-element chunks
+// half a group apart, so every load instruction reads fully used 128-byte runs.
+// ---------------------------------------------------------------------------
+template <int DT, int GROUP, int UNROLL, bool STRIDED_SCALE, bool TO_INT8>
+__global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
+                                                          float* __restrict__ s, uint32_t num_groups,
+                                                          FastDiv groups_per_row, int64_t s_stride_row,
+                                                          int64_t s_stride_col, float eps, float qmin, float qmax,
+                                                          float rqmax) {
+  constexpr int LPG = GROUP / 16;  // lanes per group
+  constexpr int GPB = 256 / LPG;   // groups per block per step
+  constexpr int EB = elem_bytes<DT>();
+  const uint32_t t = threadIdx.x;
+  const uint32_t sub = t % LPG;
+  const uint32_t g0 = blockIdx.x * (UNROLL * GPB) + t / LPG;
+
+  Chunk8<DT> lo[UNROLL], hi[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const uint32_t gid = g0 + u * GPB;
+    if (gid < num_groups) {
+      const char* p = x + ((int64_t)gid * GROUP + sub * 8) * EB;
+      lo[u].load(p);
+      hi[u].load(p + (GROUP / 2) * EB);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const uint32_t gid = g0 + u * GPB;
+    if (gid < num_groups) {
+      uint32_t mb = umax(lo[u].amax_bits(), hi[u].amax_bits());
+      mb = group_umax<LPG>(mb);
+      const float amax = u2f(umax(mb, f2u(eps)));
+      const float y_s = div_by(amax, qmax, rqmax);
+      const float r = 1.0f / y_s;
+      float v[8];
+      v2u o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = clampf(div_by(lo[u].get(i), y_s, r), qmin, qmax);
+      if constexpr (TO_INT8) o = I8Pack::pack(v); else o = Fp8Pack::pack(v);
+      char* qp = q + (int64_t)gid * GROUP + sub * 8;
+      *reinterpret_cast<v2u*>(qp) = o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = clampf(div_by(hi[u].get(i), y_s, r), qmin, qmax);
+      if constexpr (TO_INT8) o = I8Pack::pack(v); else o = Fp8Pack::pack(v);
+      *reinterpret_cast<v2u*>(qp + GROUP / 2) = o;
+      if (sub == 0) {
+        if constexpr (STRIDED_SCALE) {
+          const uint32_t row = groups_per_row.div(gid);
+          const uint32_t col = gid - row * groups_per_row.d;
+          s[row * s_stride_row + col * s_stride_col] = y_s;
+        } else {
+          s[gid] = y_s;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Per-token (whole-row) quantization.  TEAM lanes share one row (64 = one
+// wavefront, 256 = the block); each lane keeps V 16-byte chunks in registers.
+// ---------------------------------------------------------------------------
+constexpr int MODE_FP8 = 0;
+constexpr int MODE_INT8 = 1;
+
+template <int DT, int TEAM, int V, int MODE>
+__global__ __launch_bounds__(256) void token_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
+                                                          float* __restrict__ s, void* __restrict__ row_sum,
+                                                          int64_t rows, uint32_t chunks) {
+  constexpr int EB = elem_bytes<DT>();
+  constexpr int TEAMS = 256 / TEAM;
+  __shared__ uint32_t red_max[4];
+  __shared__ float red_sum[4];
+  const uint32_t t = threadIdx.x % TEAM;
+  const int64_t row = (int64_t)blockIdx.x * TEAMS + threadIdx.x / TEAM;
+  const bool live = row < rows;
+  const char* xr = x + row * (int64_t)chunks * 8 * EB;
+
+  Chunk8<DT> c[V];
+  uint32_t mb = 0;
+  float sum = 0.f;
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t ci = t + v * TEAM;
+    if (live && ci < chunks) c[v].load(xr + (int64_t)ci * 8 * EB);
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t ci = t + v * TEAM;
+    if (live && ci < chunks) {
+      mb = umax(mb, c[v].amax_bits());
+      if (MODE == MODE_INT8 && row_sum != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += c[v].get(i);
+      }
+    }
+  }
+  mb = wave_umax(mb);
+  if (MODE == MODE_INT8 && row_sum != nullptr) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+  }
+  if constexpr (TEAM == 256) {
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      red_max[w] = mb;
+      red_sum[w] = sum;
+    }
+    __syncthreads();
+    mb = umax(umax(red_max[0], red_max[1]), umax(red_max[2], red_max[3]));
+    sum = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]);
+  }
+  if (!live) return;
+
+  float scale, mul, lo, hi;
+  if constexpr (MODE == MODE_FP8) {
+    const float amax = u2f(mb);
+    scale = amax / 448.0f;
+    mul = (scale == 0.f) ? 0.f : 1.0f / scale;
+    lo = -448.0f;
+    hi = 448.0f;
+  } else {
+    const float amax = u2f(umax(mb, f2u(1e-10f)));
+    scale = amax / 127.0f;
+    mul = 127.0f / amax;
+    lo = -128.0f;
+    hi = 127.0f;
+  }
+  if (t == 0) {
+    s[row] = scale;
+    if (MODE == MODE_INT8 && row_sum != nullptr) {
+      if constexpr (DT == SGLQ_BF16) reinterpret_cast<__bf16*>(row_sum)[row] = (__bf16)sum;
+      else if constexpr (DT == SGLQ_FP16) reinterpret_cast<_Float16*>(row_sum)[row] = (_Float16)sum;
+      else reinterpret_cast<float*>(row_sum)[row] = sum;
+    }
+  }
+  char* qr = q + row * (int64_t)chunks * 8;
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t ci = t + v * TEAM;
+    if (ci < chunks) {
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float y = c[v].get(i) * mul;
+        if constexpr (MODE == MODE_INT8) y = __builtin_roundf(y);
+        o[i] = clampf(y, lo, hi);
+      }
+      v2u pk;
+      if constexpr (MODE == MODE_INT8) pk = I8Pack::pack(o); else pk = Fp8Pack::pack(o);
+      *reinterpret_cast<v2u*>(qr + (int64_t)ci * 8) = pk;
+    }
+  }
+}
+
+// Rows of any length (also not a multiple of 8, or longer than the register
+// budget of the kernel above): one block per row, two passes, scalar accesses.
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void token_quant_generic_kernel(const char* __restrict__ x,
+                                                                  char* __restrict__ q, float* __restrict__ s,
+                                                                  void* __restrict__ row_sum, int64_t hidden) {
+  __shared__ uint32_t red_max[4];
+  __shared__ float red_sum[4];
+  const int64_t row = blockIdx.x;
+  auto ld = [&](int64_t j) -> float {
+    const int64_t idx = row * hidden + j;
+    if constexpr (DT == SGLQ_BF16) return u2f((uint32_t)reinterpret_cast<const uint16_t*>(x)[idx] << 16);
+    else if constexpr (DT == SGLQ_FP16) return (float)reinterpret_cast<const _Float16*>(x)[idx];
+    else return reinterpret_cast<const float*>(x)[idx];
+  };
+  uint32_t mb = 0;
+  float sum = 0.f;
+  for (int64_t j = threadIdx.x; j < hidden; j += 256) {
+    const float v = ld(j);
+    mb = umax(mb, f2u(v) & 0x7fffffffu);
+    sum += v;
+  }
+  mb = wave_umax(mb);
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+  if ((threadIdx.x & 63) == 0) {
+    red_max[threadIdx.x >> 6] = mb;
+    red_sum[threadIdx.x >> 6] = sum;
+  }
+  __syncthreads();
+  mb = umax(umax(red_max[0], red_max[1]), umax(red_max[2], red_max[3]));
+  sum = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]);
+  float scale, mul, lo, hi;
+  if constexpr (MODE == MODE_FP8) {
+    scale = u2f(mb) / 448.0f;
+    mul = (scale == 0.f) ? 0.f : 1.0f / scale;
+    lo = -448.0f;
+    hi = 448.0f;
+  } else {
+    const float amax = u2f(umax(mb, f2u(1e-10f)));
+    scale = amax / 127.0f;
+    mul = 127.0f / amax;
+    lo = -128.0f;
+    hi = 127.0f;
+  }
+  if (threadIdx.x == 0) {
+    s[row] = scale;
+    if (MODE == MODE_INT8 && row_sum != nullptr) {
+      if constexpr (DT == SGLQ_BF16) reinterpret_cast<__bf16*>(row_sum)[row] = (__bf16)sum;
+      else if constexpr (DT == SGLQ_FP16) reinterpret_cast<_Float16*>(row_sum)[row] = (_Float16)sum;
+      else reinterpret_cast<float*>(row_sum)[row] = sum;
+    }
+  }
+  for (int64_t j = threadIdx.x; j < hidden; j += 256) {
+    float y = ld(j) * mul;
+    if constexpr (MODE == MODE_INT8) {
+      y = clampf(__builtin_roundf(y), lo, hi);
+      q[row * hidden + j] = (char)(int)y;
+    } else {
+      y = clampf(y, lo, hi);
+      q[row * hidden + j] = (char)(cvt_pk_e4m3<false>(y, y, 0) & 0xffu);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host-side dispatch
+// ---------------------------------------------------------------------------
+static int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return SGLQ_ELAUNCH;
+  }
+  return SGLQ_OK;
+}
+
+template <int DT, int GROUP, bool TO_INT8>
+static void launch_group_quant(const void* x, void* q, float* s, uint32_t num_groups, uint32_t gpr, bool strided,
+                               int64_t sr, int64_t sc, float eps, float qmin, float qmax, hipStream_t st) {
+  constexpr int GPB = 256 / (GROUP / 16);
+  FastDiv fd;
+  fd.init(gpr);
+  const float rq = 1.0f / qmax;
+  // two groups per lane once there is enough work to fill the chip several times over
+  const bool deep = num_groups >= (uint32_t)GPB * 2 * 2048;
+  const char* xi = static_cast<const char*>(x);
+  char* qo = static_cast<char*>(q);
+#define SGLQ_LAUNCH_GQ(U, STR)                                                                              \
+  group_quant_kernel<DT, GROUP, U, STR, TO_INT8><<<dim3((num_groups + GPB * U - 1) / (GPB * U)), dim3(256), 0, st>>>( \
+      xi, qo, s, num_groups, fd, sr, sc, eps, qmin, qmax, rq)
+  if (deep) {
+    if (strided) SGLQ_LAUNCH_GQ(2, true); else SGLQ_LAUNCH_GQ(2, false);
+  } else {
+    if (strided) SGLQ_LAUNCH_GQ(1, true); else SGLQ_LAUNCH_GQ(1, false);
+  }
+#undef SGLQ_LAUNCH_GQ
+}
+
+template <bool TO_INT8>
+static int group_quant_entry(const char* name, const void* input, int in_dtype, void* output_q, float* output_s,
+                             int64_t num_tokens, int64_t hidden, int group_size, int64_t sr, int64_t sc, float eps,
+                             float qmin, float qmax, void* stream) {
+  if (!input || !output_q || !output_s) {
+    if (num_tokens == 0) return SGLQ_OK;
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_tokens < 0 || hidden <= 0 || group_size <= 0 || hidden % group_size != 0) {
+    set_error("%s: hidden (%lld) must be a positive multiple of group_size (%d)", name, (long long)hidden, group_size);
+    return SGLQ_EINVAL;
+  }
+  if (!(qmax > 0.f) || !(eps > 0.f)) {
+    set_error("%s: eps and the 8-bit maximum must be positive", name);
+    return SGLQ_EINVAL;
+  }
+  if ((reinterpret_cast<uintptr_t>(input) & 15) || (reinterpret_cast<uintptr_t>(output_q) & 7)) {
+    set_error("%s: input must be 16-byte and output_q 8-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t gpr = hidden / group_size;
+  const int64_t ng = num_tokens * gpr;
+  if (ng == 0) return SGLQ_OK;
+  if (ng >= (1ll << 32) - 65536) {
+    set_error("%s: too many groups (%lld)", name, (long long)ng);
+    return SGLQ_EINVAL;
+  }
+  const bool strided = !(sc == 1 && sr == gpr);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define SGLQ_GQ_CASE(DT, G)                                                                                   \
+  if (in_dtype == DT && group_size == G) {                                                                    \
+    launch_group_quant<DT, G, TO_INT8>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, sc, \
+                                       eps, qmin, qmax, st);                                                  \
+    return check_launch(name);                                                                                \
+  }
+#define SGLQ_GQ_DT(DT) SGLQ_GQ_CASE(DT, 128) SGLQ_GQ_CASE(DT, 64) SGLQ_GQ_CASE(DT, 32) SGLQ_GQ_CASE(DT, 16)
+  SGLQ_GQ_DT(SGLQ_BF16)
+  SGLQ_GQ_DT(SGLQ_FP16)
+  SGLQ_GQ_DT(SGLQ_FP32)
+#undef SGLQ_GQ_DT
+#undef SGLQ_GQ_CASE
+  set_error("%s: unsupported in_dtype %d / group_size %d (group sizes built: 16, 32, 64, 128)", name, in_dtype,
+            group_size);
+  return SGLQ_EUNSUPPORTED;
+}
+
+template <int DT, int MODE>
+static int launch_token_quant(const char* name, const void* x, void* q, float* s, void* row_sum, int64_t rows,
+                              int64_t hidden, hipStream_t st) {
+  const char* xi = static_cast<const char*>(x);
+  char* qo = static_cast<char*>(q);
+  const int64_t chunks = hidden / 8;
+  if (hidden % 8 != 0 || chunks > 256 * 8) {
+    token_quant_generic_kernel<DT, MODE><<<dim3((uint32_t)rows), dim3(256), 0, st>>>(xi, qo, s, row_sum, hidden);
+    return check_launch(name);
+  }
+#define SGLQ_TQ(TEAM, V)                                                                                         \
+  token_quant_kernel<DT, TEAM, V, MODE><<<dim3((uint32_t)((rows + (256 / TEAM) - 1) / (256 / TEAM))), dim3(256), 0, st>>>( \
+      xi, qo, s, row_sum, rows, (uint32_t)chunks)
+  if (chunks <= 64) SGLQ_TQ(64, 1);
+  else if (chunks <= 128) SGLQ_TQ(64, 2);
+  else if (chunks <= 256) SGLQ_TQ(64, 4);
+  else if (chunks <= 512) SGLQ_TQ(256, 2);
+  else if (chunks <= 1024) SGLQ_TQ(256, 4);
+  else SGLQ_TQ(256, 8);
+#undef SGLQ_TQ
+  return check_launch(name);
+}
+
+template <int MODE>
+static int token_quant_entry(const char* name, const void* input, int in_dtype, void* output_q, float* output_s,
+                             void* row_sum, int64_t num_tokens, int64_t hidden, void* stream) {
+  if (num_tokens == 0) return SGLQ_OK;
+  if (!input || !output_q || !output_s) {
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_tokens < 0 || hidden <= 0 || num_tokens >= (1ll << 31)) {
+    set_error("%s: bad shape [%lld, %lld]", name, (long long)num_tokens, (long long)hidden);
+    return SGLQ_EINVAL;
+  }
+  if (MODE == MODE_FP8 && hidden % 8 != 0) {
+    set_error("%s: Hidden dimension must be divisible by 8, but got %lld", name, (long long)hidden);
+    return SGLQ_EINVAL;
+  }
+  if (hidden % 8 == 0 &&
+      ((reinterpret_cast<uintptr_t>(input) & 15) || (reinterpret_cast<uintptr_t>(output_q) & 7))) {
+    set_error("%s: input must be 16-byte and output_q 8-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (in_dtype) {
+    case SGLQ_BF16: return launch_token_quant<SGLQ_BF16, MODE>(name, input, output_q, output_s, row_sum, num_tokens, hidden, st);
+    case SGLQ_FP16: return launch_token_quant<SGLQ_FP16, MODE>(name, input, output_q, output_s, row_sum, num_tokens, hidden, st);
+    case SGLQ_FP32: return launch_token_quant<SGLQ_FP32, MODE>(name, input, output_q, output_s, row_sum, num_tokens, hidden, st);
+  }
+  set_error("%s: unsupported in_dtype %d", name, in_dtype);
+  return SGLQ_EUNSUPPORTED;
+}
+
+}  // namespace sglq
+
+extern "C" int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                              int64_t num_tokens, int64_t hidden, int group_size,
+                                              int64_t s_stride_row, int64_t s_stride_col, float eps, float fp8_min,
+                                              float fp8_max, void* stream) {
+  return sglq::group_quant_entry<false>("sgl_per_token_group_quant_fp8", input, in_dtype, output_q, output_s,
+                                        num_tokens, hidden, group_size, s_stride_row, s_stride_col, eps, fp8_min,
+                                        fp8_max, stream);
+}
+
+extern "C" int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                               int64_t num_tokens, int64_t hidden, int group_size,
+                                               int64_t s_stride_row, int64_t s_stride_col, float eps, float int8_min,
+                                               float int8_max, void* stream) {
+  return sglq::group_quant_entry<true>("sgl_per_token_group_quant_int8", input, in_dtype, output_q, output_s,
+                                       num_tokens, hidden, group_size, s_stride_row, s_stride_col, eps, int8_min,
+                                       int8_max, stream);
+}
+
+extern "C" int sglq_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                        int64_t num_tokens, int64_t hidden, void* stream) {
+  return sglq::token_quant_entry<sglq::MODE_FP8>("sgl_per_token_quant_fp8", input, in_dtype, output_q, output_s,
+                                                 nullptr, num_tokens, hidden, stream);
+}
+
+extern "C" int sglq_per_token_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                         void* row_sum, int64_t num_tokens, int64_t hidden, void* stream) {
+  return sglq::token_quant_entry<sglq::MODE_INT8>("per_token_quant_int8", input, in_dtype, output_q, output_s,
+                                                  row_sum, num_tokens, hidden, stream);
+}

@@ -1,0 +1,77 @@
+"""Host-side quantization helpers of the FP8 path, mirroring the callers in
+python/sglang/srt/layers/quantization/fp8_kernel.py (names, arguments, returned
+layouts), on top of the HIP operators."""
+
+from __future__ import annotations
+
+import torch
+
+from ..sgl_kernel import sgl_per_token_group_quant_fp8, sgl_per_token_quant_fp8
+
+# gfx950 implements the OCP formats: e4m3fn with maximum 448 (fp8_kernel.py:71-85
+# selects the fnuz/224 variant only for gfx94x).
+fp8_dtype = torch.float8_e4m3fn
+fp8_max = torch.finfo(fp8_dtype).max
+fp8_min = -fp8_max
+
+
+def create_per_token_group_quant_fp8_output_scale(
+    x_shape,
+    device,
+    group_size,
+    column_major_scales: bool,
+    scale_tma_aligned: bool,
+    scale_ue8m0: bool,
+):
+    """Scale buffer in the layout the consumer GEMM wants (fp8_kernel.py:300-341)."""
+    if scale_ue8m0:
+        raise NotImplementedError("packed UE8M0 scales are not built")
+    if column_major_scales:
+        if scale_tma_aligned:
+            aligned_size = (x_shape[-2] + 3) // 4 * 4
+            return torch.empty(
+                x_shape[:-2] + (x_shape[-1] // group_size, aligned_size), device=device, dtype=torch.float32
+            ).permute(-1, -2)[: x_shape[-2], :]
+        return torch.empty(
+            (x_shape[-1] // group_size,) + x_shape[:-1], device=device, dtype=torch.float32
+        ).permute(-1, -2)
+    return torch.empty(x_shape[:-1] + (x_shape[-1] // group_size,), device=device, dtype=torch.float32)
+
+
+def sglang_per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    column_major_scales: bool = False,
+    scale_tma_aligned: bool = False,
+    scale_ue8m0: bool = False,
+):
+    """fp8_kernel.py:344-372."""
+    assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
+    assert x.is_contiguous(), "`x` is not contiguous"
+    x_q = torch.empty_like(x, device=x.device, dtype=fp8_dtype)
+    x_s = create_per_token_group_quant_fp8_output_scale(
+        x_shape=tuple(x.shape),
+        device=x.device,
+        group_size=group_size,
+        column_major_scales=column_major_scales,
+        scale_tma_aligned=scale_tma_aligned,
+        scale_ue8m0=scale_ue8m0,
+    )
+    if x.shape[0] > 0:
+        sgl_per_token_group_quant_fp8(x, x_q, x_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0)
+    return x_q, x_s
+
+
+# The reference's `per_token_group_quant_fp8` (fp8_kernel.py:217-297) is the Triton
+# twin with the same signature; here both names run the HIP kernel.
+per_token_group_quant_fp8 = sglang_per_token_group_quant_fp8
+
+
+def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
+    """fp8_kernel.py:375-391."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    x_q = torch.empty_like(x, device=x.device, dtype=dtype)
+    x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
+    sgl_per_token_quant_fp8(x, x_q, x_s)
+    return x_q, x_s

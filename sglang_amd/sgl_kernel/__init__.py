@@ -1,0 +1,22 @@
+"""Stand-in for the part of the reference's ``sgl_kernel`` package that serves the
+W8A8 quantized-linear path (sgl-kernel/python/sgl_kernel/__init__.py)."""
+
+from .gemm import (
+    fp8_blockwise_scaled_mm,
+    fp8_scaled_mm,
+    int8_mm_i32,
+    int8_scaled_mm,
+    sgl_per_token_group_quant_fp8,
+    sgl_per_token_group_quant_int8,
+    sgl_per_token_quant_fp8,
+)
+
+__all__ = [
+    "fp8_blockwise_scaled_mm",
+    "fp8_scaled_mm",
+    "int8_mm_i32",
+    "int8_scaled_mm",
+    "sgl_per_token_group_quant_fp8",
+    "sgl_per_token_group_quant_int8",
+    "sgl_per_token_quant_fp8",
+]

@@ -1,0 +1,294 @@
+"""Operators of the W8A8 path under their ``sgl_kernel`` names and signatures
+(sgl-kernel/python/sgl_kernel/gemm.py:13-42,100-145).
+
+Each public function forwards positionally to ``torch.ops.sgl_kernel.<op>``,
+as the reference wrappers do; the op implementations registered here validate
+their arguments the way the reference's C++ entry points do (same conditions,
+``RuntimeError`` on violation), allocate the output with torch and enqueue the
+HIP kernel on the current stream through the C ABI.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from .._lib import DTYPE_CODE
+
+FP8 = torch.float8_e4m3fn
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+# ---------------------------------------------------------------------------
+# argument validation (device-independent so that it can be exercised on CPU tensors)
+# ---------------------------------------------------------------------------
+def check_mm_common(mat_a, mat_b, out_dtype, elem_dtype, elem_name, require_cuda=True):
+    """Checks shared by the three GEMM entry points
+    (int8_gemm_kernel.cu:670-683, fp8_gemm_kernel.cu:1078-1094,
+    fp8_blockwise_gemm_kernel.cu:351-365)."""
+    if require_cuda:
+        _check(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+        _check(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _check(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _check(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _check(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _check(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _check(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _check((mat_a.size(1) * mat_a.element_size()) % 16 == 0, "mat_a must be multiple of 16 bytes for memory alignment")
+    _check((mat_b.size(0) * mat_b.element_size()) % 16 == 0, "mat_b must be multiple of 16 bytes for memory alignment")
+    _check(mat_a.dtype == elem_dtype, f"mat_a must be {elem_name}")
+    _check(mat_b.dtype == elem_dtype, f"mat_b must be {elem_name}")
+    _check(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+    # kernel-side requirements on strides that the reference leaves to its GEMM library
+    _check(mat_a.size(0) <= 1 or mat_a.stride(0) % 16 == 0, "mat_a row stride must be a multiple of 16 bytes")
+    _check(mat_b.size(1) <= 1 or mat_b.stride(1) % 16 == 0, "mat_b column stride must be a multiple of 16 bytes")
+
+
+def check_rowcol_scales(mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
+    """int8_gemm_kernel.cu:685-696 / fp8_gemm_kernel.cu:1096-1105."""
+    _check(scales_a.numel() == mat_a.size(0), "size of scales_a is not matched")
+    _check(scales_b.numel() == mat_b.size(1), "size of scales_b is not matched")
+    _check(scales_a.is_contiguous(), "scales_a must be contiguous")
+    _check(scales_b.is_contiguous(), "scales_b msut be contiguous")
+    _check(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _check(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    if bias is not None:
+        _check(bias.numel() == mat_b.size(1), "size of bias is not matched")
+        _check(bias.is_contiguous(), "bias must be contiguous")
+        _check(bias.dtype == out_dtype, "bias dtype must match output dtype")
+
+
+def _is_contiguous_vector(t: torch.Tensor) -> bool:
+    return t.is_contiguous() and (t.dim() == 1 or (t.dim() == 2 and min(t.shape) == 1))
+
+
+def check_blockwise_scales(mat_a, mat_b, scales_a, scales_b):
+    """fp8_blockwise_gemm_kernel.cu:367-380.  Scale extents use ceil division so
+    that N (or K) that is not a multiple of 128 is accepted with the scale shapes
+    the callers allocate (fp8.py:276-306); for multiples of 128 this is the
+    reference's condition."""
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    _check(scales_a.dim() == 2 and scales_b.dim() == 2, "scales must be 2D tensors")
+    _check(m == scales_a.size(0), "size of scales_a is not matched")
+    _check((k + 127) // 128 == scales_a.size(1), "size of scales_a is not matched")
+    _check(scales_a.stride(0) == 1 or _is_contiguous_vector(scales_a), "scales_a must be M major")
+    _check((k + 127) // 128 == scales_b.size(0), "size of scales_b is not matched")
+    _check((n + 127) // 128 == scales_b.size(1), "size of scales_b is not matched")
+    _check(scales_b.stride(0) == 1 or _is_contiguous_vector(scales_b), "scales_b must be K major")
+    _check(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _check(scales_b.dtype == torch.float32, "scales_b must be Float32")
+
+
+def check_group_quant(input, output_q, output_s, group_size, q_dtype, require_cuda=True):
+    """per_token_group_quant_8bit.cu:125-131 (+ CHECK_INPUT = CUDA and contiguous)."""
+    for name, t in (("input", input), ("output_q", output_q)):
+        if require_cuda:
+            _check(t.is_cuda, f"{name} must be a CUDA tensor")
+        _check(t.is_contiguous(), f"{name} must be contiguous")
+    if require_cuda:
+        _check(output_s.is_cuda, "output_s must be a CUDA tensor")
+    _check(input.dtype in DTYPE_CODE, "input must be Float, Half or BFloat16")
+    _check(output_q.dtype == q_dtype, f"output_q must be {q_dtype}")
+    _check(output_q.shape == input.shape, "output_q must have the shape of input")
+    _check(group_size > 0 and input.numel() % group_size == 0, "input.numel() must be divisible by group_size")
+    _check(input.dim() >= 1 and input.shape[-1] % group_size == 0, "the last dimension must be divisible by group_size")
+    _check(output_s.dim() == 2, "output_s must be a 2D tensor")
+    _check(output_s.dtype == torch.float32, "output_s must be Float32")
+    rows = input.numel() // input.shape[-1] if input.numel() else 0
+    _check(tuple(output_s.shape) == (rows, input.shape[-1] // group_size), "output_s has the wrong shape")
+
+
+def check_token_quant_fp8(input, output_q, output_s, require_cuda=True):
+    """per_token_quant_fp8.cu:166-173."""
+    for name, t in (("input", input), ("output_q", output_q), ("output_s", output_s)):
+        if require_cuda:
+            _check(t.is_cuda, f"{name} must be a CUDA tensor")
+        _check(t.is_contiguous(), f"{name} must be contiguous")
+    _check(input.dim() == 2, "input must be a 2D tensor")
+    _check(input.dtype in DTYPE_CODE, "input must be Float, Half or BFloat16")
+    _check(output_q.dtype == FP8 and output_q.shape == input.shape, "output_q must be Float8_e4m3fn with input's shape")
+    _check(output_s.dtype == torch.float32 and output_s.numel() == input.size(0), "output_s must hold one Float32 per token")
+    _check(input.size(1) % 8 == 0, f"Hidden dimension must be divisible by 8, but got {input.size(1)}")
+
+
+# ---------------------------------------------------------------------------
+# op implementations (CUDA dispatch key = ROCm device tensors)
+# ---------------------------------------------------------------------------
+def _int8_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    check_mm_common(mat_a, mat_b, out_dtype, torch.int8, "Int8")
+    _check(mat_a.size(1) % 16 == 0, "mat_a.size(1) must be multiple of 16 for memory alignment")
+    _check(mat_b.size(0) % 16 == 0, "mat_b.size(0) must be multiple of 16 for memory alignment")
+    _check(mat_b.size(1) % 8 == 0, "mat_b.size(1) must be multiple of 8 for memory alignment")
+    check_rowcol_scales(mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    out = torch.empty((m, n), dtype=out_dtype, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_int8_scaled_mm(
+        mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_a.data_ptr(), scales_b.data_ptr(), bias.data_ptr() if bias is not None else None,
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "int8_scaled_mm")
+    return out
+
+
+def _fp8_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    check_mm_common(mat_a, mat_b, out_dtype, FP8, "Float8_e4m3fn")
+    check_rowcol_scales(mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((m, n), dtype=out_dtype, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_fp8_scaled_mm(
+        mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_a.data_ptr(), scales_b.data_ptr(), bias.data_ptr() if bias is not None else None,
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "fp8_scaled_mm")
+    return out
+
+
+def _fp8_blockwise_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    check_mm_common(mat_a, mat_b, out_dtype, FP8, "Float8_e4m3fn")
+    check_blockwise_scales(mat_a, mat_b, scales_a, scales_b)
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((m, n), dtype=out_dtype, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_fp8_blockwise_scaled_mm(
+        mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
+        scales_b.data_ptr(), scales_b.stride(0), scales_b.stride(1),
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "fp8_blockwise_scaled_mm")
+    return out
+
+
+def _group_quant_impl(fn_name, q_dtype, input, output_q, output_s, group_size, eps, qmin, qmax):
+    check_group_quant(input, output_q, output_s, group_size, q_dtype)
+    if input.numel() == 0:
+        return
+    hidden = input.shape[-1]
+    rows = input.numel() // hidden
+    lib = _lib.load()
+    rc = getattr(lib, fn_name)(
+        input.data_ptr(), DTYPE_CODE[input.dtype], output_q.data_ptr(), output_s.data_ptr(), rows, hidden,
+        int(group_size), output_s.stride(0), output_s.stride(1), float(eps), float(qmin), float(qmax),
+        _lib.stream_ptr(input.device))
+    _lib.check(rc, fn_name)
+
+
+def _sgl_per_token_group_quant_fp8_impl(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0):
+    if scale_ue8m0:
+        raise NotImplementedError("sgl_per_token_group_quant_fp8: scale_ue8m0=True (packed power-of-two scales) is not built")
+    _group_quant_impl("sglq_per_token_group_quant_fp8", FP8, input, output_q, output_s, group_size, eps, fp8_min, fp8_max)
+
+
+def _sgl_per_token_group_quant_int8_impl(input, output_q, output_s, group_size, eps, int8_min, int8_max):
+    _group_quant_impl("sglq_per_token_group_quant_int8", torch.int8, input, output_q, output_s, group_size, eps, int8_min, int8_max)
+
+
+def _sgl_per_token_quant_fp8_impl(input, output_q, output_s):
+    check_token_quant_fp8(input, output_q, output_s)
+    if input.numel() == 0:
+        return
+    lib = _lib.load()
+    rc = lib.sglq_per_token_quant_fp8(
+        input.data_ptr(), DTYPE_CODE[input.dtype], output_q.data_ptr(), output_s.data_ptr(),
+        input.size(0), input.size(1), _lib.stream_ptr(input.device))
+    _lib.check(rc, "sgl_per_token_quant_fp8")
+
+
+_SCHEMAS = {
+    # sgl-kernel/csrc/common_extension.cc:101-130
+    "int8_scaled_mm": "(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? bias) -> Tensor",
+    "fp8_scaled_mm": "(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? bias) -> Tensor",
+    "fp8_blockwise_scaled_mm": "(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype) -> Tensor",
+    "sgl_per_token_group_quant_fp8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s, int group_size, float eps, float fp8_min, float fp8_max, bool scale_ue8m0) -> ()",
+    "sgl_per_token_group_quant_int8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s, int group_size, float eps, float int8_min, float int8_max) -> ()",
+    "sgl_per_token_quant_fp8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s) -> ()",
+}
+_IMPLS = {
+    "int8_scaled_mm": _int8_scaled_mm_impl,
+    "fp8_scaled_mm": _fp8_scaled_mm_impl,
+    "fp8_blockwise_scaled_mm": _fp8_blockwise_scaled_mm_impl,
+    "sgl_per_token_group_quant_fp8": _sgl_per_token_group_quant_fp8_impl,
+    "sgl_per_token_group_quant_int8": _sgl_per_token_group_quant_int8_impl,
+    "sgl_per_token_quant_fp8": _sgl_per_token_quant_fp8_impl,
+}
+
+_library = torch.library.Library("sgl_kernel", "FRAGMENT")
+for _name, _schema in _SCHEMAS.items():
+    _library.define(_name + _schema)
+    _library.impl(_name, _IMPLS[_name], "CUDA")
+
+
+# ---------------------------------------------------------------------------
+# public wrappers: same names, argument order and forwarding as the reference
+# ---------------------------------------------------------------------------
+def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    return torch.ops.sgl_kernel.int8_scaled_mm.default(mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+
+
+def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    return torch.ops.sgl_kernel.fp8_blockwise_scaled_mm.default(mat_a, mat_b, scales_a, scales_b, out_dtype)
+
+
+def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    return torch.ops.sgl_kernel.fp8_scaled_mm.default(mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+
+
+def sgl_per_token_group_quant_fp8(
+    input: torch.Tensor,
+    output_q: torch.Tensor,
+    output_s: torch.Tensor,
+    group_size: int,
+    eps: float,
+    fp8_min: float,
+    fp8_max: float,
+    scale_ue8m0: bool,
+) -> None:
+    torch.ops.sgl_kernel.sgl_per_token_group_quant_fp8.default(
+        input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0
+    )
+
+
+def sgl_per_token_group_quant_int8(
+    input: torch.Tensor,
+    output_q: torch.Tensor,
+    output_s: torch.Tensor,
+    group_size: int,
+    eps: float,
+    int8_min: float,
+    int8_max: float,
+) -> None:
+    torch.ops.sgl_kernel.sgl_per_token_group_quant_int8.default(
+        input, output_q, output_s, group_size, eps, int8_min, int8_max
+    )
+
+
+def sgl_per_token_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
+    torch.ops.sgl_kernel.sgl_per_token_quant_fp8.default(input, output_q, output_s)
+
+
+def int8_mm_i32(mat_a: torch.Tensor, mat_b: torch.Tensor) -> torch.Tensor:
+    """INT32 accumulators of ``int8_scaled_mm`` before its epilogue (no reference
+    counterpart; used to compare the accumulators bit for bit)."""
+    check_mm_common(mat_a, mat_b, torch.bfloat16, torch.int8, "Int8")
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    out = torch.empty((m, n), dtype=torch.int32, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_int8_mm_i32(mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(),
+                              mat_b.stride(1) if n > 1 else k, out.data_ptr(), out.stride(0), m, n, k,
+                              _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "int8_mm_i32")
+    return out

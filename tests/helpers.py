@@ -1,0 +1,62 @@
+"""Shared helpers for the tests: dtype plumbing between torch and the C oracle."""
+import ctypes
+
+import numpy as np
+import torch
+
+DT = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+
+def raw_ptr(t: torch.Tensor):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def c_group_quant_fp8(lib, x: torch.Tensor, group: int, eps=1e-10, lo=-448.0, hi=448.0):
+    x = x.contiguous()
+    n = x.numel()
+    q = torch.empty(n, dtype=torch.uint8)
+    s = torch.empty(n // group, dtype=torch.float32)
+    lib.oracle_group_quant_fp8(raw_ptr(x), DT[x.dtype], ctypes.c_int64(n // group), ctypes.c_int(group),
+                               ctypes.c_float(eps), ctypes.c_float(lo), ctypes.c_float(hi), raw_ptr(q), raw_ptr(s))
+    return q.reshape(x.shape), s.reshape(x.shape[:-1] + (x.shape[-1] // group,))
+
+
+def c_token_quant_int8(lib, x: torch.Tensor):
+    x = x.contiguous()
+    rows, cols = x.numel() // x.shape[-1], x.shape[-1]
+    q = torch.empty(x.shape, dtype=torch.int8)
+    s = torch.empty(rows, dtype=torch.float32)
+    lib.oracle_token_quant_int8(raw_ptr(x), DT[x.dtype], ctypes.c_int64(rows), ctypes.c_int64(cols), raw_ptr(q), raw_ptr(s))
+    return q, s.reshape(x.shape[:-1] + (1,))
+
+
+def c_token_quant_fp8(lib, x: torch.Tensor):
+    x = x.contiguous()
+    rows, cols = x.shape
+    q = torch.empty(x.shape, dtype=torch.uint8)
+    s = torch.empty(rows, dtype=torch.float32)
+    lib.oracle_token_quant_fp8(raw_ptr(x), DT[x.dtype], ctypes.c_int64(rows), ctypes.c_int64(cols), raw_ptr(q), raw_ptr(s))
+    return q, s.reshape(rows, 1)
+
+
+def fp8_bits(t: torch.Tensor) -> torch.Tensor:
+    return t.view(torch.uint8)
+
+
+def f32_bits(t: torch.Tensor) -> torch.Tensor:
+    return t.contiguous().view(torch.int32)
+
+
+def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
+    got, want = got.cpu(), want.cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    if got.dtype == torch.float32:
+        got, want = f32_bits(got), f32_bits(want)
+    elif got.dtype == torch.float8_e4m3fn:
+        got, want = fp8_bits(got), fp8_bits(want)
+    bad = (got != want)
+    nbad = int(bad.sum())
+    if nbad:
+        idx = bad.nonzero()[:5].tolist()
+        raise AssertionError(f"{what}: {nbad} of {got.numel()} elements differ, first at {idx}: "
+                             f"got {[got[tuple(i)].item() for i in idx]} want {[want[tuple(i)].item() for i in idx]}")

@@ -1,0 +1,164 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+symbol the header declares, the torch ops are registered under the reference's
+schemas, and argument validation raises what the reference's entry points raise."""
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+FP8 = torch.float8_e4m3fn
+
+
+def declared_symbols():
+    text = (ROOT / "include" / "sglq.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sglq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from sglang_amd import _lib
+
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/sglq.h but not exported"
+    assert lib.sglq_abi_version() == 1
+    assert set(_lib.SIGNATURES) <= set(names)
+
+
+def test_ops_registered_with_reference_schemas():
+    import sglang_amd.sgl_kernel  # noqa: F401
+
+    want = {
+        "int8_scaled_mm": ["mat_a", "mat_b", "scales_a", "scales_b", "out_dtype", "bias"],
+        "fp8_scaled_mm": ["mat_a", "mat_b", "scales_a", "scales_b", "out_dtype", "bias"],
+        "fp8_blockwise_scaled_mm": ["mat_a", "mat_b", "scales_a", "scales_b", "out_dtype"],
+        "sgl_per_token_group_quant_fp8": ["input", "output_q", "output_s", "group_size", "eps", "fp8_min", "fp8_max", "scale_ue8m0"],
+        "sgl_per_token_group_quant_int8": ["input", "output_q", "output_s", "group_size", "eps", "int8_min", "int8_max"],
+        "sgl_per_token_quant_fp8": ["input", "output_q", "output_s"],
+    }
+    for name, args in want.items():
+        schema = getattr(torch.ops.sgl_kernel, name).default._schema
+        assert [a.name for a in schema.arguments] == args
+
+
+def test_cpu_tensors_are_refused_by_dispatch():
+    from sglang_amd.sgl_kernel import int8_scaled_mm
+
+    a = torch.zeros(4, 16, dtype=torch.int8)
+    with pytest.raises(NotImplementedError):
+        int8_scaled_mm(a, a.t(), torch.ones(4), torch.ones(4), torch.bfloat16)
+
+
+def test_mm_argument_validation_messages():
+    from sglang_amd.sgl_kernel import gemm as G
+
+    a = torch.zeros(4, 32, dtype=torch.int8)
+    w = torch.zeros(8, 32, dtype=torch.int8)
+    ok = dict(out_dtype=torch.bfloat16, elem_dtype=torch.int8, elem_name="Int8", require_cuda=False)
+    G.check_mm_common(a, w.t(), **ok)
+    with pytest.raises(RuntimeError, match="mat_a must be a CUDA tensor"):
+        G.check_mm_common(a, w.t(), torch.bfloat16, torch.int8, "Int8")
+    with pytest.raises(RuntimeError, match="mat_b must be a column major tensor"):
+        G.check_mm_common(a, torch.zeros(32, 8, dtype=torch.int8), **ok)
+    with pytest.raises(RuntimeError, match="mat_a must be a row major tensor"):
+        G.check_mm_common(torch.zeros(32, 4, dtype=torch.int8).t(), w.t(), **ok)
+    with pytest.raises(RuntimeError, match="cannot be multiplied"):
+        G.check_mm_common(a, torch.zeros(8, 48, dtype=torch.int8).t(), **ok)
+    with pytest.raises(RuntimeError, match="multiple of 16 bytes"):
+        G.check_mm_common(torch.zeros(4, 24, dtype=torch.int8), torch.zeros(8, 24, dtype=torch.int8).t(), **ok)
+    with pytest.raises(RuntimeError, match="mat_a must be Int8"):
+        G.check_mm_common(a.to(torch.uint8), w.t(), **ok)
+    with pytest.raises(RuntimeError, match="out_dtype must be Half or BFloat16"):
+        G.check_mm_common(a, w.t(), torch.float32, torch.int8, "Int8", require_cuda=False)
+    with pytest.raises(RuntimeError, match="mat_a must be a 2D tensor"):
+        G.check_mm_common(a[None], w.t(), **ok)
+
+    sa, sb = torch.ones(4, 1), torch.ones(8, 1)
+    G.check_rowcol_scales(a, w.t(), sa, sb, torch.bfloat16, None)
+    with pytest.raises(RuntimeError, match="size of scales_a is not matched"):
+        G.check_rowcol_scales(a, w.t(), torch.ones(3), sb, torch.bfloat16, None)
+    with pytest.raises(RuntimeError, match="scales_b must be Float32"):
+        G.check_rowcol_scales(a, w.t(), sa, sb.double(), torch.bfloat16, None)
+    with pytest.raises(RuntimeError, match="bias dtype must match output dtype"):
+        G.check_rowcol_scales(a, w.t(), sa, sb, torch.bfloat16, torch.zeros(8, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="size of bias is not matched"):
+        G.check_rowcol_scales(a, w.t(), sa, sb, torch.bfloat16, torch.zeros(7, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="scales_a must be contiguous"):
+        G.check_rowcol_scales(a, w.t(), torch.ones(4, 2)[:, 0], sb, torch.bfloat16, None)
+
+
+def test_blockwise_scale_validation():
+    from sglang_amd.sgl_kernel import gemm as G
+
+    a = torch.zeros(6, 256, dtype=FP8)
+    w = torch.zeros(384, 256, dtype=FP8)
+    sfa = torch.zeros(2, 6).t()          # [M, K/128] M-major
+    sfb = torch.zeros(3, 2).t()          # weight_scale_inv [N/128, K/128] transposed -> K-major
+    G.check_blockwise_scales(a, w.t(), sfa, sfb)
+    with pytest.raises(RuntimeError, match="scales_a must be M major"):
+        G.check_blockwise_scales(a, w.t(), torch.zeros(6, 2), sfb)
+    with pytest.raises(RuntimeError, match="scales_b must be K major"):
+        G.check_blockwise_scales(a, w.t(), sfa, torch.zeros(2, 3))
+    with pytest.raises(RuntimeError, match="size of scales_b is not matched"):
+        G.check_blockwise_scales(a, w.t(), sfa, torch.zeros(2, 2).t())
+    with pytest.raises(RuntimeError, match="size of scales_a is not matched"):
+        G.check_blockwise_scales(a, w.t(), torch.zeros(3, 6).t(), sfb)
+    # ceil-division: N = 136 takes two scale columns
+    G.check_blockwise_scales(a, torch.zeros(136, 256, dtype=FP8).t(), sfa, torch.zeros(2, 2).t())
+
+
+def test_quant_argument_validation():
+    from sglang_amd.sgl_kernel import gemm as G
+
+    x = torch.zeros(4, 256, dtype=torch.bfloat16)
+    q = torch.zeros(4, 256, dtype=FP8)
+    G.check_group_quant(x, q, torch.zeros(4, 2), 128, FP8, require_cuda=False)
+    G.check_group_quant(x, q, torch.zeros(2, 4).t(), 128, FP8, require_cuda=False)  # column-major scales
+    with pytest.raises(RuntimeError, match="divisible by group_size"):
+        G.check_group_quant(x, q, torch.zeros(4, 2), 96, FP8, require_cuda=False)
+    with pytest.raises(RuntimeError, match="output_s must be a 2D tensor"):
+        G.check_group_quant(x, q, torch.zeros(8), 128, FP8, require_cuda=False)
+    with pytest.raises(RuntimeError, match="input must be contiguous"):
+        G.check_group_quant(torch.zeros(256, 4, dtype=torch.bfloat16).t(), q, torch.zeros(4, 2), 128, FP8, require_cuda=False)
+    with pytest.raises(RuntimeError, match="input must be a CUDA tensor"):
+        G.check_group_quant(x, q, torch.zeros(4, 2), 128, FP8)
+    with pytest.raises(RuntimeError, match="Hidden dimension must be divisible by 8, but got 12"):
+        G.check_token_quant_fp8(torch.zeros(2, 12), torch.zeros(2, 12, dtype=FP8), torch.zeros(2, 1), require_cuda=False)
+
+
+def test_scale_buffer_layouts_match_reference_allocator():
+    from sglang_amd.quantization.fp8_kernel import create_per_token_group_quant_fp8_output_scale as mk
+
+    s = mk((6, 512), "cpu", 128, False, False, False)
+    assert tuple(s.shape) == (6, 4) and s.is_contiguous()
+    s = mk((6, 512), "cpu", 128, True, False, False)
+    assert tuple(s.shape) == (6, 4) and s.stride() == (1, 6)
+    s = mk((6, 512), "cpu", 128, True, True, False)
+    assert tuple(s.shape) == (6, 4) and s.stride() == (1, 8)
+    with pytest.raises(NotImplementedError):
+        mk((6, 512), "cpu", 128, True, True, True)
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu():
+    """Entry points validate before they touch the device."""
+    from sglang_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(4096, dtype=torch.uint8)
+    p = buf.data_ptr()
+    rc = lib.sglq_per_token_group_quant_fp8(p, 0, p, p, 4, 100, 128, 1, 1, 1e-10, -448.0, 448.0, None)
+    assert rc == 1 and b"multiple of group_size" in lib.sglq_last_error()
+    rc = lib.sglq_per_token_group_quant_fp8(p, 0, p, p, 4, 96, 48, 2, 1, 1e-10, -448.0, 448.0, None)
+    assert rc == 2  # group size not built
+    rc = lib.sglq_per_token_quant_fp8(p, 0, p, p, 4, 12, None)
+    assert rc == 1 and b"divisible by 8" in lib.sglq_last_error()
+    rc = lib.sglq_int8_scaled_mm(p, 24, p, 24, p, p, None, p, 8, 0, 4, 8, 24, None)
+    assert rc == 1 and b"multiple of 16" in lib.sglq_last_error()
+    rc = lib.sglq_fp8_blockwise_scaled_mm(p, 128, p, 128, p, 1, 4, p, 1, 1, p, 8, 2, 4, 8, 128, None)
+    assert rc == 1 and b"out_dtype" in lib.sglq_last_error()
+    # empty problems are a no-op
+    assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None) == 0

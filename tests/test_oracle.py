@@ -1,0 +1,291 @@
+"""Pins the CPU oracle (oracle/w8a8_oracle.py) without the reference: closed forms,
+an independent bit-level e4m3fn encoder, the scalar C restatement, torch's own
+CPU casts, float64/int64 brute force.  The reference holds no golden vectors for
+this path (its tests draw fresh random tensors), so none are compared."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bits_equal, c_group_quant_fp8, c_token_quant_fp8, c_token_quant_int8, fp8_bits
+from oracle import w8a8_oracle as O
+
+FP8 = torch.float8_e4m3fn
+
+
+def all_e4m3_values():
+    codes = torch.arange(256, dtype=torch.uint8)
+    vals = O.e4m3fn_decode(codes)
+    return codes, vals
+
+
+# ------------------------------------------------------------------ e4m3fn
+def test_e4m3_decode_matches_torch_and_c(c_oracle):
+    codes, vals = all_e4m3_values()
+    tv = codes.view(FP8).to(torch.float32)
+    finite = ~torch.isnan(vals)
+    assert torch.equal(torch.isnan(tv), torch.isnan(vals))
+    assert torch.equal(tv[finite], vals[finite])
+    assert vals[finite].abs().max().item() == 448.0
+    assert int(finite.sum()) == 254
+    for c in range(256):
+        cv = c_oracle.oracle_e4m3fn_decode(c)
+        assert (math.isnan(cv) and math.isnan(vals[c].item())) or cv == vals[c].item()
+
+
+def test_e4m3_encode_three_ways_agree(c_oracle):
+    """Every representable value, every midpoint between neighbours (the ties) and
+    the floats just below/above each midpoint: bit-twiddling C encoder, the
+    float64 formula encoder and torch's CPU cast give the same byte."""
+    _, vals = all_e4m3_values()
+    pos = torch.sort(vals[(~torch.isnan(vals)) & (vals >= 0)]).values.unique()
+    mids = (pos[:-1].double() + pos[1:].double()) / 2
+    mids32 = mids.float()
+    assert torch.equal(mids32.double(), mids)  # midpoints are exact in fp32
+    cand = torch.cat([pos, mids32, torch.nextafter(mids32, torch.tensor(0.0)), torch.nextafter(mids32, torch.tensor(1e9))])
+    g = torch.Generator().manual_seed(1)
+    cand = torch.cat([cand, torch.rand(200000, generator=g) * 448, torch.rand(50000, generator=g) * 0.05])
+    cand = torch.cat([cand, -cand]).clamp(-448, 448)
+    want = fp8_bits(cand.to(FP8))
+    got_formula = O.e4m3fn_encode_rne(cand)
+    got_c = torch.tensor([c_oracle.oracle_e4m3fn_encode(ctypes.c_float(v)) for v in cand[: 4 * len(pos) * 2 + 4000].tolist()],
+                         dtype=torch.uint8)
+    # -0.0 keeps its sign bit in all three
+    assert_bits_equal(got_formula, want, "formula encoder vs torch cast")
+    assert_bits_equal(got_c, want[: got_c.numel()], "C encoder vs torch cast")
+
+
+def test_e4m3_ties_go_to_even():
+    # 17 lies midway between 16 (mantissa 000) and 18 (001): even is 16; 19 -> 20
+    x = torch.tensor([17.0, 19.0, -17.0, 0.0009765625, 464.0 - 16.0])
+    got = x.to(FP8).float()
+    assert got.tolist() == [16.0, 20.0, -16.0, 0.0, 448.0]
+    assert O.e4m3fn_decode(O.e4m3fn_encode_rne(x)).tolist() == got.tolist()
+
+
+# ------------------------------------------------------------------ a1 group quant
+def make_closed_form_groups(m, groups, group=128, seed=0, dtype=torch.float32):
+    """x = value(code) * scale with +-448 present in every group and power-of-two
+    scales, so scale and codes are known without any division rounding
+    (the construction of test/srt/quant/test_fp8_kernel.py:24-44)."""
+    g = torch.Generator().manual_seed(seed)
+    codes = torch.randint(0, 256, (m, groups, group), generator=g, dtype=torch.int32)
+    codes = torch.where((codes & 0x7F) == 0x7F, codes & 0x80, codes)  # no NaN codes
+    codes[:, :, 0] = torch.where(torch.rand((m, groups), generator=g) < 0.5, 0x7E, 0xFE)  # +-448
+    vals = O.e4m3fn_decode(codes.to(torch.uint8))
+    exp = torch.randint(-8, 5, (m, groups, 1), generator=g)
+    scale = torch.pow(2.0, exp.float())
+    x = (vals * scale).reshape(m, groups * group)
+    return x.to(dtype), codes.to(torch.uint8).reshape(m, groups * group), scale.reshape(m, groups)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_group_quant_closed_form(dtype):
+    x, codes, scale = make_closed_form_groups(7, 5, dtype=dtype)
+    assert torch.equal(x.float(), (O.e4m3fn_decode(codes).reshape(7, 5, 128) * scale[:, :, None]).reshape(7, 640))
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    assert_bits_equal(s, scale, "scale")
+    # +0 and -0 both decode to 0: compare values, and codes where the value is non-zero
+    assert torch.equal(q.float(), O.e4m3fn_decode(codes))
+    nz = O.e4m3fn_decode(codes) != 0
+    assert torch.equal(fp8_bits(q)[nz], codes[nz])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("group", [128, 64, 32, 16])
+def test_group_quant_vs_c_restatement(c_oracle, dtype, group):
+    g = torch.Generator().manual_seed(group)
+    x = torch.randn((37, 512), generator=g)
+    x[3, 128:256] = 0  # all-zero group -> eps floor
+    x[5] *= 1e-6
+    x[6] *= 3e4 if dtype != torch.float16 else 100.0
+    x = x.to(dtype)
+    q, s = O.per_token_group_quant_fp8(x, group)
+    qc, sc = c_group_quant_fp8(c_oracle, x, group)
+    assert_bits_equal(s, sc, "scales")
+    assert_bits_equal(fp8_bits(q), qc, "codes")
+
+
+def test_group_quant_invariants():
+    x = O.gen_activation(64, 1024, seed=5, outliers=True)
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    xf = x.float().reshape(64, 8, 128)
+    amax = xf.abs().amax(dim=2)
+    assert_bits_equal(s, amax / 448.0, "scale == absmax/448 (one IEEE divide)")
+    qf = q.float().reshape(64, 8, 128)
+    # the group's max element maps to +-448
+    assert torch.equal(qf.abs().amax(dim=2), torch.full((64, 8), 448.0))
+    # dequantization error is at most half an e4m3 ulp at the quotient's binade
+    quo = (xf / s[:, :, None]).abs()
+    ulp = torch.pow(2.0, torch.floor(torch.log2(torch.clamp(quo, min=2.0**-6))) - 3)
+    assert bool(((qf.abs() - quo).abs() <= ulp / 2 * (1 + 1e-6)).all())
+    # all-zero group: scale = eps/448, codes 0
+    z = torch.zeros(2, 256, dtype=torch.bfloat16)
+    qz, sz = O.per_token_group_quant_fp8(z, 128)
+    assert_bits_equal(sz, torch.full((2, 2), 1e-10, dtype=torch.float32) / 448.0, "zero-group scale")
+    assert int(fp8_bits(qz).max()) == 0
+
+
+def test_group_scale_buffer_layouts():
+    for cm, tma in ((False, False), (True, False), (True, True)):
+        b = O.make_group_scale_buffer(6, 512, 128, cm, tma)
+        assert tuple(b.shape) == (6, 4)
+        if cm:
+            assert b.stride(0) == 1 and b.stride(1) == (8 if tma else 6)
+        else:
+            assert b.is_contiguous()
+
+
+# ------------------------------------------------------------------ a2 int8 per token
+def test_int8_quant_closed_form_and_ties():
+    # x = k * (absmax / 127) with absmax = 127 * 2^j  ->  x = k * 2^j exactly, code k
+    k = torch.arange(-127, 128, dtype=torch.float32)
+    for j in (-3, 0, 4):
+        x = (k * 2.0**j).reshape(1, -1)
+        q, s = O.per_token_quant_int8(x)
+        assert q.flatten().tolist() == k.int().tolist()
+        assert s.item() == 2.0**j
+    # ties: (k + 0.5) * 2^j rounds away from zero, unlike torch.round (half to even)
+    halves = torch.tensor([[0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, -126.5, 127.0]])
+    q, s = O.per_token_quant_int8(halves)
+    assert s.item() == 1.0
+    assert q.flatten().tolist() == [1, 2, 3, -1, -2, -3, 127, -127, 127]
+    assert torch.round(halves).flatten().tolist()[:6] == [0.0, 2.0, 2.0, -0.0, -2.0, -2.0]
+    # 0.49999997 must not round up through x + 0.5
+    assert O.round_half_away(torch.tensor([0.49999997, -0.49999997, 8388609.0])).tolist() == [0.0, -0.0, 8388609.0]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_int8_quant_vs_c_restatement(c_oracle, dtype):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((19, 1000), generator=g)
+    x[2] = 0
+    x[4] *= 1e-7
+    x = x.to(dtype)
+    q, s = O.per_token_quant_int8(x)
+    qc, sc = c_token_quant_int8(c_oracle, x)
+    assert_bits_equal(s, sc, "scales")
+    assert_bits_equal(q, qc, "codes")
+    assert s[2].item() == np.float32(1e-10) / np.float32(127)
+    # library cross-check: half-even rounding differs only at exact .5 products
+    prod = x.float() * (torch.tensor(127.0) / torch.clamp(x.float().abs().amax(-1, keepdim=True), min=1e-10))
+    he = torch.round(prod).to(torch.int8)
+    diff = he != q
+    assert bool(((prod[diff] - torch.trunc(prod[diff])).abs() == 0.5).all())
+
+
+# ------------------------------------------------------------------ a3 fp8 per token
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_token_fp8_quant_vs_c_and_formula(c_oracle, dtype):
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((23, 1368), generator=g)
+    x[1] = 0  # zero row: scale 0, inverse guarded to 0, codes 0
+    x = x.to(dtype)
+    q, s = O.per_token_quant_fp8(x)
+    qc, sc = c_token_quant_fp8(c_oracle, x)
+    assert_bits_equal(s, sc, "scales")
+    assert_bits_equal(fp8_bits(q), qc, "codes")
+    assert s[1].item() == 0.0 and int(fp8_bits(q)[1].max()) == 0
+    # the reference test's formula (sgl-kernel/tests/test_per_token_quant_fp8.py:14-23) on non-zero rows
+    rows = [i for i in range(23) if i != 1]
+    want = (x.float()[rows] * (1.0 / s[rows])).clamp(-448, 448).to(FP8)
+    assert_bits_equal(q[rows], want, "codes vs reference-test formula")
+
+
+def test_token_fp8_closed_form():
+    x, codes, scale = make_closed_form_groups(9, 1, group=256, seed=11)
+    q, s = O.per_token_quant_fp8(x)
+    assert_bits_equal(s, scale.reshape(9, 1), "scale")
+    assert torch.equal(q.float(), O.e4m3fn_decode(codes))
+
+
+# ------------------------------------------------------------------ GEMMs
+def rand_fp8(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).clamp(-448, 448).to(FP8)
+
+
+def test_blockwise_mm_reduces_to_plain_matmul_with_unit_scales():
+    a, w = rand_fp8((5, 256), 1), rand_fp8((128, 256), 2)
+    sa, sb = torch.ones(5, 2), torch.ones(2, 1)
+    out = O.fp8_blockwise_scaled_mm(a, w.t(), sa, sb, torch.float32)
+    ref = a.double() @ w.double().t()
+    torch.testing.assert_close(out.double(), ref, rtol=1e-6, atol=1e-5)
+
+
+def test_blockwise_mm_one_hot_rows_select_scaled_weight_rows():
+    w = rand_fp8((256, 384), 3)
+    sb = torch.rand(3, 2) + 0.5  # [K/128, N/128]
+    sa = torch.rand(4, 3) + 0.5
+    a = torch.zeros(4, 384)
+    ks = [0, 130, 255, 383]
+    for i, k in enumerate(ks):
+        a[i, k] = 2.0
+    out = O.fp8_blockwise_scaled_mm(a.to(FP8), w.t(), sa, sb, torch.float32)
+    for i, k in enumerate(ks):
+        kb = k // 128
+        want = 2.0 * w.float()[:, k] * sa[i, kb] * sb[kb].repeat_interleave(128)
+        torch.testing.assert_close(out[i], want, rtol=1e-6, atol=0)
+
+
+def test_blockwise_mm_vs_c_double_brute_force(c_oracle):
+    m, n, k = 3, 136, 384  # N not a multiple of 128: scale index n // 128 with ceil-div shape
+    a, w = rand_fp8((m, k), 5, 50.0), rand_fp8((n, k), 6, 0.5)
+    g = torch.Generator().manual_seed(7)
+    sa = torch.rand((m, 3), generator=g) * 1e-2
+    sbw = torch.rand((2, 3), generator=g) * 1e-3  # weight_scale_inv layout [N/128, K/128]
+    out = O.fp8_blockwise_scaled_mm(a, w.t(), sa, sbw.t(), torch.float32, acc_dtype=torch.float64)
+    ref = torch.empty((m, n), dtype=torch.float64)
+    c_oracle.oracle_fp8_blockwise_mm(
+        ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(w.contiguous().data_ptr()), ctypes.c_void_p(sa.contiguous().data_ptr()),
+        ctypes.c_void_p(sbw.contiguous().data_ptr()), ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+        ctypes.c_void_p(ref.data_ptr()))
+    torch.testing.assert_close(out.double(), ref, rtol=1e-6, atol=1e-9)
+    # the reference tests' dequantize-then-matmul baseline (sgl-kernel/tests/test_fp8_blockwise_gemm.py:19-58)
+    deq_a = a.double() * sa.double().repeat_interleave(128, dim=1)
+    deq_w = w.double() * sbw.double().repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)
+    torch.testing.assert_close(out.double(), deq_a @ deq_w.t(), rtol=1e-6, atol=1e-9)
+
+
+def test_int8_accumulators_exact(c_oracle):
+    g = torch.Generator().manual_seed(8)
+    a = torch.randint(-128, 128, (5, 4096), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (24, 4096), generator=g, dtype=torch.int8)
+    acc = O.int8_mm_i32(a, w.t())
+    ref = torch.empty((5, 24), dtype=torch.int32)
+    c_oracle.oracle_int8_mm_i32(ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(w.data_ptr()), ctypes.c_int64(5),
+                                ctypes.c_int64(24), ctypes.c_int64(4096), ctypes.c_void_p(ref.data_ptr()))
+    assert torch.equal(acc, ref)
+    assert torch.equal(acc.long(), a.long() @ w.long().t())
+    # extreme case: all -128 against all -128
+    a2 = torch.full((1, 4096), -128, dtype=torch.int8)
+    assert O.int8_mm_i32(a2, a2.t()).item() == 4096 * 128 * 128
+
+
+def test_scaled_mm_epilogues_match_reference_test_formulas():
+    g = torch.Generator().manual_seed(9)
+    a8 = torch.randint(-127, 128, (6, 64), generator=g, dtype=torch.int8)
+    w8 = torch.randint(-127, 128, (16, 64), generator=g, dtype=torch.int8)
+    sa, sb = torch.rand((6, 1), generator=g), torch.rand((16, 1), generator=g)
+    bias = torch.randn(16, generator=g).to(torch.bfloat16)
+    out = O.int8_scaled_mm(a8, w8.t(), sa, sb, torch.bfloat16, bias)
+    # sgl-kernel/tests/test_int8_gemm.py:10-16
+    ref = (torch.matmul(a8.float(), w8.t().float()) * sa.view(-1, 1) * sb.view(1, -1) + bias).to(torch.bfloat16)
+    torch.testing.assert_close(out.float(), ref.float(), rtol=1e-2, atol=1e-2)
+    af, wf = rand_fp8((6, 64), 10), rand_fp8((16, 64), 11)
+    out = O.fp8_scaled_mm(af, wf.t(), sa, sb, torch.bfloat16, bias)
+    # sgl-kernel/tests/test_fp8_gemm.py:6-14
+    ref = ((af.float() @ wf.t().float()) * sa.view(-1, 1) * sb.view(1, -1)).to(torch.bfloat16) + bias
+    torch.testing.assert_close(out.float(), ref.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_block_quant_weight_roundtrip():
+    w = O.gen_weight(200, 300, seed=1)
+    q, s = O.block_quant_weight(w)
+    assert tuple(q.shape) == (200, 300) and tuple(s.shape) == (2, 3)
+    deq = q.float() * s.repeat_interleave(128, 0)[:200].repeat_interleave(128, 1)[:, :300]
+    assert float((deq - w).abs().max()) <= float(s.max()) * 16 + 1e-12  # within half an ulp at the top binade (32/2)
+    qt, st = O.per_tensor_quant_weight(w)
+    assert tuple(st.shape) == (200, 1) and float(qt.float().abs().max()) == 448.0
