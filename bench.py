@@ -1,0 +1,367 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 quantized-linear hot path on one MI355X.
+
+One step = one pass of the block-FP8 linear path (per-token-group FP8 quantization
+of the bf16 activations, then the block-scaled FP8 GEMM) over the five
+DeepSeek-V3 linear shapes at a prefill chunk of M = 4096, through the public
+operator API.  Inputs are synthetic and resident in HBM before timing starts.
+
+Prints ONE JSON line: whole-step block-FP8 GEMM throughput, the roofline of the
+dominant kernel (the GEMM, timed with events on the launch stream), the
+quantization kernel's HBM figure, and a CPU baseline (the torch restatement of
+the same path, timed on a bounded row sample on the host cores).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --sweep gpurun_out/sweep.jsonl     # every configuration, one line per shape
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+PEAK_FP8_TFLOPS = 5000.0    # dense FP8 MFMA, published (no sparsity)
+PEAK_INT8_TOPS = 5000.0
+
+DSV3_NK = [(24576, 1536), (32768, 512), (7168, 16384), (4096, 7168), (2112, 7168)]
+LLAMA8B_NK = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
+LLAMA70B_NK = [("qkv", 10240, 8192), ("o", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)]
+
+
+def group_quant_bytes(m, k):
+    return 2 * m * k + m * k + 4 * m * (k // 128)
+
+
+def token_quant_bytes(m, k):
+    return 3 * m * k + 4 * m
+
+
+def block_gemm_bytes(m, n, k):
+    kb, nb = (k + 127) // 128, (n + 127) // 128
+    return m * k + n * k + 4 * m * kb + 4 * nb * kb + 2 * m * n
+
+
+def rowcol_gemm_bytes(m, n, k, bias=False):
+    return m * k + n * k + 4 * m + 4 * n + 2 * m * n + (2 * n if bias else 0)
+
+
+def make_block_weight(n, k, seed, dev):
+    """N(0, 0.02) weights quantized per 128x128 block on the device (input data, not timed)."""
+    import torch
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    w = torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02
+    nb, kb = (n + 127) // 128, (k + 127) // 128
+    wp = torch.zeros((nb * 128, kb * 128), device=dev)
+    wp[:n, :k] = w
+    t = wp.view(nb, 128, kb, 128).permute(0, 2, 1, 3)
+    scale = t.abs().amax(dim=(2, 3)) / 448.0
+    scale = torch.where(scale == 0, torch.ones_like(scale), scale)
+    q = (t / scale[:, :, None, None]).clamp(-448, 448).permute(0, 2, 1, 3).reshape(nb * 128, kb * 128)[:n, :k]
+    return q.contiguous().to(torch.float8_e4m3fn), scale.contiguous()
+
+
+def make_activation(m, k, seed, dev):
+    import torch
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    return torch.randn((m, k), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+
+class Timer:
+    """Sums event-timed durations of individual launches on the current stream."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def time(self, fn):
+        import torch
+
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        out = fn()
+        e.record()
+        self.pairs.append((s, e))
+        return out
+
+    def total_ms(self):
+        return sum(s.elapsed_time(e) for s, e in self.pairs)
+
+    def count(self):
+        return len(self.pairs)
+
+
+def cpu_baseline(m_sample):
+    """The torch restatement of the same step on the host cores, on the first
+    m_sample activation rows of every shape (weights in full)."""
+    import torch
+
+    from oracle import w8a8_oracle as O
+
+    cores = torch.get_num_threads()
+    flops = 0.0
+    secs = 0.0
+    for i, (n, k) in enumerate(DSV3_NK):
+        x = O.gen_activation(m_sample, k, seed=2000 + i)
+        w = torch.randn((n, k), generator=torch.Generator().manual_seed(i)) * 0.02
+        wq, ws = O.block_quant_weight(w)
+        del w
+        t0 = time.perf_counter()
+        xq, xs = O.per_token_group_quant_fp8(x, 128)
+        O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+        secs += time.perf_counter() - t0
+        flops += 2.0 * m_sample * n * k
+    return {
+        "value": round(flops / secs / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {m_sample} of 4096 activation rows of each of the 5 shapes, full weights, {secs:.1f} s of CPU time",
+    }
+
+
+def run_headline(args):
+    import torch
+
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    m = 4096
+    layers = []
+    for i, (n, k) in enumerate(DSV3_NK):
+        wq, ws = make_block_weight(n, k, 2000 + i, dev)
+        layers.append((n, k, make_activation(m, k, 2000 + i, dev), wq, ws))
+    torch.cuda.synchronize()
+
+    def step(tq=None, tg=None):
+        for n, k, x, wq, ws in layers:
+            if tq is None:
+                xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+                fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+            else:
+                xq, xs = tq.time(lambda: sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True))
+                tg.time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # per-kernel durations on the launch stream (separate pass so the events do not perturb the wall clock above)
+    tq, tg = Timer(), Timer()
+    for _ in range(args.steps):
+        step(tq, tg)
+    torch.cuda.synchronize()
+
+    flops_step = sum(2.0 * m * n * k for n, k, *_ in layers)
+    qbytes_step = sum(group_quant_bytes(m, k) for _, k, *_ in layers)
+    ms_per_step = wall * 1e3 / args.steps
+    gemm_ms = tg.total_ms() / args.steps
+    quant_ms = tq.total_ms() / args.steps
+    gemm_tflops = flops_step / (gemm_ms * 1e-3) / 1e12
+    quant_gbs = qbytes_step / (quant_ms * 1e-3) / 1e9
+    props = torch.cuda.get_device_properties(dev)
+
+    out = {
+        "metric": "block-FP8 GEMM TFLOPS (% of FP8 MFMA peak); quant kernel GB/s (% of HBM)",
+        "value": round(flops_step / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn (fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {
+            "workload": "cfg2 DeepSeek-V3 block-FP8 linears, M=4096, (N,K) in "
+                        "{(24576,1536),(32768,512),(7168,16384),(4096,7168),(2112,7168)}: "
+                        "per-token-group-128 FP8 quant + 128x128 block-scaled FP8 GEMM, bf16 in/out",
+            "value_is": "sum of 2MNK over the 5 GEMMs / wall time of the whole step (quant kernels included)",
+        },
+        "roofline": {
+            "kernel": "fp8_blockwise_scaled_mm (gemm_kernel<FP8_BLOCK>)",
+            "bound": "mfma",
+            "achieved": round(gemm_tflops, 2),
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(gemm_tflops / PEAK_FP8_TFLOPS, 4),
+            "traffic": None,
+            "avg_launch_ms": round(gemm_ms / len(layers), 4),
+            "flops_per_launch_avg": flops_step / len(layers),
+        },
+        "quant": {
+            "kernel": "sgl_per_token_group_quant_fp8 (group_quant_kernel)",
+            "bound": "hbm",
+            "achieved": round(quant_gbs, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(quant_gbs / PEAK_HBM_GBS, 4),
+            "avg_launch_ms": round(quant_ms / len(layers), 4),
+            "bytes_per_launch_avg": qbytes_step / len(layers),
+        },
+        "device": {"name": props.name, "cus": props.multi_processor_count,
+                   "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_rows)
+    print(json.dumps(out), flush=True)
+
+
+# ---------------------------------------------------------------------------
+# --sweep: every configuration, one JSON line per (config, shape)
+# ---------------------------------------------------------------------------
+def time_kernel(fn, iters, rotate=1):
+    import torch
+
+    for i in range(3):
+        fn(i % rotate)
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for i in range(iters):
+        fn(i % rotate)
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def run_sweep(args):
+    import torch
+
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_quant_fp8
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_scaled_mm
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    out_path = Path(args.sweep)
+    out_path.parent.mkdir(parents=True, exist_ok=True)
+    f = open(out_path, "w")
+
+    def emit(**kw):
+        f.write(json.dumps(kw) + "\n")
+        f.flush()
+        print(json.dumps(kw), flush=True)
+
+    def rot_count(nbytes):  # rotate over enough copies to exceed the 256 MiB last-level cache
+        return max(1, min(8, int(600e6 // max(nbytes, 1))))
+
+    def block_case(cfg, name, m, n, k, seed):
+        wq, ws = make_block_weight(n, k, seed, dev)
+        r = rot_count(3 * m * k)
+        xs_in = [make_activation(m, k, seed + j, dev) for j in range(r)]
+        tq = time_kernel(lambda j: sglang_per_token_group_quant_fp8(xs_in[j], 128, column_major_scales=True), args.iters, r)
+        xq, xs = sglang_per_token_group_quant_fp8(xs_in[0], 128, column_major_scales=True)
+        rw = rot_count(n * k)
+        wqs = [wq] + [wq.clone() for _ in range(rw - 1)]
+        tg = time_kernel(lambda j: fp8_blockwise_scaled_mm(xq, wqs[j].t(), xs, ws.t(), torch.bfloat16), args.iters, rw)
+        fl = 2.0 * m * n * k
+        emit(cfg=cfg, op="group_quant_fp8+fp8_blockwise_scaled_mm", name=name, M=m, N=n, K=k,
+             quant_us=round(tq * 1e3, 2), quant_GBs=round(group_quant_bytes(m, k) / tq / 1e6, 1),
+             quant_frac_hbm=round(group_quant_bytes(m, k) / tq / 1e6 / PEAK_HBM_GBS, 4),
+             gemm_us=round(tg * 1e3, 2), gemm_TFLOPs=round(fl / tg / 1e9, 2),
+             gemm_frac_mfma=round(fl / tg / 1e9 / PEAK_FP8_TFLOPS, 4),
+             gemm_GBs=round(block_gemm_bytes(m, n, k) / tg / 1e6, 1),
+             gemm_frac_hbm=round(block_gemm_bytes(m, n, k) / tg / 1e6 / PEAK_HBM_GBS, 4))
+        return tq, tg
+
+    # cfg 0
+    block_case(0, "cfg0", 256, 2048, 7168, 0)
+    # cfg 1
+    g = torch.Generator(device=dev).manual_seed(1000)
+    n, k = 14336, 4096
+    w8 = torch.randint(-127, 128, (n, k), generator=g, device=dev, dtype=torch.int8)
+    s_b = torch.rand((n,), generator=g, device=dev) * 9e-3 + 1e-3
+    bias = (torch.randn((n,), generator=g, device=dev) * 0.1).to(torch.bfloat16)
+    w8s = [w8] + [w8.clone() for _ in range(7)]
+    for m in (1, 16, 128, 1024):
+        x = make_activation(m, k, 1000 + m, dev)
+        tq = time_kernel(lambda j: per_token_quant_int8(x), args.iters)
+        xq, xs = per_token_quant_int8(x)
+        tg = time_kernel(lambda j: int8_scaled_mm(xq, w8s[j].t(), xs, s_b, torch.bfloat16, bias), args.iters, 8)
+        fl = 2.0 * m * n * k
+        emit(cfg=1, op="per_token_quant_int8+int8_scaled_mm", M=m, N=n, K=k, quant_us=round(tq * 1e3, 2),
+             quant_GBs=round(token_quant_bytes(m, k) / tq / 1e6, 1), gemm_us=round(tg * 1e3, 2),
+             gemm_TOPs=round(fl / tg / 1e9, 2), gemm_frac_mfma=round(fl / tg / 1e9 / PEAK_INT8_TOPS, 4),
+             gemm_GBs=round(rowcol_gemm_bytes(m, n, k, True) / tg / 1e6, 1),
+             gemm_frac_hbm=round(rowcol_gemm_bytes(m, n, k, True) / tg / 1e6 / PEAK_HBM_GBS, 4))
+    del w8s
+    # cfg 2
+    for i, (n, k) in enumerate(DSV3_NK):
+        for m in (1, 8, 64, 512, 4096, 8192):
+            block_case(2, "dsv3", m, n, k, 2000 + i)
+    # cfg 3
+    for i, (n, k) in enumerate(LLAMA8B_NK):
+        g = torch.Generator(device=dev).manual_seed(3000 + i)
+        w = torch.randn((n, k), generator=g, device=dev) * 0.02
+        sc = w.abs().amax() / 448.0
+        wq = (w / sc).clamp(-448, 448).to(torch.float8_e4m3fn)
+        ws = sc.reshape(1, 1).expand(n, 1).contiguous()
+        rw = rot_count(n * k)
+        wqs = [wq] + [wq.clone() for _ in range(rw - 1)]
+        for m in (1, 32, 256, 2048):
+            x = make_activation(m, k, 3000 + m, dev)
+            tq = time_kernel(lambda j: sglang_per_token_quant_fp8(x), args.iters)
+            xq, xs = sglang_per_token_quant_fp8(x)
+            tg = time_kernel(lambda j: fp8_scaled_mm(xq, wqs[j].t(), xs, ws, torch.bfloat16, None), args.iters, rw)
+            fl = 2.0 * m * n * k
+            emit(cfg=3, op="per_token_quant_fp8+fp8_scaled_mm", M=m, N=n, K=k, quant_us=round(tq * 1e3, 2),
+                 quant_GBs=round(token_quant_bytes(m, k) / tq / 1e6, 1), gemm_us=round(tg * 1e3, 2),
+                 gemm_TFLOPs=round(fl / tg / 1e9, 2), gemm_frac_mfma=round(fl / tg / 1e9 / PEAK_FP8_TFLOPS, 4),
+                 gemm_GBs=round(rowcol_gemm_bytes(m, n, k) / tg / 1e6, 1),
+                 gemm_frac_hbm=round(rowcol_gemm_bytes(m, n, k) / tg / 1e6 / PEAK_HBM_GBS, 4))
+        del wqs
+    # cfg 4
+    for m in (4096, 64):
+        tot = 0.0
+        fl_tot = 0.0
+        for i, (name, n, k) in enumerate(LLAMA70B_NK):
+            tq, tg = block_case(4, name, m, n, k, 4000 + i)
+            tot += tq + tg
+            fl_tot += 2.0 * m * n * k
+            torch.cuda.empty_cache()
+        emit(cfg=4, op="total", M=m, total_us=round(tot * 1e3, 1), TFLOPs=round(fl_tot / tot / 1e9, 2))
+    f.close()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-rows", type=int, default=256, help="activation rows in the CPU-baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
+    ap.add_argument("--iters", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is measured on one GPU only (it needs no exchange between GPUs; "
+              "a tensor-parallel deployment shards N or K per rank and all-reduces outside it). Run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+    if args.sweep:
+        run_sweep(args)
+    else:
+        run_headline(args)
+
+
+if __name__ == "__main__":
+    main()

@@ -124,11 +124,23 @@ struct FastDiv {
   }
 };
 
+template <bool CLAMP>
+SGLQ_DEV float quantize_elem(float x, float y_s, float r, float qmin, float qmax) {
+  float q = div_by(x, y_s, r);
+  if constexpr (CLAMP) q = clampf(q, qmin, qmax);
+  return __builtin_copysignf(q, x);
+}
+
 // ---------------------------------------------------------------------------
 // Per-token-group quantization.  16 elements per lane as two 8-element chunks
 // half a group apart, so every load instruction reads fully used 128-byte runs.
 // ---------------------------------------------------------------------------
-template <int DT, int GROUP, int UNROLL, bool STRIDED_SCALE, bool TO_INT8>
+//
+// CLAMP = false is the standard e4m3fn case (bounds -448/+448): |x| <= amax bounds
+// the quotient by 448 * (1 + 2^-22), which rounds to the code of 448 anyway, so
+// the explicit clamp is dropped.  The quotient's sign is copied from x so that
+// -0.0 stays -0.0 (the remainder correction would turn it into +0.0).
+template <int DT, int GROUP, int UNROLL, bool STRIDED_SCALE, bool TO_INT8, bool CLAMP>
 __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
                                                           float* __restrict__ s, uint32_t num_groups,
                                                           FastDiv groups_per_row, int64_t s_stride_row,
@@ -163,12 +175,12 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict
       float v[8];
       v2u o;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = clampf(div_by(lo[u].get(i), y_s, r), qmin, qmax);
+      for (int i = 0; i < 8; ++i) v[i] = quantize_elem<CLAMP>(lo[u].get(i), y_s, r, qmin, qmax);
       if constexpr (TO_INT8) o = I8Pack::pack(v); else o = Fp8Pack::pack(v);
       char* qp = q + (int64_t)gid * GROUP + sub * 8;
       *reinterpret_cast<v2u*>(qp) = o;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = clampf(div_by(hi[u].get(i), y_s, r), qmin, qmax);
+      for (int i = 0; i < 8; ++i) v[i] = quantize_elem<CLAMP>(hi[u].get(i), y_s, r, qmin, qmax);
       if constexpr (TO_INT8) o = I8Pack::pack(v); else o = Fp8Pack::pack(v);
       *reinterpret_cast<v2u*>(qp + GROUP / 2) = o;
       if (sub == 0) {
@@ -358,7 +370,7 @@ static int check_launch(const char* what) {
   return SGLQ_OK;
 }
 
-template <int DT, int GROUP, bool TO_INT8>
+template <int DT, int GROUP, bool TO_INT8, bool CLAMP>
 static void launch_group_quant(const void* x, void* q, float* s, uint32_t num_groups, uint32_t gpr, bool strided,
                                int64_t sr, int64_t sc, float eps, float qmin, float qmax, hipStream_t st) {
   constexpr int GPB = 256 / (GROUP / 16);
@@ -370,7 +382,7 @@ static void launch_group_quant(const void* x, void* q, float* s, uint32_t num_gr
   const char* xi = static_cast<const char*>(x);
   char* qo = static_cast<char*>(q);
 #define SGLQ_LAUNCH_GQ(U, STR)                                                                              \
-  group_quant_kernel<DT, GROUP, U, STR, TO_INT8><<<dim3((num_groups + GPB * U - 1) / (GPB * U)), dim3(256), 0, st>>>( \
+  group_quant_kernel<DT, GROUP, U, STR, TO_INT8, CLAMP><<<dim3((num_groups + GPB * U - 1) / (GPB * U)), dim3(256), 0, st>>>( \
       xi, qo, s, num_groups, fd, sr, sc, eps, qmin, qmax, rq)
   if (deep) {
     if (strided) SGLQ_LAUNCH_GQ(2, true); else SGLQ_LAUNCH_GQ(2, false);
@@ -409,11 +421,16 @@ static int group_quant_entry(const char* name, const void* input, int in_dtype, 
     return SGLQ_EINVAL;
   }
   const bool strided = !(sc == 1 && sr == gpr);
+  const bool standard = !TO_INT8 && qmin == -448.0f && qmax == 448.0f;
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define SGLQ_GQ_CASE(DT, G)                                                                                   \
   if (in_dtype == DT && group_size == G) {                                                                    \
-    launch_group_quant<DT, G, TO_INT8>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, sc, \
-                                       eps, qmin, qmax, st);                                                  \
+    if (standard)                                                                                             \
+      launch_group_quant<DT, G, TO_INT8, false>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, \
+                                                sc, eps, qmin, qmax, st);                                     \
+    else                                                                                                      \
+      launch_group_quant<DT, G, TO_INT8, true>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, \
+                                               sc, eps, qmin, qmax, st);                                      \
     return check_launch(name);                                                                                \
   }
 #define SGLQ_GQ_DT(DT) SGLQ_GQ_CASE(DT, 128) SGLQ_GQ_CASE(DT, 64) SGLQ_GQ_CASE(DT, 32) SGLQ_GQ_CASE(DT, 16)

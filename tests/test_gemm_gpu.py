@@ -1,0 +1,185 @@
+"""GPU parity of the three GEMMs against the CPU oracle: INT32 accumulators
+bit-exact, bf16/fp16 outputs within rtol 1e-2 / atol 1e-2 (the tolerance the
+path's contract states for floating-point outputs)."""
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+RTOL, ATOL = 1e-2, 1e-2
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def rand_i8(shape, seed, lo=-128, hi=128):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi, shape, generator=g, dtype=torch.int8)
+
+
+def sample_rows(m, cap=48):
+    if m <= cap:
+        return torch.arange(m)
+    g = torch.Generator().manual_seed(m)
+    idx = torch.randperm(m, generator=g)[: cap - 4]
+    return torch.cat([idx, torch.tensor([0, 1, m - 2, m - 1])]).unique()
+
+
+@pytest.fixture(params=[1, 0], ids=["direct_lds", "via_regs"])
+def load_path(request):
+    from sglang_amd import _lib
+
+    _lib.load().sglq_debug_set_direct_lds(request.param)
+    yield request.param
+    _lib.load().sglq_debug_set_direct_lds(1)
+
+
+@pytest.mark.parametrize("mnk", [(1, 128, 64), (5, 136, 128), (16, 8, 16), (33, 264, 208), (127, 256, 4096), (128, 1024, 512),
+                                 (130, 640, 1040), (512, 14336, 4096)])
+def test_int8_accumulators_bit_exact(gpu, load_path, mnk):
+    from sglang_amd.sgl_kernel import int8_mm_i32
+
+    say("int8 acc", mnk, "direct" if load_path else "regs")
+    m, n, k = mnk
+    a, w = rand_i8((m, k), 1), rand_i8((n, k), 2)
+    if m > 2:
+        a[1] = -128
+        w[0] = -128  # extreme products
+    rows = sample_rows(m)
+    ref = O.int8_mm_i32(a[rows], w.t())
+    got = int8_mm_i32(a.to(gpu), w.to(gpu).t()).cpu()
+    assert tuple(got.shape) == (m, n)
+    bad = got[rows] != ref
+    assert not bool(bad.any()), f"{int(bad.sum())} accumulators differ, first {bad.nonzero()[:4].tolist()}"
+
+
+@pytest.mark.parametrize("m", [1, 16, 128, 1024])
+def test_int8_scaled_mm_config(gpu, m):
+    """A[M,4096] per-token INT8 x B[4096,14336] with per-column scales and bf16 bias."""
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+    from sglang_amd.sgl_kernel import int8_mm_i32, int8_scaled_mm
+
+    say("int8_scaled_mm config M", m)
+    x = O.gen_activation(m, 4096, seed=1000 + m)
+    wt, s_b, bias = O.gen_int8_weight(4096, 14336, seed=1000)
+    xq_ref, xs_ref = O.per_token_quant_int8(x)
+    xq, xs = per_token_quant_int8(x.to(gpu))
+    assert torch.equal(xq.cpu(), xq_ref) and torch.equal(xs.cpu(), xs_ref)
+    wg = wt.t().contiguous().to(gpu).t()  # [K, N] view with stride(0) == 1
+    rows = sample_rows(m, 24)
+    acc = int8_mm_i32(xq, wg).cpu()
+    assert torch.equal(acc[rows], O.int8_mm_i32(xq_ref[rows], wt))
+    for b in (None, bias):
+        out = int8_scaled_mm(xq, wg, xs, s_b.to(gpu), torch.bfloat16, None if b is None else b.to(gpu)).cpu()
+        ref = O.int8_scaled_mm(xq_ref[rows], wt, xs_ref[rows], s_b, torch.bfloat16, b)
+        torch.testing.assert_close(out[rows].float(), ref.float(), rtol=RTOL, atol=ATOL)
+
+
+def make_block_case(m, n, k, seed, outliers=False):
+    x = O.gen_activation(m, k, seed=seed, outliers=outliers)
+    w = O.gen_weight(n, k, seed=seed)
+    wq, ws = O.block_quant_weight(w)
+    xq, xs = O.per_token_group_quant_fp8(x, 128) if k % 128 == 0 else (None, None)
+    return x, xq, xs, wq, ws
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (3, 256, 512), (5, 2112, 1536), (127, 512, 7168), (128, 4096, 512),
+                                 (256, 2048, 7168), (512, 1536, 1024), (1024, 640, 2048)])
+def test_fp8_blockwise_scaled_mm(gpu, load_path, mnk, out_dtype):
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("fp8_blockwise", mnk, out_dtype, "direct" if load_path else "regs")
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = sample_rows(m)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()  # [M, K/128], stride(0) == 1
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), out_dtype)
+    assert out.dtype == out_dtype and tuple(out.shape) == (m, n)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_fp8_blockwise_unit_scales_is_plain_matmul(gpu):
+    """All scales 1 and small integer-valued operands: every partial sum is an
+    integer below 2^24, so the result is exact whatever the summation order."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("fp8_blockwise exact integers")
+    g = torch.Generator().manual_seed(5)
+    m, n, k = 77, 384, 1024
+    a = torch.randint(-4, 5, (m, k), generator=g).float().to(FP8)
+    w = torch.randint(-4, 5, (n, k), generator=g).float().to(FP8)
+    ref = (a.double() @ w.double().t())
+    assert float(ref.abs().max()) < 2**24  # exact in the fp32 accumulator
+    sa = torch.ones((k // 128, m)).t().to(gpu)
+    sb = torch.ones((n // 128, k // 128)).to(gpu).t()
+    out = fp8_blockwise_scaled_mm(a.to(gpu), w.to(gpu).t(), sa, sb, torch.bfloat16).cpu()
+    assert torch.equal(out.double(), ref.to(torch.bfloat16).double())
+
+
+def test_fp8_blockwise_row_major_scales_vector(gpu):
+    """K = 128: scales_a is a contiguous [M, 1] vector, which the reference accepts
+    as well as an M-major matrix."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    m, n, k = 9, 256, 128
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=77)
+    ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs.to(gpu), ws.to(gpu).t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("mnk", [(1, 4096, 4096), (32, 6144, 4096), (256, 4096, 14336), (2048, 1024, 4096), (7, 16, 32), (100, 264, 1040)])
+def test_fp8_scaled_mm(gpu, mnk, with_bias):
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    say("fp8_scaled_mm", mnk, with_bias)
+    m, n, k = mnk
+    x = O.gen_activation(m, k, seed=3000 + m)
+    w = O.gen_weight(n, k, seed=3000 + n)
+    xq, xs = O.per_token_quant_fp8(x)
+    wq, ws = O.per_tensor_quant_weight(w)
+    g = torch.Generator().manual_seed(m)
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16) if with_bias else None
+    rows = sample_rows(m)
+    ref = O.fp8_scaled_mm(xq[rows], wq.t(), xs[rows], ws, torch.float32, bias, acc_dtype=torch.float64)
+    out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs.to(gpu), ws.to(gpu), torch.bfloat16,
+                        None if bias is None else bias.to(gpu))
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_gemm_linearity_at_full_size(gpu):
+    """Full-size DeepSeek-V3 shape (M=4096, N=7168, K=16384): doubling the
+    activation scales doubles the output exactly (power-of-two scaling commutes
+    with every rounding), and a row sample matches the oracle."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("fp8_blockwise full size")
+    m, n, k = 4096, 7168, 16384
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((m, k), generator=g, device=gpu).to(torch.bfloat16)
+    w = O.gen_weight(n, k, seed=2)
+    wq, ws = O.block_quant_weight(w)
+    xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    wqg, wsg = wq.to(gpu), ws.to(gpu)
+    out = fp8_blockwise_scaled_mm(xq, wqg.t(), xs, wsg.t(), torch.bfloat16)
+    out2 = fp8_blockwise_scaled_mm(xq, wqg.t(), (xs * 2.0).t().contiguous().t(), wsg.t(), torch.bfloat16)
+    assert torch.equal(out2.float(), out.float() * 2.0)
+    rows = sample_rows(m, 12)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows.to(gpu)].cpu(), wq.t(), xs[rows.to(gpu)].cpu(), ws.t(), torch.float32)
+    torch.testing.assert_close(out[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_gemm_empty_m(gpu):
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, int8_scaled_mm
+
+    a = torch.empty((0, 128), dtype=torch.int8, device=gpu)
+    w = torch.zeros((16, 128), dtype=torch.int8, device=gpu)
+    out = int8_scaled_mm(a, w.t(), torch.empty((0, 1), device=gpu), torch.ones((16, 1), device=gpu), torch.bfloat16)
+    assert tuple(out.shape) == (0, 16)

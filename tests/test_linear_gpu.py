@@ -1,0 +1,53 @@
+"""End-to-end glue (quantize -> GEMM -> bias) against the oracle's same sequence."""
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_block_fp8_linear_config0(gpu):
+    """A[256,7168] with 1% x20 outliers, W[2048,7168] block-quantized, bias added by the caller."""
+    from sglang_amd.quantization.fp8_utils import w8a8_block_fp8_linear
+
+    print("block fp8 linear cfg0", flush=True)
+    x = O.gen_activation(256, 7168, seed=0, outliers=True)
+    wq, ws = O.block_quant_weight(O.gen_weight(2048, 7168, seed=0))
+    bias = (torch.randn(2048, generator=torch.Generator().manual_seed(1)) * 0.1).to(torch.bfloat16)
+    xq, xs = O.per_token_group_quant_fp8(x, 128)
+    mm = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32)
+    ref = mm + bias.float()
+    out = w8a8_block_fp8_linear(x.to(gpu).view(2, 128, 7168), wq.to(gpu), [128, 128], ws.to(gpu), bias=bias.to(gpu))
+    assert tuple(out.shape) == (2, 128, 2048) and out.dtype == torch.bfloat16
+    # the caller rounds the GEMM output to bf16 before adding the bias (fp8_utils.py:207-211):
+    # allow one bf16 ulp of that intermediate on top of the path's rtol/atol of 1e-2
+    tol = 1e-2 + 1e-2 * ref.abs() + mm.abs() * 2.0**-8
+    err = (out.cpu().view(256, 2048).float() - ref).abs()
+    assert bool((err <= tol).all()), f"max excess {(err - tol).max().item()}"
+
+
+def test_int8_linear(gpu):
+    from sglang_amd.quantization.w8a8_int8 import apply_w8a8_int8_linear, process_weights_after_loading
+
+    print("int8 linear", flush=True)
+    x = O.gen_activation(16, 4096, seed=1001)
+    wt, s_b, bias = O.gen_int8_weight(4096, 14336, seed=1000)
+    xq, xs = O.per_token_quant_int8(x)
+    ref = O.int8_scaled_mm(xq, wt, xs, s_b, torch.bfloat16, bias)
+    w_stored = wt.t().contiguous().to(gpu)  # [N, K] as loaded
+    w_view, w_scale = process_weights_after_loading(w_stored, s_b.reshape(-1, 1).to(gpu))
+    out = apply_w8a8_int8_linear(x.to(gpu), w_view, w_scale, bias.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_fp8_per_channel_linear(gpu):
+    from sglang_amd.quantization.fp8_utils import apply_fp8_linear
+
+    print("fp8 linear", flush=True)
+    x = O.gen_activation(32, 4096, seed=3001)
+    wq, ws = O.per_tensor_quant_weight(O.gen_weight(6144, 4096, seed=3000))
+    xq, xs = O.per_token_quant_fp8(x)
+    ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16)
+    out = apply_fp8_linear(x.to(gpu), wq.to(gpu).t(), ws.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)

@@ -1,0 +1,206 @@
+"""GPU parity of the quantization kernels against the CPU oracle: FP8 codes, INT8
+codes and fp32 scales must be bit-identical.  Everything goes through the
+operator wrappers, i.e. through the C ABI of libsglq.so."""
+import pytest
+import torch
+
+from helpers import assert_bits_equal, fp8_bits
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def group_quant_gpu(x, group, column_major=False, tma=False, eps=1e-10):
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    return sglang_per_token_group_quant_fp8(x, group, eps=eps, column_major_scales=column_major, scale_tma_aligned=tma)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 128), (3, 256), (127, 512), (256, 7168), (1000, 1536), (33, 16384)])
+def test_group_quant_fp8_bit_exact(gpu, dtype, shape):
+    say("group_quant", dtype, shape)
+    m, k = shape
+    x = O.gen_activation(m, k, seed=m * 7 + k, outliers=True).float()
+    if m > 2:
+        x[1, :128] = 0
+        x[2] *= 1e-5
+        x[0, 1:9] = torch.tensor([-0.0, 0.0, -0.0, -1e-30, 1e-30, -0.0, 0.0, -0.0])  # signed zeros survive
+    x = x.to(dtype)
+    q_ref, s_ref = O.per_token_group_quant_fp8(x, 128)
+    for cm, tma in ((False, False), (True, False), (True, True)):
+        q, s = group_quant_gpu(x.to(gpu), 128, cm, tma)
+        torch.cuda.synchronize()
+        if cm:
+            assert s.stride(0) == 1
+        assert_bits_equal(s, s_ref, f"scales cm={cm} tma={tma}")
+        assert_bits_equal(q, q_ref, f"codes cm={cm} tma={tma}")
+
+
+@pytest.mark.parametrize("group", [16, 32, 64, 128])
+def test_group_quant_fp8_group_sizes(gpu, group):
+    say("group_quant group", group)
+    x = O.gen_activation(129, 1024, seed=group, outliers=True)
+    q_ref, s_ref = O.per_token_group_quant_fp8(x, group)
+    q, s = group_quant_gpu(x.to(gpu), group)
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+    q, s = group_quant_gpu(x.to(gpu), group, column_major=True)
+    assert_bits_equal(s, s_ref, "scales (column-major)")
+
+
+def test_group_quant_fp8_every_code_and_tie(gpu):
+    """fp32 groups whose scale is exactly 1 (absmax 448): every e4m3fn value, every
+    midpoint between neighbours and the floats next to each midpoint."""
+    say("group_quant conversions")
+    codes = torch.arange(256, dtype=torch.uint8)
+    vals = O.e4m3fn_decode(codes)
+    pos = torch.sort(vals[(~torch.isnan(vals)) & (vals >= 0)]).values.unique()
+    mids = ((pos[:-1].double() + pos[1:].double()) / 2).float()
+    cand = torch.cat([pos, mids, torch.nextafter(mids, torch.tensor(0.0)), torch.nextafter(mids, torch.tensor(1e9))])
+    cand = torch.cat([cand, -cand])
+    n = (cand.numel() + 126) // 127
+    x = torch.zeros(n, 128)
+    x[:, 0] = 448.0
+    flat = torch.zeros(n * 127)
+    flat[: cand.numel()] = cand
+    x[:, 1:] = flat.reshape(n, 127)
+    q_ref, s_ref = O.per_token_group_quant_fp8(x, 128)
+    assert float(s_ref.min()) == 1.0 and float(s_ref.max()) == 1.0
+    q, s = group_quant_gpu(x.to(gpu), 128)
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+
+
+def test_group_quant_fp8_custom_bounds(gpu):
+    """Bounds other than +-448 take the clamping variant of the kernel."""
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8
+
+    say("group_quant custom bounds")
+    x = O.gen_activation(65, 512, seed=12, outliers=True)
+    x[0, 3] = -0.0
+    for lo, hi in ((-224.0, 224.0), (-448.0, 240.0)):
+        q_ref, s_ref = O.per_token_group_quant_8bit(x, 128, 1e-10, lo, hi, FP8)
+        xg = x.to(gpu)
+        q = torch.empty_like(xg, dtype=FP8)
+        s = torch.empty((65, 4), dtype=torch.float32, device=gpu)
+        sgl_per_token_group_quant_fp8(xg, q, s, 128, 1e-10, lo, hi, False)
+        assert_bits_equal(s, s_ref, f"scales {lo},{hi}")
+        assert_bits_equal(q, q_ref, f"codes {lo},{hi}")
+
+
+def test_group_quant_int8_bit_exact(gpu):
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_int8
+
+    say("group_quant int8")
+    x = O.gen_activation(77, 1024, seed=3, outliers=True)
+    q_ref, s_ref = O.per_token_group_quant_8bit(x, 128, 1e-10, -128.0, 127.0, torch.int8)
+    xg = x.to(gpu)
+    q = torch.empty_like(xg, dtype=torch.int8)
+    s = torch.empty((77, 8), dtype=torch.float32, device=gpu)
+    sgl_per_token_group_quant_int8(xg, q, s, 128, 1e-10, -128.0, 127.0)
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 4096), (16, 4096), (128, 4096), (1024, 4096), (5, 1000), (7, 1003), (3, 14336),
+                                   (2, 20000), (9, 512), (300, 256), (4, 8)])
+def test_token_quant_int8_bit_exact(gpu, dtype, shape):
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+
+    say("token_quant_int8", dtype, shape)
+    m, k = shape
+    x = O.gen_activation(m, k, seed=m + k).float()
+    if m > 2:
+        x[1] = 0
+        x[2, 0] = 0.5 * x[2].abs().max()  # an exact .5 product when absmax/127 is a power of two is rare; force ties below
+    x = x.to(dtype)
+    q_ref, s_ref = O.per_token_quant_int8(x)
+    q, s = per_token_quant_int8(x.to(gpu))
+    assert tuple(s.shape) == (m, 1)
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+
+
+def test_token_quant_int8_ties_round_away(gpu):
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+
+    say("token_quant_int8 ties")
+    k = torch.arange(-127, 128, dtype=torch.float32)
+    row = torch.cat([k, k[:-1] + 0.5, torch.zeros(6)]).reshape(1, -1)  # 255 + 254 + 6 = 515 -> pad to 520
+    row = torch.cat([row, torch.zeros(1, 5)], dim=1)
+    q_ref, s_ref = O.per_token_quant_int8(row)
+    assert s_ref.item() == 1.0
+    q, s = per_token_quant_int8(row.to(gpu))
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+    assert q[0, 255:259].tolist() == [-127, -126, -125, -124]  # -126.5 -> -127 ...
+
+
+def test_token_quant_int8_row_sum(gpu):
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+
+    x = O.gen_activation(33, 4096, seed=9)
+    q, s, rs = per_token_quant_int8(x.to(gpu), cal_sum=True)
+    # summation order is not defined by the reference (a Triton reduction): tolerance only
+    torch.testing.assert_close(rs.float().cpu(), x.float().sum(-1), rtol=2e-2, atol=0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 4096), (32, 4096), (256, 14336), (2048, 4096), (5, 1368), (130, 512), (3, 24576), (2, 8)])
+def test_token_quant_fp8_bit_exact(gpu, dtype, shape):
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_quant_fp8
+
+    say("token_quant_fp8", dtype, shape)
+    m, k = shape
+    x = O.gen_activation(m, k, seed=3 * m + k).float()
+    if m > 1:
+        x[1] = 0  # zero row: scale 0, codes 0
+    x = x.to(dtype)
+    q_ref, s_ref = O.per_token_quant_fp8(x)
+    q, s = sglang_per_token_quant_fp8(x.to(gpu))
+    assert tuple(s.shape) == (m, 1)
+    assert_bits_equal(s, s_ref, "scales")
+    assert_bits_equal(q, q_ref, "codes")
+
+
+def test_quant_empty_inputs(gpu):
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_quant_fp8
+    from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+
+    x = torch.empty((0, 256), dtype=torch.bfloat16, device=gpu)
+    q, s = sglang_per_token_group_quant_fp8(x, 128)
+    assert tuple(q.shape) == (0, 256) and tuple(s.shape) == (0, 2)
+    q, s = per_token_quant_int8(x)
+    assert tuple(q.shape) == (0, 256) and tuple(s.shape) == (0, 1)
+    q, s = sglang_per_token_quant_fp8(x)
+    assert tuple(q.shape) == (0, 256)
+
+
+def test_group_quant_full_size_properties(gpu):
+    """Largest configuration (8192 x 16384): idempotence of the codes under
+    re-quantization of the dequantized tensor, max code 448 in every group, and
+    bit-exactness on a row sample."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    say("group_quant full size")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((8192, 16384), generator=g, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+    q, s = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    qa = q.view(8192, 128, 128).float().abs().amax(dim=2)
+    assert bool((qa == 448.0).all())
+    rows = torch.tensor([0, 1, 17, 4095, 4096, 8191])
+    q_ref, s_ref = O.per_token_group_quant_fp8(x[rows.to(gpu)].cpu(), 128)
+    assert_bits_equal(q[rows.to(gpu)], q_ref, "codes (row sample)")
+    assert_bits_equal(s[rows.to(gpu)].contiguous(), s_ref, "scales (row sample)")
+    # dequantize (exactly representable in fp32) and quantize again: same codes, same scales
+    deq = (q.view(8192, 128, 128).float() * s.contiguous().view(8192, 128, 1)).view(8192, 16384)
+    q2, s2 = sglang_per_token_group_quant_fp8(deq, 128, column_major_scales=True)
+    assert bool((s2 == s).all())
+    assert bool((q2.view(torch.uint8) == q.view(torch.uint8)).all())
