@@ -110,6 +110,9 @@ int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, c
  * copy global memory straight into LDS with buffer loads, zero stages the same
  * bytes through registers.  Both must give identical results. */
 void sglq_debug_set_direct_lds(int on);
+/* Test hook: 0 = choose the GEMM tile by shape (default), 128 / 256 = always use
+ * the 128x128 / 256x256 kernel. */
+void sglq_debug_force_tile(int tile);
 
 #ifdef __cplusplus
 }

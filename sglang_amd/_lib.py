@@ -55,6 +55,8 @@ def load() -> ctypes.CDLL:
     lib.sglq_abi_version.argtypes = []
     lib.sglq_debug_set_direct_lds.argtypes = [c_int]
     lib.sglq_debug_set_direct_lds.restype = None
+    lib.sglq_debug_force_tile.argtypes = [c_int]
+    lib.sglq_debug_force_tile.restype = None
     _lib = lib
     return lib
 

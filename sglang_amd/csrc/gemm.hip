@@ -95,6 +95,40 @@ SGLQ_DEV void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn)
   tn = in_group / gsz;
 }
 
+// Scale, add bias and store a wave's accumulators.  acc[i][j][e] belongs to
+// C[m_base + 16 i + r16][n_base + 16 j + 4 g + e].
+template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
+SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int n_base, int r16, int g) {
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m_base + i * 16 + r16;
+    if (m >= p.M) continue;
+    float sam = 1.f;
+    if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = p.sa[m];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n_base + j * 16 + g * 4;
+      if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
+      const int64_t idx = (int64_t)m * p.ldo + n;
+      if constexpr (KIND == KIND_I8_RAW) {
+        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = acc[i][j];
+      } else if constexpr (KIND == KIND_FP8_BLOCK) {
+        store4<OUT_DT>(p.out, idx, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      } else {
+        float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
+        const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
+        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbn[e] * sam, bv[e]);
+          else o[e] = __builtin_fmaf(sam, sbn[e] * acc[i][j][e], bv[e]);
+        }
+        store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
+      }
+    }
+  }
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT, bool DMA>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const GemmArgs p) {
   constexpr int NW = WAVES_M * WAVES_N;
@@ -246,35 +280,202 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     }
   }
 
-  // ---- epilogue
+  epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+}
+
+// ---------------------------------------------------------------------------
+// Prefill kernel: 256 x 256 output tile, 8 wavefronts (2 per SIMD), each owning
+// 128 (m) x 64 (n).  One K step (128 bytes) is 2 x 32 MFMAs x 32 cycles = 2048
+// MFMA-pipe cycles per SIMD, about a microsecond, which is what hides the
+// latency of the next stage's global -> LDS copies with only two 64 KiB stages.
+// A wave keeps its four weight fragments of the step in registers and streams
+// the eight activation fragments through a two-deep register queue, so each LDS
+// byte is read once per wave and the 128 accumulator registers leave room for
+// two waves per SIMD.
+// ---------------------------------------------------------------------------
+template <int KIND, int OUT_DT>
+__global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
+  constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
+  constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
+  constexpr int STAGE_BYTES = (BM + BN) * 128;
+  constexpr int NLOAD = (BM + BN) / 8 / NW;  // 8 one-KiB copies per wave per stage: 4 of A, 4 of B
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
+
+  // Copy j of this wave fills stage rows 8 (wave + 8 j) .. + 7; lane l brings row
+  // l / 8 of those, chunk (l % 8) ^ swz(row).  swz depends on l / 8 and the parity
+  // of the wave only, so all four A copies (and all four B copies) share one
+  // per-lane offset and differ by a multiple of 64 rows.  Rows past M / N fall
+  // beyond the buffer's extent and read as zero; the K offset travels in the
+  // scalar operand (K is a multiple of 128 for this kernel).
+  const int l8 = lane >> 3;
+  const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
+  const uint32_t off_a = (uint32_t)(m0 + wave * 8 + l8) * p.lda + c16;
+  const uint32_t off_b = (uint32_t)(n0 + wave * 8 + l8) * p.ldb + c16;
+  const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
+  auto issue_load = [&](int j, int stage, int k0) {
+    const bool is_a = j < NLOAD / 2;
+    const int i = wave + j * NW;
+    char* dst = smem + stage * STAGE_BYTES + i * 1024;
+    const uint32_t off = is_a ? off_a + (uint32_t)j * step_a : off_b + (uint32_t)(j - NLOAD / 2) * step_b;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(is_a ? ra : rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0,
+                                             0, 0);
+  };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  const int a_base = (wm * TM) * 128;
+  const int b_base = (BM + wn * TN) * 128;
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * TM + i * 16 + r16;
-    if (m >= p.M) continue;
-    float sam = 1.f;
-    if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = p.sa[m];
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      const int n = n0 + wn * TN + j * 16 + g * 4;
-      if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
-      const int64_t idx = (int64_t)m * p.ldo + n;
-      if constexpr (KIND == KIND_I8_RAW) {
-        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = acc[i][j];
-      } else if constexpr (KIND == KIND_FP8_BLOCK) {
-        store4<OUT_DT>(p.out, idx, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-      } else {
-        float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
-        const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
-        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv);
+    for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+  // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].
+  // A lane owns row r16 of each of the wave's 16-row fragments; rows past M read
+  // as zero through the buffer's extent (they are never stored).
+  const int nkb = p.K >> 7;
+  float sfa_cur[MI];
+  float sfb_cur = 0.f;
+  __amdgpu_buffer_rsrc_t rs = ra;
+  uint32_t sfa_off = 0;
+  int sfa_frag = 0, sfa_step = 0, nb = 0;
+  if constexpr (KIND == KIND_FP8_BLOCK) {
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    const int nblocks = (p.N + 127) >> 7;
+    nb = (n0 + wn * TN) >> 7;
+    if (nb >= nblocks) nb = nblocks - 1;
+    const int mrow = m0 + wm * TM + r16;
+    // a row past M must not alias a valid element of another K block: send it out of range
+    sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
+    sfa_frag = (int)(16 * p.sa_stride_m * 4);
+    sfa_step = (int)(p.sa_stride_k * 4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbn[e] * sam, bv[e]);
-          else o[e] = __builtin_fmaf(sam, sbn[e] * acc[i][j][e], bv[e]);
+    for (int i = 0; i < MI; ++i) {
+      const bool ok = mrow + i * 16 < p.M;
+      sfa_cur[i] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok ? sfa_off + i * sfa_frag : OOB, 0, 0));
+    }
+    sfb_cur = p.sb[nb * p.sb_stride_n];
+  }
+  // validity of fragment i's row for the scale prefetch, as a bit mask
+  uint32_t sfa_ok = 0;
+  if constexpr (KIND == KIND_FP8_BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_ok |= (m0 + wm * TM + r16 + i * 16 < p.M ? 1u : 0u) << i;
+  }
+
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+#pragma unroll
+  for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
+
+  // One K step.  more_tag = another step follows: its copies and scales are issued here,
+  // in the shadow of the MFMAs, so that no wave spends issue slots on them while the
+  // MFMA pipe is idle.
+  auto k_step = [&](int kb, auto more_tag) {
+    constexpr bool more = decltype(more_tag)::value;
+    const int cur = kb & 1;
+    __builtin_amdgcn_s_waitcnt(0);  // this stage has landed (copies were issued one K step ago)
+    __syncthreads();                // ... for every wave, and nobody still reads the other stage
+
+    const char* st = smem + cur * STAGE_BYTES;
+    v8i bf[NI];
+    bf[0] = read_frag(st + b_base);
+    v8i a_cur = read_frag(st + a_base);
+#pragma unroll
+    for (int j = 1; j < NI; ++j) bf[j] = read_frag(st + b_base + j * 16 * 128);
+    float sc = 0.f, sc_prev = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4f part_prev = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      v8i a_nxt = a_cur;
+      if constexpr (KIND == KIND_FP8_BLOCK) {
+        sc_prev = sc;
+        sc = sfa_cur[i] * sfb_cur;
+      }
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const int idx = i * NI + j;
+        if constexpr (KIND == KIND_FP8_BLOCK) {
+          const v4f z = {0.f, 0.f, 0.f, 0.f};
+          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, z, 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
+          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+          if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
+            const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
+            const float s_use = (pi == i) ? sc : sc_prev;
+            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], s_use, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], s_use, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
+          }
+          // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
+          if (more && j == 1 && i >= 1)
+            sfa_cur[i - 1] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rs, ((sfa_ok >> (i - 1)) & 1) ? sfa_off + (i - 1) * sfa_frag : OOB,
+                                                            (kb + 1) * sfa_step, 0));
+          part_prev = part;
+        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, acc[i][j], 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
+          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+        } else {
+          const v4i b0 = {bf[j][0], bf[j][1], bf[j][2], bf[j][3]}, b1 = {bf[j][4], bf[j][5], bf[j][6], bf[j][7]};
+          const v4i a0 = {a_cur[0], a_cur[1], a_cur[2], a_cur[3]}, a1 = {a_cur[4], a_cur[5], a_cur[6], a_cur[7]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
+          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
         }
-        store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      a_cur = a_nxt;
+    }
+    if constexpr (KIND == KIND_FP8_BLOCK) {
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+      if constexpr (more) {
+        sfa_cur[MI - 1] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(rs, ((sfa_ok >> (MI - 1)) & 1) ? sfa_off + (MI - 1) * sfa_frag : OOB,
+                                                        (kb + 1) * sfa_step, 0));
+        sfb_cur = p.sb[(kb + 1) * p.sb_stride_k + nb * p.sb_stride_n];
       }
     }
-  }
+  };
+  for (int kb = 0; kb + 1 < nkb; ++kb) k_step(kb, std::true_type{});
+  k_step(nkb - 1, std::false_type{});
+
+  epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
 }
 
 // ---------------------------------------------------------------------------
@@ -291,8 +492,21 @@ static void launch_cfg(GemmArgs& p, hipStream_t st) {
   else gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, false><<<grid, block, 0, st>>>(p);
 }
 
+static int g_force_tile = 0;  // test hook: 0 = heuristic, 128 = always the 128x128 kernel, 256 = always 256x256
+
+template <int KIND, int OUT_DT>
+static void launch_big(GemmArgs& p, hipStream_t st) {
+  p.tiles_m = (p.M + 255) / 256;
+  p.tiles_n = (p.N + 255) / 256;
+  gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(512), 0, st>>>(p);
+}
+
 template <int KIND, int OUT_DT>
 static void launch_kind(GemmArgs& p, hipStream_t st) {
+  if ((p.K & 127) == 0 && (g_force_tile == 256 || (g_force_tile == 0 && g_use_dma && p.M > 1024))) {
+    launch_big<KIND, OUT_DT>(p, st);
+    return;
+  }
   if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, st);
   else if (p.M <= 64) launch_cfg<KIND, 64, 128, 1, 4, OUT_DT>(p, st);
   else launch_cfg<KIND, 128, 128, 2, 2, OUT_DT>(p, st);
@@ -365,6 +579,7 @@ using namespace sglq;
 // Test hook: choose between direct-to-LDS buffer loads (default) and loads staged
 // through registers.  Both fill LDS identically.
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
+extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 
 extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                                             int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,

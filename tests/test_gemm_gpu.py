@@ -37,12 +37,23 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
+@pytest.fixture(params=[0, 128, 256], ids=["tile_auto", "tile128", "tile256"])
+def tile(request):
+    from sglang_amd import _lib
+
+    _lib.load().sglq_debug_force_tile(request.param)
+    yield request.param
+    _lib.load().sglq_debug_force_tile(0)
+
+
 @pytest.mark.parametrize("mnk", [(1, 128, 64), (5, 136, 128), (16, 8, 16), (33, 264, 208), (127, 256, 4096), (128, 1024, 512),
                                  (130, 640, 1040), (512, 14336, 4096)])
-def test_int8_accumulators_bit_exact(gpu, load_path, mnk):
+def test_int8_accumulators_bit_exact(gpu, load_path, tile, mnk):
     from sglang_amd.sgl_kernel import int8_mm_i32
 
-    say("int8 acc", mnk, "direct" if load_path else "regs")
+    if tile == 256 and not load_path:
+        pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
+    say("int8 acc", mnk, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
     a, w = rand_i8((m, k), 1), rand_i8((n, k), 2)
     if m > 2:
@@ -89,10 +100,12 @@ def make_block_case(m, n, k, seed, outliers=False):
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(1, 128, 128), (3, 256, 512), (5, 2112, 1536), (127, 512, 7168), (128, 4096, 512),
                                  (256, 2048, 7168), (512, 1536, 1024), (1024, 640, 2048)])
-def test_fp8_blockwise_scaled_mm(gpu, load_path, mnk, out_dtype):
+def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
-    say("fp8_blockwise", mnk, out_dtype, "direct" if load_path else "regs")
+    if tile == 256 and not load_path:
+        pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
+    say("fp8_blockwise", mnk, out_dtype, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
     _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
     rows = sample_rows(m)
@@ -135,10 +148,10 @@ def test_fp8_blockwise_row_major_scales_vector(gpu):
 
 @pytest.mark.parametrize("with_bias", [False, True])
 @pytest.mark.parametrize("mnk", [(1, 4096, 4096), (32, 6144, 4096), (256, 4096, 14336), (2048, 1024, 4096), (7, 16, 32), (100, 264, 1040)])
-def test_fp8_scaled_mm(gpu, mnk, with_bias):
+def test_fp8_scaled_mm(gpu, tile, mnk, with_bias):
     from sglang_amd.sgl_kernel import fp8_scaled_mm
 
-    say("fp8_scaled_mm", mnk, with_bias)
+    say("fp8_scaled_mm", mnk, with_bias, "tile", tile)
     m, n, k = mnk
     x = O.gen_activation(m, k, seed=3000 + m)
     w = O.gen_weight(n, k, seed=3000 + n)
