@@ -6,12 +6,14 @@ resolved, importing the operators raises."""
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from pathlib import Path
 
 import torch
 
-LIB_PATH = Path(__file__).resolve().parent / "libsglq.so"
+# SGLQ_LIBRARY points at another build of the same C ABI (kernel development)
+LIB_PATH = Path(os.environ.get("SGLQ_LIBRARY") or Path(__file__).resolve().parent / "libsglq.so")
 
 SGLQ_BF16, SGLQ_FP16, SGLQ_FP32, SGLQ_I32 = 0, 1, 2, 3
 DTYPE_CODE = {torch.bfloat16: SGLQ_BF16, torch.float16: SGLQ_FP16, torch.float32: SGLQ_FP32}

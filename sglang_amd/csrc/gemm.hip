@@ -353,7 +353,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   // as zero through the buffer's extent (they are never stored).
   const int nkb = p.K >> 7;
   float sfa_cur[MI];
-  float sfb_cur = 0.f;
+  float sfb_cur = 0.f, sfb_next = 0.f;
   __amdgpu_buffer_rsrc_t rs = ra;
   uint32_t sfa_off = 0;
   int sfa_frag = 0, sfa_step = 0, nb = 0;
@@ -363,6 +363,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     const int nblocks = (p.N + 127) >> 7;
     nb = (n0 + wn * TN) >> 7;
     if (nb >= nblocks) nb = nblocks - 1;
+    nb = __builtin_amdgcn_readfirstlane(nb);
     const int mrow = m0 + wm * TM + r16;
     // a row past M must not alias a valid element of another K block: send it out of range
     sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
@@ -391,6 +392,8 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 
 #pragma unroll
   for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
 
   // One K step.  more_tag = another step follows: its copies and scales are issued here,
   // in the shadow of the MFMAs, so that no wave spends issue slots on them while the
@@ -398,9 +401,6 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   auto k_step = [&](int kb, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int cur = kb & 1;
-    __builtin_amdgcn_s_waitcnt(0);  // this stage has landed (copies were issued one K step ago)
-    __syncthreads();                // ... for every wave, and nobody still reads the other stage
-
     const char* st = smem + cur * STAGE_BYTES;
     v8i bf[NI];
     bf[0] = read_frag(st + b_base);
@@ -435,6 +435,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
             acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
             acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
           }
+          if (more && idx == NLOAD) sfb_next = p.sb[(kb + 1) * p.sb_stride_k + nb * p.sb_stride_n];
           // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
           if (more && j == 1 && i >= 1)
             sfa_cur[i - 1] = __builtin_bit_cast(
@@ -468,8 +469,19 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
         sfa_cur[MI - 1] = __builtin_bit_cast(
             float, __builtin_amdgcn_raw_buffer_load_b32(rs, ((sfa_ok >> (MI - 1)) & 1) ? sfa_off + (MI - 1) * sfa_frag : OOB,
                                                         (kb + 1) * sfa_step, 0));
-        sfb_cur = p.sb[(kb + 1) * p.sb_stride_k + nb * p.sb_stride_n];
+        sfb_cur = sfb_next;
       }
+    }
+    if constexpr (more) {
+      // The next stage's copies were the first eight vector-memory loads of this step
+      // and loads retire in order, so it is enough to wait until at most the
+      // SCALE_LOADS_AFTER_COPIES younger ones (activation-scale refills, none for the
+      // other kinds) are still in flight; lgkmcnt(0) covers this wave's LDS reads of the
+      // stage that the next step overwrites.  A bare s_barrier: the waits above are
+      // the only ordering needed, a fence would drain the scale refills as well.
+      constexpr int SCALE_LOADS_AFTER_COPIES = (KIND == KIND_FP8_BLOCK) ? MI - 1 : 0;
+      __builtin_amdgcn_s_waitcnt(SCALE_LOADS_AFTER_COPIES | (7 << 4));
+      __builtin_amdgcn_s_barrier();
     }
   };
   for (int kb = 0; kb + 1 < nkb; ++kb) k_step(kb, std::true_type{});
