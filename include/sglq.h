@@ -79,11 +79,20 @@ int sglq_per_token_quant_int8(const void* input, int in_dtype, void* output_q, f
  *   sfa fp32 [M, ceil(K/128)]  at sfa[m*sfa_stride_m + kb*sfa_stride_k]
  *   sfb fp32 [ceil(K/128), ceil(N/128)] at sfb[kb*sfb_stride_k + nb*sfb_stride_n]
  *   out [M, N] row stride ldo, out_dtype in {BF16, FP16}
- * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, a and b 16-byte aligned. */
+ * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, a and b 16-byte aligned.
+ *
+ * workspace (all four GEMM entry points): optional device scratch of
+ * workspace_bytes bytes, 16-byte aligned, owned by the caller and not shared
+ * with a call running concurrently on another stream.  For M <= 64 the weight
+ * matrix is streamed by several blocks per output tile (split-K) whose fp32 /
+ * int32 partial sums pass through it; it plays the part of the per-call
+ * workspace tensor that the reference's launchers allocate
+ * (fp8_blockwise_gemm_kernel.cu:153-155).  NULL or too small only costs speed. */
 int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                                  int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
                                  int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
-                                 int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+                                 int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                 int64_t workspace_bytes, void* stream);
 
 /* Replaces torch.ops.sgl_kernel.int8_scaled_mm
  * (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; schema common_extension.cc:101-104).
@@ -91,20 +100,20 @@ int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int6
  * bias may be NULL and otherwise has out_dtype. */
 int sglq_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
                         const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
-                        int64_t M, int64_t N, int64_t K, void* stream);
+                        int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* The INT32 accumulators of sglq_int8_scaled_mm before its epilogue, written
  * as int32 [M, N] with row stride ldo.  No counterpart op in the reference;
  * it exists so the accumulators can be compared bit for bit. */
 int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64_t ldb, int32_t* out, int64_t ldo,
-                     int64_t M, int64_t N, int64_t K, void* stream);
+                     int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Replaces torch.ops.sgl_kernel.fp8_scaled_mm
  * (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1071-1146; schema common_extension.cc:106-109).
  * out = scales_a[m] * (scales_b[n] * sum_k a*b) + bias[n], fp32 accumulation. */
 int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
                        const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
-                       int64_t M, int64_t N, int64_t K, void* stream);
+                       int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Test hook without a reference counterpart: non-zero (default) makes the GEMMs
  * copy global memory straight into LDS with buffer loads, zero stages the same
@@ -113,6 +122,9 @@ void sglq_debug_set_direct_lds(int on);
 /* Test hook: 0 = choose the GEMM tile by shape (default), 128 / 256 = always use
  * the 128x128 / 256x256 kernel. */
 void sglq_debug_force_tile(int tile);
+/* Test hook: > 0 fixes the split-K factor of the M <= 64 kernels (0 = by shape);
+ * with sglq_debug_force_tile(64 / 128 / 256): 64 = always the M <= 64 kernel where it applies. */
+void sglq_debug_force_splits(int splits);
 
 #ifdef __cplusplus
 }

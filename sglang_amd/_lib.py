@@ -20,17 +20,18 @@ DTYPE_CODE = {torch.bfloat16: SGLQ_BF16, torch.float16: SGLQ_FP16, torch.float32
 
 # name -> argtypes; every function returns int.  Mirrors include/sglq.h.
 _GROUP_QUANT = [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_int64, c_float, c_float, c_float, c_void_p]
-_ROWCOL_MM = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]
+_ROWCOL_MM = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64,
+              c_void_p, c_int64, c_void_p]
 SIGNATURES = {
     "sglq_per_token_group_quant_fp8": _GROUP_QUANT,
     "sglq_per_token_group_quant_int8": _GROUP_QUANT,
     "sglq_per_token_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_token_quant_int8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
-                                     c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
+                                     c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_int8_scaled_mm": _ROWCOL_MM,
     "sglq_fp8_scaled_mm": _ROWCOL_MM,
-    "sglq_int8_mm_i32": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    "sglq_int8_mm_i32": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
 }
 
 _lib = None
@@ -59,6 +60,8 @@ def load() -> ctypes.CDLL:
     lib.sglq_debug_set_direct_lds.restype = None
     lib.sglq_debug_force_tile.argtypes = [c_int]
     lib.sglq_debug_force_tile.restype = None
+    lib.sglq_debug_force_splits.argtypes = [c_int]
+    lib.sglq_debug_force_splits.restype = None
     _lib = lib
     return lib
 
@@ -69,6 +72,22 @@ def check(rc: int, what: str) -> None:
         if rc == 2:
             raise NotImplementedError(msg or what)
         raise RuntimeError(msg or f"{what} failed with code {rc}")
+
+
+_workspaces = {}
+WORKSPACE_BYTES = 64 << 20
+
+
+def workspace(device: torch.device):
+    """Per-device scratch for the split-K partial sums of the M <= 64 GEMM kernels,
+    allocated on first use (the reference caches its GEMM workspaces the same way,
+    sgl-kernel/python/sgl_kernel/utils.py `_get_cache_buf`).  Returns (pointer, bytes)."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    buf = _workspaces.get(key)
+    if buf is None:
+        buf = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf.data_ptr(), buf.numel()
 
 
 def stream_ptr(device: torch.device) -> int:

@@ -46,7 +46,13 @@ struct GemmArgs {
   uint32_t a_bytes, b_bytes;
   int M, N, K;
   int tiles_m, tiles_n;
+  void* ws;        // split-K partial sums [splits][M][N], fp32 or int32
+  int splits;
 };
+
+// s_waitcnt immediate: wait until at most `vm` vector-memory loads are outstanding
+// and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
+constexpr int waitcnt_vm_lgkm0(int vm) { return (vm & 0xf) | (((vm >> 4) & 3) << 14) | (7 << 4); }
 
 SGLQ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
@@ -95,6 +101,27 @@ SGLQ_DEV void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn)
   tn = in_group / gsz;
 }
 
+// Scale, add bias and store four consecutive outputs C[m][n..n+3] from their accumulators.
+template <int KIND, int OUT_DT, typename acc_t>
+SGLQ_DEV void finish4(const GemmArgs& p, int m, int n, const acc_t& a, float sam) {
+  const int64_t idx = (int64_t)m * p.ldo + n;
+  if constexpr (KIND == KIND_I8_RAW) {
+    *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = a;
+  } else if constexpr (KIND == KIND_FP8_BLOCK) {
+    store4<OUT_DT>(p.out, idx, a[0], a[1], a[2], a[3]);
+  } else {
+    float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
+    const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
+    if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)a[e], sbn[e] * sam, bv[e]);
+      else o[e] = __builtin_fmaf(sam, sbn[e] * a[e], bv[e]);
+    }
+    store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
+  }
+}
+
 // Scale, add bias and store a wave's accumulators.  acc[i][j][e] belongs to
 // C[m_base + 16 i + r16][n_base + 16 j + 4 g + e].
 template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
@@ -109,22 +136,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + j * 16 + g * 4;
       if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
-      const int64_t idx = (int64_t)m * p.ldo + n;
-      if constexpr (KIND == KIND_I8_RAW) {
-        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = acc[i][j];
-      } else if constexpr (KIND == KIND_FP8_BLOCK) {
-        store4<OUT_DT>(p.out, idx, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-      } else {
-        float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
-        const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
-        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbn[e] * sam, bv[e]);
-          else o[e] = __builtin_fmaf(sam, sbn[e] * acc[i][j][e], bv[e]);
-        }
-        store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
-      }
+      finish4<KIND, OUT_DT>(p, m, n, acc[i][j], sam);
     }
   }
 }
@@ -480,7 +492,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
       // stage that the next step overwrites.  A bare s_barrier: the waits above are
       // the only ordering needed, a fence would drain the scale refills as well.
       constexpr int SCALE_LOADS_AFTER_COPIES = (KIND == KIND_FP8_BLOCK) ? MI - 1 : 0;
-      __builtin_amdgcn_s_waitcnt(SCALE_LOADS_AFTER_COPIES | (7 << 4));
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(SCALE_LOADS_AFTER_COPIES));
       __builtin_amdgcn_s_barrier();
     }
   };
@@ -488,6 +500,190 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   k_step(nkb - 1, std::false_type{});
 
   epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+}
+
+
+// ---------------------------------------------------------------------------
+// Decode kernel (M <= 64): the weight matrix is streamed once from HBM, so the
+// job is to keep enough bytes in flight.  A block owns 128 weight rows and a
+// contiguous range of K blocks (split-K across blocks); its four waves take 32
+// rows each.  Weight tiles (16 KiB), the activation tile and, for the block-scaled
+// kind, the activation scales of each K block are copied global -> LDS through a
+// ring of NSTAGE stages, NSTAGE - 1 copies ahead of the MFMAs (80-100 KiB in
+// flight per CU).  All copies of a stage are vector-memory loads that retire in
+// order, so "stage t has landed" is a vmcnt wait that leaves the younger stages'
+// loads outstanding.  With splits > 1 the partial sums go to a workspace and
+// splitk_reduce_kernel applies the epilogue.
+// ---------------------------------------------------------------------------
+template <int KIND, int MI, int OUT_DT>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
+  constexpr int BN = 128, NI = 2;
+  constexpr int AR = MI * 16 < 32 ? 32 : MI * 16;  // activation rows staged (at least one copy per wave)
+  constexpr int ACW = AR / 32;                     // activation copies per wave per stage
+  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  constexpr int CPW = 4 + ACW + (BLOCK ? 1 : 0);   // vector-memory loads per wave per stage
+  constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 1024 : 0;
+  constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
+  constexpr int NSTAGE = MI <= 2 ? 6 : 5;
+  constexpr int MAX_STEPS = 1024;                  // K blocks per split that the weight-scale table holds
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+
+  __shared__ __attribute__((aligned(1024))) char smem[NSTAGE * STAGE_BYTES];
+  __shared__ float sfb_tab[BLOCK ? MAX_STEPS : 1];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4, l8 = lane >> 3;
+
+  const int tile_n = blockIdx.x % p.tiles_n, split = blockIdx.x / p.tiles_n;
+  const int n0 = tile_n * BN;
+  const int nkb = p.K >> 7;
+  const int kb0 = (int)((int64_t)split * nkb / p.splits), kb1 = (int)((int64_t)(split + 1) * nkb / p.splits);
+  const int nsteps = kb1 - kb0;
+
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
+  __amdgpu_buffer_rsrc_t rs = ra;
+
+  // Same copy plan as the prefill kernel: lane l brings row l / 8 of an 8-row
+  // group, chunk (l % 8) ^ swz(row); copies of one wave differ by 32 rows.
+  const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
+  const uint32_t off_w = (uint32_t)(n0 + wave * 8 + l8) * p.ldb + c16;
+  const uint32_t off_a = (uint32_t)(wave * 8 + l8) * p.lda + c16;
+  const uint32_t step_w = 32u * p.ldb, step_a = 32u * p.lda;
+  uint32_t off_s = 0;
+  int sfa_step = 0;
+  if constexpr (BLOCK) {
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    off_s = lane < p.M ? (uint32_t)(lane * p.sa_stride_m * 4) : OOB;  // lane = activation row
+    sfa_step = (int)(p.sa_stride_k * 4);
+    const int nblocks = (p.N + 127) >> 7;
+    const int nb = tile_n < nblocks ? tile_n : nblocks - 1;
+    for (int t = threadIdx.x; t < nsteps; t += 256)
+      sfb_tab[t] = p.sb[(int64_t)(kb0 + t) * p.sb_stride_k + nb * p.sb_stride_n];
+  }
+
+  auto issue_group = [&](int t) {  // all copies of K block kb0 + t into stage t % NSTAGE
+    char* st = smem + (t % NSTAGE) * STAGE_BYTES;
+    const int k0 = (kb0 + t) * 128;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(st + (wave + 4 * j) * 1024),
+                                               16, off_w + j * step_w, k0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < ACW; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          ra, (__attribute__((address_space(3))) void*)(st + W_BYTES + (wave + 4 * j) * 1024), 16, off_a + j * step_a,
+          k0, 0, 0);
+    if constexpr (BLOCK)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rs, (__attribute__((address_space(3))) void*)(st + W_BYTES + A_BYTES + wave * 256), 4, off_s,
+          (kb0 + t) * sfa_step, 0, 0);
+  };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+  // the sfb table was filled with ordinary loads and LDS stores: make it visible before the ring starts
+  __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
+
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t)
+    if (t < nsteps) issue_group(t);
+
+  for (int t = 0; t < nsteps; ++t) {
+    // wait for stage t: at most NSTAGE - 2 younger groups may stay in flight
+    if (nsteps - 1 - t >= NSTAGE - 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NSTAGE - 2) * CPW));
+    else __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_s_barrier();  // visible to all waves; and everyone is done with stage (t - 1) % NSTAGE
+    if (t + NSTAGE - 1 < nsteps) issue_group(t + NSTAGE - 1);
+
+    const char* st = smem + (t % NSTAGE) * STAGE_BYTES;
+    v8i wf[NI], af[MI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) wf[j] = read_frag(st + (wave * 32 + j * 16) * 128);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) af[i] = read_frag(st + W_BYTES + i * 16 * 128);
+    float sc[MI];
+    if constexpr (BLOCK) {
+      const float sfb = sfb_tab[t];
+      const float* sfa = reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + wave * 256);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sc[i] = sfa[i * 16 + r16] * sfb;
+    }
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        if constexpr (BLOCK) {
+          const v4f z = {0.f, 0.f, 0.f, 0.f};
+          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], sc[i], acc[i][j][e]);
+        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+        } else {
+          const v4i b0 = {wf[j][0], wf[j][1], wf[j][2], wf[j][3]}, b1 = {wf[j][4], wf[j][5], wf[j][6], wf[j][7]};
+          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]}, a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  if (p.splits == 1) {
+    epilogue<KIND, OUT_DT, MI, NI>(p, acc, 0, n0 + wave * 32, r16, g);
+  } else {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int m = i * 16 + r16;
+      if (m >= p.M) continue;
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const int n = n0 + wave * 32 + j * 16 + g * 4;
+        if (n >= p.N) continue;
+        acc_t* dst =
+            reinterpret_cast<acc_t*>(reinterpret_cast<char*>(p.ws) + (((int64_t)split * p.M + m) * p.N + n) * 4);
+        *dst = acc[i][j];
+      }
+    }
+  }
+}
+
+// Sum the split-K partials in split order and apply the epilogue; one thread per
+// run of four consecutive n.
+template <int KIND, int OUT_DT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  const int n4 = p.N >> 2;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)p.M * n4) return;
+  const int m = (int)(id / n4), n = (int)(id % n4) * 4;
+  const acc_t* src =
+      reinterpret_cast<const acc_t*>(reinterpret_cast<const char*>(p.ws) + ((int64_t)m * p.N + n) * 4);
+  const int64_t stride = (int64_t)p.M * p.N / 4;  // in acc_t units
+  acc_t a = src[0];
+  for (int s = 1; s < p.splits; ++s) a += src[s * stride];
+  float sam = 1.f;
+  if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = p.sa[m];
+  finish4<KIND, OUT_DT>(p, m, n, a, sam);
 }
 
 // ---------------------------------------------------------------------------
@@ -513,8 +709,47 @@ static void launch_big(GemmArgs& p, hipStream_t st) {
   gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(512), 0, st>>>(p);
 }
 
+static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor of the decode kernel
+
+template <int KIND, int MI, int OUT_DT>
+static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
+  gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits)), dim3(256), 0, st>>>(p);
+  if (p.splits > 1) {
+    const int64_t work = (int64_t)p.M * (p.N >> 2);
+    splitk_reduce_kernel<KIND, OUT_DT><<<dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st>>>(p);
+  }
+}
+
+// Decode path: choose the split-K factor so that a few blocks per CU stream weights
+// concurrently, without letting the fp32 partials exceed a quarter of the weight bytes.
 template <int KIND, int OUT_DT>
-static void launch_kind(GemmArgs& p, hipStream_t st) {
+static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  p.tiles_m = 1;
+  p.tiles_n = (p.N + 127) / 128;
+  const int nkb = p.K >> 7;
+  int splits = (768 + p.tiles_n - 1) / p.tiles_n;          // aim at ~3 blocks per CU
+  const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;          // at least two K blocks per split
+  const int by_traffic = (int)(p.K / (16 * (int64_t)p.M)) > 0 ? (int)(p.K / (16 * (int64_t)p.M)) : 1;
+  if (splits > by_steps) splits = by_steps;
+  if (splits > by_traffic) splits = by_traffic;
+  if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
+  const int64_t per_split = (int64_t)p.M * p.N * 4;
+  if (!p.ws || ws_bytes < per_split * 2) splits = 1;
+  else if (splits * per_split > ws_bytes) splits = (int)(ws_bytes / per_split);
+  if (splits < 1) splits = 1;
+  p.splits = splits;
+  if (p.M <= 16) launch_skinny_mi<KIND, 1, OUT_DT>(p, st);
+  else if (p.M <= 32) launch_skinny_mi<KIND, 2, OUT_DT>(p, st);
+  else launch_skinny_mi<KIND, 4, OUT_DT>(p, st);
+}
+
+template <int KIND, int OUT_DT>
+static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  // the decode kernel keeps one weight scale per K block of its split in a 1024-entry table
+  if ((p.K & 127) == 0 && p.M <= 64 && p.K <= 1024 * 128 && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
+    launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
+    return;
+  }
   if ((p.K & 127) == 0 && (g_force_tile == 256 || (g_force_tile == 0 && g_use_dma && p.M > 1024))) {
     launch_big<KIND, OUT_DT>(p, st);
     return;
@@ -592,11 +827,13 @@ using namespace sglq;
 // through registers.  Both fill LDS identically.
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
+extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
 
 extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                                             int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
                                             int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
-                                            int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+                                            int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                            int64_t workspace_bytes, void* stream) {
   const char* name = "fp8_blockwise_scaled_mm";
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
@@ -617,15 +854,17 @@ extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const vo
   p.sa_stride_k = sfa_stride_k;
   p.sb_stride_k = sfb_stride_k;
   p.sb_stride_n = sfb_stride_n;
+  p.ws = workspace;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_BLOCK, SGLQ_BF16>(p, st);
-  else launch_kind<KIND_FP8_BLOCK, SGLQ_FP16>(p, st);
+  if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_BLOCK, SGLQ_BF16>(p, workspace_bytes, st);
+  else launch_kind<KIND_FP8_BLOCK, SGLQ_FP16>(p, workspace_bytes, st);
   return finish(name);
 }
 
 static int rowcol_entry(const char* name, bool fp8, const void* a, int64_t lda, const void* b, int64_t ldb,
                         const float* scales_a, const float* scales_b, const void* bias, void* out, int64_t ldo,
-                        int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+                        int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                        void* stream) {
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
@@ -646,39 +885,44 @@ static int rowcol_entry(const char* name, bool fp8, const void* a, int64_t lda, 
   p.sa = scales_a;
   p.sb = scales_b;
   p.bias = bias;
+  p.ws = workspace;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fp8) {
-    if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_ROWCOL, SGLQ_BF16>(p, st);
-    else launch_kind<KIND_FP8_ROWCOL, SGLQ_FP16>(p, st);
+    if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_ROWCOL, SGLQ_BF16>(p, workspace_bytes, st);
+    else launch_kind<KIND_FP8_ROWCOL, SGLQ_FP16>(p, workspace_bytes, st);
   } else {
-    if (out_dtype == SGLQ_BF16) launch_kind<KIND_I8_ROWCOL, SGLQ_BF16>(p, st);
-    else launch_kind<KIND_I8_ROWCOL, SGLQ_FP16>(p, st);
+    if (out_dtype == SGLQ_BF16) launch_kind<KIND_I8_ROWCOL, SGLQ_BF16>(p, workspace_bytes, st);
+    else launch_kind<KIND_I8_ROWCOL, SGLQ_FP16>(p, workspace_bytes, st);
   }
   return finish(name);
 }
 
 extern "C" int sglq_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
                                    const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
-                                   int64_t M, int64_t N, int64_t K, void* stream) {
+                                   int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                   void* stream) {
   return rowcol_entry("int8_scaled_mm", false, a, lda, b, ldb, scales_a, scales_b, bias, out, ldo, out_dtype, M, N, K,
-                      stream);
+                      workspace, workspace_bytes, stream);
 }
 
 extern "C" int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* scales_a,
                                   const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
-                                  int64_t M, int64_t N, int64_t K, void* stream) {
+                                  int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                  void* stream) {
   return rowcol_entry("fp8_scaled_mm", true, a, lda, b, ldb, scales_a, scales_b, bias, out, ldo, out_dtype, M, N, K,
-                      stream);
+                      workspace, workspace_bytes, stream);
 }
 
 extern "C" int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64_t ldb, int32_t* out, int64_t ldo,
-                                int64_t M, int64_t N, int64_t K, void* stream) {
+                                int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                void* stream) {
   const char* name = "int8_mm_i32";
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 4);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
   GemmArgs p;
   fill_common(p, a, lda, b, ldb, out, ldo, M, N, K);
-  launch_kind<KIND_I8_RAW, SGLQ_BF16>(p, static_cast<hipStream_t>(stream));
+  p.ws = workspace;
+  launch_kind<KIND_I8_RAW, SGLQ_BF16>(p, workspace_bytes, static_cast<hipStream_t>(stream));
   return finish(name);
 }

@@ -134,7 +134,8 @@ def _int8_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None)
     rc = lib.sglq_int8_scaled_mm(
         mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
         scales_a.data_ptr(), scales_b.data_ptr(), bias.data_ptr() if bias is not None else None,
-        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, *_lib.workspace(mat_a.device),
+        _lib.stream_ptr(mat_a.device))
     _lib.check(rc, "int8_scaled_mm")
     return out
 
@@ -150,7 +151,8 @@ def _fp8_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
     rc = lib.sglq_fp8_scaled_mm(
         mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
         scales_a.data_ptr(), scales_b.data_ptr(), bias.data_ptr() if bias is not None else None,
-        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, *_lib.workspace(mat_a.device),
+        _lib.stream_ptr(mat_a.device))
     _lib.check(rc, "fp8_scaled_mm")
     return out
 
@@ -167,7 +169,8 @@ def _fp8_blockwise_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype):
         mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
         scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
         scales_b.data_ptr(), scales_b.stride(0), scales_b.stride(1),
-        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, _lib.stream_ptr(mat_a.device))
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, *_lib.workspace(mat_a.device),
+        _lib.stream_ptr(mat_a.device))
     _lib.check(rc, "fp8_blockwise_scaled_mm")
     return out
 
@@ -289,6 +292,6 @@ def int8_mm_i32(mat_a: torch.Tensor, mat_b: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     rc = lib.sglq_int8_mm_i32(mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(),
                               mat_b.stride(1) if n > 1 else k, out.data_ptr(), out.stride(0), m, n, k,
-                              _lib.stream_ptr(mat_a.device))
+                              *_lib.workspace(mat_a.device), _lib.stream_ptr(mat_a.device))
     _lib.check(rc, "int8_mm_i32")
     return out

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
 
     lib = _lib.load()
     names = declared_symbols()
-    assert len(names) >= 11
+    assert len(names) >= 13
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/sglq.h but not exported"
     assert lib.sglq_abi_version() == 1
@@ -156,9 +156,9 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == 2  # group size not built
     rc = lib.sglq_per_token_quant_fp8(p, 0, p, p, 4, 12, None)
     assert rc == 1 and b"divisible by 8" in lib.sglq_last_error()
-    rc = lib.sglq_int8_scaled_mm(p, 24, p, 24, p, p, None, p, 8, 0, 4, 8, 24, None)
+    rc = lib.sglq_int8_scaled_mm(p, 24, p, 24, p, p, None, p, 8, 0, 4, 8, 24, None, 0, None)
     assert rc == 1 and b"multiple of 16" in lib.sglq_last_error()
-    rc = lib.sglq_fp8_blockwise_scaled_mm(p, 128, p, 128, p, 1, 4, p, 1, 1, p, 8, 2, 4, 8, 128, None)
+    rc = lib.sglq_fp8_blockwise_scaled_mm(p, 128, p, 128, p, 1, 4, p, 1, 1, p, 8, 2, 4, 8, 128, None, 0, None)
     assert rc == 1 and b"out_dtype" in lib.sglq_last_error()
     # empty problems are a no-op
-    assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None) == 0
+    assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0

@@ -37,7 +37,7 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
-@pytest.fixture(params=[0, 128, 256], ids=["tile_auto", "tile128", "tile256"])
+@pytest.fixture(params=[0, 128, 256], ids=["tile_auto", "tile128", "tile256"])  # tile_auto sends M <= 64 to the decode kernel
 def tile(request):
     from sglang_amd import _lib
 
@@ -187,6 +187,51 @@ def test_gemm_linearity_at_full_size(gpu):
     rows = sample_rows(m, 12)
     ref = O.fp8_blockwise_scaled_mm(xq[rows.to(gpu)].cpu(), wq.t(), xs[rows.to(gpu)].cpu(), ws.t(), torch.float32)
     torch.testing.assert_close(out[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.fixture(params=[0, 1, 2, 5], ids=["splits_auto", "splits1", "splits2", "splits5"])
+def splits(request):
+    from sglang_amd import _lib
+
+    _lib.load().sglq_debug_force_splits(request.param)
+    yield request.param
+    _lib.load().sglq_debug_force_splits(0)
+
+
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (7, 2112, 7168), (16, 7168, 2048), (17, 264, 1024), (33, 4096, 512),
+                                 (64, 1536, 4096), (48, 136, 16384)])
+def test_decode_kernel_split_k(gpu, splits, mnk):
+    """M <= 64 runs on the weight-streaming kernel; its split-K partial sums and the
+    reduction must reproduce the oracle for every kind and any split factor."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32, int8_scaled_mm
+
+    say("decode kernel", mnk, "splits", splits)
+    m, n, k = mnk
+    # block-scaled FP8
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m * n + k, outliers=True)
+    ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs.to(gpu) if k == 128 else xs_cm, ws.to(gpu).t(), torch.float16)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    # per-row / per-column FP8 with bias
+    g = torch.Generator().manual_seed(m + n)
+    sa = torch.rand((m, 1), generator=g) * 0.05 + 0.01
+    sb = torch.rand((n, 1), generator=g) * 0.001 + 0.0005
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16)
+    ref = O.fp8_scaled_mm(xq, wq.t(), sa, sb, torch.float32, bias, acc_dtype=torch.float64)
+    out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    # INT8: accumulators exact, epilogue within tolerance
+    a8, w8 = rand_i8((m, k), 3), rand_i8((n, k), 4)
+    acc_ref = O.int8_mm_i32(a8, w8.t())
+    acc = int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()
+    assert torch.equal(acc, acc_ref)
+    sa8 = sa * 0.01
+    ref = O.int8_scaled_mm(a8, w8.t(), sa8, sb, torch.bfloat16, bias)
+    out = int8_scaled_mm(a8.to(gpu), w8.to(gpu).t(), sa8.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
 
 
 def test_gemm_empty_m(gpu):
