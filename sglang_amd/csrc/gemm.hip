@@ -54,6 +54,27 @@ struct GemmArgs {
 // and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
 constexpr int waitcnt_vm_lgkm0(int vm) { return (vm & 0xf) | (((vm >> 4) & 3) << 14) | (7 << 4); }
 
+// Global -> LDS copies written as assembly (16 or 4 bytes per lane; lane l lands at
+// lds_dst + l * size).  The decode kernel keeps several stages of such copies in flight and
+// waits for them with explicit vmcnt counts; copies issued through the compiler's builtin
+// are tracked by its wait-count pass, which cannot tell the ring's stages apart and would
+// drain every copy in flight before each LDS read.
+SGLQ_DEV v4u make_rsrc_sgpr(const void* ptr, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+  return v4u{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+             (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+             (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+}
+SGLQ_DEV void lds_copy16(v4u rsrc, uint32_t lds_dst, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+SGLQ_DEV void lds_copy4(v4u rsrc, uint32_t lds_dst, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds" : : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+SGLQ_DEV uint32_t lds_addr(const void* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p);
+}
+
 SGLQ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
 template <int OUT_DT>
@@ -524,7 +545,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int CPW = 4 + ACW + (BLOCK ? 1 : 0);   // vector-memory loads per wave per stage
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 1024 : 0;
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
-  constexpr int NSTAGE = MI <= 2 ? 6 : 5;
+  constexpr int NSTAGE = 3;  // 64-77 KiB of LDS: two blocks (eight waves) per CU
   constexpr int MAX_STEPS = 1024;                  // K blocks per split that the weight-scale table holds
   constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
 
@@ -538,12 +559,15 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   const int tile_n = blockIdx.x % p.tiles_n, split = blockIdx.x / p.tiles_n;
   const int n0 = tile_n * BN;
   const int nkb = p.K >> 7;
-  const int kb0 = (int)((int64_t)split * nkb / p.splits), kb1 = (int)((int64_t)(split + 1) * nkb / p.splits);
-  const int nsteps = kb1 - kb0;
+  // Split s takes the K blocks s, s + splits, s + 2 splits, ...: the blocks that share a
+  // weight tile then read neighbouring 128-byte pieces of the same rows at about the same
+  // time, which keeps DRAM pages open longer than giving each split one contiguous K range.
+  const int kb0 = split, kstride = p.splits;
+  const int nsteps = (nkb - split + p.splits - 1) / p.splits;
 
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
-  __amdgpu_buffer_rsrc_t rs = ra;
+  const v4u ra = make_rsrc_sgpr(p.a, p.a_bytes);
+  const v4u rb = make_rsrc_sgpr(p.b, p.b_bytes);
+  v4u rs = ra;
 
   // Same copy plan as the prefill kernel: lane l brings row l / 8 of an 8-row
   // group, chunk (l % 8) ^ swz(row); copies of one wave differ by 32 rows.
@@ -555,31 +579,25 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   int sfa_step = 0;
   if constexpr (BLOCK) {
     const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
-    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    rs = make_rsrc_sgpr(p.sa, (uint32_t)(sfa_elems * 4));
     off_s = lane < p.M ? (uint32_t)(lane * p.sa_stride_m * 4) : OOB;  // lane = activation row
     sfa_step = (int)(p.sa_stride_k * 4);
     const int nblocks = (p.N + 127) >> 7;
     const int nb = tile_n < nblocks ? tile_n : nblocks - 1;
     for (int t = threadIdx.x; t < nsteps; t += 256)
-      sfb_tab[t] = p.sb[(int64_t)(kb0 + t) * p.sb_stride_k + nb * p.sb_stride_n];
+      sfb_tab[t] = p.sb[(int64_t)(kb0 + t * kstride) * p.sb_stride_k + nb * p.sb_stride_n];
   }
 
+  const uint32_t smem_base = lds_addr(smem);
   auto issue_group = [&](int t) {  // all copies of K block kb0 + t into stage t % NSTAGE
-    char* st = smem + (t % NSTAGE) * STAGE_BYTES;
-    const int k0 = (kb0 + t) * 128;
+    const uint32_t st = smem_base + (uint32_t)(t % NSTAGE) * STAGE_BYTES;
+    const uint32_t k0 = (uint32_t)(kb0 + t * kstride) * 128u;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(st + (wave + 4 * j) * 1024),
-                                               16, off_w + j * step_w, k0, 0, 0);
+    for (int j = 0; j < 4; ++j) lds_copy16(rb, st + (wave + 4 * j) * 1024, off_w + j * step_w, k0);
 #pragma unroll
-    for (int j = 0; j < ACW; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          ra, (__attribute__((address_space(3))) void*)(st + W_BYTES + (wave + 4 * j) * 1024), 16, off_a + j * step_a,
-          k0, 0, 0);
-    if constexpr (BLOCK)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rs, (__attribute__((address_space(3))) void*)(st + W_BYTES + A_BYTES + wave * 256), 4, off_s,
-          (kb0 + t) * sfa_step, 0, 0);
+    for (int j = 0; j < ACW; ++j) lds_copy16(ra, st + W_BYTES + (wave + 4 * j) * 1024, off_a + j * step_a, k0);
+    // one dword per lane: its row's activation scale for this K block
+    if constexpr (BLOCK) lds_copy4(rs, st + W_BYTES + A_BYTES + wave * 256, off_s, (uint32_t)((kb0 + t * kstride) * sfa_step));
   };
 
   const int sw = (r16 & 7) ^ (r16 >> 3);
@@ -721,15 +739,16 @@ static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
 }
 
 // Decode path: choose the split-K factor so that a few blocks per CU stream weights
-// concurrently, without letting the fp32 partials exceed a quarter of the weight bytes.
+// concurrently, without letting the partial sums' traffic exceed an eighth of the weight bytes.
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = 1;
   p.tiles_n = (p.N + 127) / 128;
   const int nkb = p.K >> 7;
-  int splits = (768 + p.tiles_n - 1) / p.tiles_n;          // aim at ~3 blocks per CU
+  int splits = (512 + p.tiles_n / 2) / p.tiles_n;          // aim at two blocks (eight waves) per CU
   const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;          // at least two K blocks per split
-  const int by_traffic = (int)(p.K / (16 * (int64_t)p.M)) > 0 ? (int)(p.K / (16 * (int64_t)p.M)) : 1;
+  // partial sums cost 8 * M * N * splits bytes of traffic against N * K of weights: keep them under an eighth
+  const int by_traffic = (int)(p.K / (64 * (int64_t)p.M)) > 0 ? (int)(p.K / (64 * (int64_t)p.M)) : 1;
   if (splits > by_steps) splits = by_steps;
   if (splits > by_traffic) splits = by_traffic;
   if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
