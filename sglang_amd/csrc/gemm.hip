@@ -162,6 +162,80 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
   }
 }
 
+// Epilogue of the 256 x 256 kernel for 16-bit outputs: every wave converts its
+// accumulators (scales and bias applied) and drops them into a 256 x 512-byte image of
+// the C tile in LDS, then the block writes the image out in rows, 16 bytes per lane, so
+// that a wavefront store covers two full 512-byte row segments instead of sixteen
+// 32-byte pieces.  Chunk c (16 bytes) of row r sits at chunk position c ^ (r & 31).
+// The caller guarantees that nobody reads the stage buffers any more.
+template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
+SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* smem, int m0, int n0, int wm, int wn,
+                               int r16, int g, int lane, int wave) {
+  constexpr int TM = MI * 16, TN = NI * 16;
+  float bv[NI][4], sbv[NI][4];
+  if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n0 + wn * TN + j * 16 + g * 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bv[j][e] = 0.f;
+        sbv[j][e] = 0.f;
+      }
+      if (n < p.N) {
+        const v4f t = *reinterpret_cast<const v4f*>(p.sb + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sbv[j][e] = t[e];
+        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv[j]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int ml = wm * TM + i * 16 + r16;
+    float sam = 1.f;
+    if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = (m0 + ml < p.M) ? p.sa[m0 + ml] : 0.f;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[j][e] * sam, bv[j][e]);
+        else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam, sbv[j][e] * acc[i][j][e], bv[j][e]);
+        else o[e] = acc[i][j][e];
+      }
+      const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
+      char* dst = smem + ml * 512 + ((chunk ^ (ml & 31)) * 16) + (g & 1) * 8;
+      if constexpr (OUT_DT == SGLQ_BF16) {
+        typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<bf4*>(dst) = bf4{(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
+      } else {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<h4*>(dst) = h4{(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
+      }
+    }
+  }
+  __syncthreads();
+  // 256 rows, 8 waves: wave w writes rows 32 w .. 32 w + 31, two rows per store instruction
+  const int c = lane & 31;
+  const int n = n0 + c * 8;
+  char* out = reinterpret_cast<char*>(p.out);
+#pragma unroll 4
+  for (int it = 0; it < 16; ++it) {
+    const int ml = wave * 32 + it * 2 + (lane >> 5);
+    const int m = m0 + ml;
+    const v4i v = *reinterpret_cast<const v4i*>(smem + ml * 512 + ((c ^ (ml & 31)) * 16));
+    if (m < p.M) {
+      char* row = out + ((int64_t)m * p.ldo + n) * 2;
+      if (n + 8 <= p.N) {
+        *reinterpret_cast<v4i*>(row) = v;
+      } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
+        *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[0], (uint32_t)v[1]};
+      }
+    }
+  }
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT, bool DMA>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const GemmArgs p) {
   constexpr int NW = WAVES_M * WAVES_N;
@@ -520,7 +594,18 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   for (int kb = 0; kb + 1 < nkb; ++kb) k_step(kb, std::true_type{});
   k_step(nkb - 1, std::false_type{});
 
-  epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+  if constexpr (KIND == KIND_I8_RAW) {
+    epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+  } else {
+    // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
+    const bool aligned = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    if (aligned) {
+      __syncthreads();  // every wave is done with the last stage: the buffers become the C image
+      epilogue_via_lds<KIND, OUT_DT, MI, NI>(p, acc, smem, m0, n0, wm, wn, r16, g, lane, wave);
+    } else {
+      epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+    }
+  }
 }
 
 
