@@ -228,15 +228,22 @@ def run_headline(args):
 # --sweep: every configuration, one JSON line per (config, shape)
 # ---------------------------------------------------------------------------
 def time_kernel(fn, iters, rotate=1):
+    """Device-side time per call: `iters` calls captured into one HIP graph (no host
+    launch gaps inside), inputs rotated so that consecutive calls do not reuse cached data."""
     import torch
 
-    for i in range(3):
+    for i in range(max(2, rotate)):
         fn(i % rotate)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(iters):
+            fn(i % rotate)
+    g.replay()
     torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
-    for i in range(iters):
-        fn(i % rotate)
+    g.replay()
     e.record()
     torch.cuda.synchronize()
     return s.elapsed_time(e) / iters

@@ -143,6 +143,24 @@ SGLQ_DEV void finish4(const GemmArgs& p, int m, int n, const acc_t& a, float sam
   }
 }
 
+// Split-K: store a wave's raw accumulators as partial sums of split `split` in the
+// workspace, laid out [split][M][N] (fp32 or int32); splitk_reduce_kernel finishes them.
+template <int MI, int NI, typename acc_t>
+SGLQ_DEV void store_partials(const GemmArgs& p, acc_t (&acc)[MI][NI], int split, int m_base, int n_base, int r16, int g) {
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m_base + i * 16 + r16;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n_base + j * 16 + g * 4;
+      if (n >= p.N) continue;
+      acc_t* dst = reinterpret_cast<acc_t*>(reinterpret_cast<char*>(p.ws) + (((int64_t)split * p.M + m) * p.N + n) * 4);
+      *dst = acc[i][j];
+    }
+  }
+}
+
 // Scale, add bias and store a wave's accumulators.  acc[i][j][e] belongs to
 // C[m_base + 16 i + r16][n_base + 16 j + 4 g + e].
 template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
@@ -254,8 +272,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int r16 = lane & 15, g = lane >> 4;
 
+  // blockIdx = split * tiles + tile; split s works on K blocks [kb_lo, kb_hi)
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int split = blockIdx.x / tiles;
   int tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  tile_of_block(blockIdx.x - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
@@ -310,7 +331,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
   // ---- block scales: one activation scale per lane per 16-row fragment
-  const int nkb = (p.K + 127) >> 7;
+  const int nkb_all = (p.K + 127) >> 7;
+  const int kb_lo = (int)((int64_t)split * nkb_all / p.splits), nkb = (int)((int64_t)(split + 1) * nkb_all / p.splits);
   float sfa_next[MI];
   float sfb_next = 0.f;
   int sfa_row[MI];
@@ -323,14 +345,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     for (int i = 0; i < MI; ++i) {
       int m = m0 + wm * TM + i * 16 + r16;
       sfa_row[i] = m < p.M ? m : p.M - 1;
-      sfa_next[i] = p.sa[sfa_row[i] * p.sa_stride_m];
+      sfa_next[i] = p.sa[sfa_row[i] * p.sa_stride_m + kb_lo * p.sa_stride_k];
     }
-    sfb_next = p.sb[nb * p.sb_stride_n];
+    sfb_next = p.sb[kb_lo * p.sb_stride_k + nb * p.sb_stride_n];
   }
 
-  issue_loads(0, 0);
+  issue_loads(kb_lo & 1, kb_lo * 128);
 
-  for (int kb = 0; kb < nkb; ++kb) {
+  for (int kb = kb_lo; kb < nkb; ++kb) {
     const int cur = kb & 1;
     __builtin_amdgcn_s_waitcnt(0);  // this stage's copies (and prefetched scales) have landed
     __syncthreads();                // for every wave; and all waves are done reading the other stage
@@ -387,7 +409,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     }
   }
 
-  epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+  if (p.splits > 1) store_partials<MI, NI>(p, acc, split, m0 + wm * TM, n0 + wn * TN, r16, g);
+  else epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
 }
 
 // ---------------------------------------------------------------------------
@@ -750,23 +773,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
     }
   }
 
-  if (p.splits == 1) {
-    epilogue<KIND, OUT_DT, MI, NI>(p, acc, 0, n0 + wave * 32, r16, g);
-  } else {
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      const int m = i * 16 + r16;
-      if (m >= p.M) continue;
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        const int n = n0 + wave * 32 + j * 16 + g * 4;
-        if (n >= p.N) continue;
-        acc_t* dst =
-            reinterpret_cast<acc_t*>(reinterpret_cast<char*>(p.ws) + (((int64_t)split * p.M + m) * p.N + n) * 4);
-        *dst = acc[i][j];
-      }
-    }
-  }
+  if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, 0, n0 + wave * 32, r16, g);
+  else store_partials<MI, NI>(p, acc, split, 0, n0 + wave * 32, r16, g);
 }
 
 // Sum the split-K partials in split order and apply the epilogue; one thread per
@@ -794,13 +802,38 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------
 static bool g_use_dma = true;
 
+static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
+
+template <int KIND, int OUT_DT>
+static void launch_reduce(GemmArgs& p, hipStream_t st);
+
+// 128 x 128 (and narrower) tiles.  When the tiles do not fill the chip (two blocks per
+// CU), K is split across blocks as far as the workspace and the partial sums' traffic allow.
 template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT>
-static void launch_cfg(GemmArgs& p, hipStream_t st) {
+static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  dim3 grid((uint32_t)(p.tiles_m * p.tiles_n)), block(WAVES_M * WAVES_N * 64);
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int nkb = (p.K + 127) >> 7;
+  int splits = 1;
+  if (tiles < 384) {
+    splits = (512 + tiles / 2) / tiles;
+    const int by_steps = nkb / 4 > 0 ? nkb / 4 : 1;  // at least four K blocks per split
+    // partial sums: 8 * M * N * splits bytes written and read, against (M + N) * K of operands
+    const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
+    if (splits > by_steps) splits = by_steps;
+    if (splits > by_traffic) splits = (int)(by_traffic > 0 ? by_traffic : 1);
+  }
+  if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
+  const int64_t per_split = (int64_t)p.M * p.N * 4;
+  if (!p.ws || ws_bytes < per_split * 2) splits = 1;
+  else if (splits * per_split > ws_bytes) splits = (int)(ws_bytes / per_split);
+  if (splits < 1) splits = 1;
+  p.splits = splits;
+  dim3 grid((uint32_t)(tiles * splits)), block(WAVES_M * WAVES_N * 64);
   if (g_use_dma) gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, true><<<grid, block, 0, st>>>(p);
   else gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, false><<<grid, block, 0, st>>>(p);
+  if (splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
 static int g_force_tile = 0;  // test hook: 0 = heuristic, 128 = always the 128x128 kernel, 256 = always 256x256
@@ -809,33 +842,34 @@ template <int KIND, int OUT_DT>
 static void launch_big(GemmArgs& p, hipStream_t st) {
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 255) / 256;
+  p.splits = 1;
   gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(512), 0, st>>>(p);
 }
 
-static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor of the decode kernel
+template <int KIND, int OUT_DT>
+static void launch_reduce(GemmArgs& p, hipStream_t st) {
+  const int64_t work = (int64_t)p.M * (p.N >> 2);
+  splitk_reduce_kernel<KIND, OUT_DT><<<dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st>>>(p);
+}
 
 template <int KIND, int MI, int OUT_DT>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
   gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits)), dim3(256), 0, st>>>(p);
-  if (p.splits > 1) {
-    const int64_t work = (int64_t)p.M * (p.N >> 2);
-    splitk_reduce_kernel<KIND, OUT_DT><<<dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st>>>(p);
-  }
+  if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
-// Decode path: choose the split-K factor so that a few blocks per CU stream weights
-// concurrently, without letting the partial sums' traffic exceed an eighth of the weight bytes.
+// Decode path: choose the split-K factor so that every CU streams weights.
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = 1;
   p.tiles_n = (p.N + 127) / 128;
   const int nkb = p.K >> 7;
-  int splits = (512 + p.tiles_n / 2) / p.tiles_n;          // aim at two blocks (eight waves) per CU
-  const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;          // at least two K blocks per split
-  // partial sums cost 8 * M * N * splits bytes of traffic against N * K of weights: keep them under an eighth
-  const int by_traffic = (int)(p.K / (64 * (int64_t)p.M)) > 0 ? (int)(p.K / (64 * (int64_t)p.M)) : 1;
+  // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
+  // more blocks only add partial-sum traffic.
+  int splits = 256 / p.tiles_n;
+  const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
   if (splits > by_steps) splits = by_steps;
-  if (splits > by_traffic) splits = by_traffic;
+  if (splits < 1) splits = 1;
   if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
   const int64_t per_split = (int64_t)p.M * p.N * 4;
   if (!p.ws || ws_bytes < per_split * 2) splits = 1;
@@ -858,9 +892,9 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     launch_big<KIND, OUT_DT>(p, st);
     return;
   }
-  if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, st);
-  else if (p.M <= 64) launch_cfg<KIND, 64, 128, 1, 4, OUT_DT>(p, st);
-  else launch_cfg<KIND, 128, 128, 2, 2, OUT_DT>(p, st);
+  if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, ws_bytes, st);
+  else if (p.M <= 64) launch_cfg<KIND, 64, 128, 1, 4, OUT_DT>(p, ws_bytes, st);
+  else launch_cfg<KIND, 128, 128, 2, 2, OUT_DT>(p, ws_bytes, st);
 }
 
 static int gemm_common_checks(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb,

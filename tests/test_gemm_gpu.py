@@ -234,6 +234,30 @@ def test_decode_kernel_split_k(gpu, splits, mnk):
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("mnk", [(100, 384, 1024), (256, 2048, 7168), (130, 136, 2048), (1000, 256, 1536)])
+def test_mid_m_split_k(gpu, splits, mnk):
+    """The 128 x 128 kernel splits K across blocks when its tiles do not fill the chip."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32
+
+    say("mid-M split-K", mnk, "splits", splits)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = sample_rows(m)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+    g = torch.Generator().manual_seed(m)
+    sa = torch.rand((m, 1), generator=g) * 0.05 + 0.01
+    sb = torch.rand((n, 1), generator=g) * 0.001 + 0.0005
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.float16)
+    ref = O.fp8_scaled_mm(xq[rows], wq.t(), sa[rows], sb, torch.float32, bias, acc_dtype=torch.float64)
+    out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.float16, bias.to(gpu))
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+    a8, w8 = rand_i8((m, k), 5), rand_i8((n, k), 6)
+    assert torch.equal(int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()[rows], O.int8_mm_i32(a8[rows], w8.t()))
+
+
 def test_gemm_empty_m(gpu):
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, int8_scaled_mm
 
