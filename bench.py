@@ -122,7 +122,7 @@ def cpu_baseline(m_sample):
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"first {m_sample} of 4096 activation rows of each of the 5 shapes, full weights, {secs:.1f} s of CPU time",
+        "sample": f"{m_sample} of 4096 activation rows of each of the 5 shapes, full weights, one pass, {secs:.1f} s of CPU time",
     }
 
 
@@ -144,13 +144,20 @@ def run_headline(args):
     torch.cuda.synchronize()
 
     def step(tq=None, tg=None):
-        for n, k, x, wq, ws in layers:
+        for li, (n, k, x, wq, ws) in enumerate(layers):
             if tq is None:
                 xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
                 fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
             else:
-                xq, xs = tq.time(lambda: sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True))
-                tg.time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+                xq, xs = tq[li].time(lambda: sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True))
+                tg[li].time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+
+    if args.calibrate_copy:
+        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)  # a plain elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -162,7 +169,7 @@ def run_headline(args):
     wall = time.perf_counter() - t0
 
     # per-kernel durations on the launch stream (separate pass so the events do not perturb the wall clock above)
-    tq, tg = Timer(), Timer()
+    tq, tg = [Timer() for _ in layers], [Timer() for _ in layers]
     for _ in range(args.steps):
         step(tq, tg)
     torch.cuda.synchronize()
@@ -170,8 +177,32 @@ def run_headline(args):
     flops_step = sum(2.0 * m * n * k for n, k, *_ in layers)
     qbytes_step = sum(group_quant_bytes(m, k) for _, k, *_ in layers)
     ms_per_step = wall * 1e3 / args.steps
-    gemm_ms = tg.total_ms() / args.steps
-    quant_ms = tq.total_ms() / args.steps
+    gemm_ms = sum(t.total_ms() for t in tg) / args.steps
+    quant_ms = sum(t.total_ms() for t in tq) / args.steps
+    per_shape = []
+    for (n, k, *_), a, b in zip(layers, tq, tg):
+        qm, gm = a.total_ms() / args.steps, b.total_ms() / args.steps
+        per_shape.append({"N": n, "K": k, "quant_us": round(qm * 1e3, 1),
+                          "quant_GBs": round(group_quant_bytes(m, k) / qm / 1e6, 1),
+                          "gemm_us": round(gm * 1e3, 1), "gemm_TFLOPs": round(2.0 * m * n * k / gm / 1e9, 1)})
+    big = max(range(len(layers)), key=lambda i: layers[i][1])  # the launch with the most activation bytes
+    quant_in_step_gbs = per_shape[big]["quant_GBs"]
+    # the same launch back to back on two alternating inputs: the kernel on its own, without the
+    # write-back of the preceding GEMM's output competing for HBM
+    xs_iso = [layers[big][2], layers[big][2].clone()]
+    iso = Timer()
+    for i in range(2 + 10):
+        if i < 2:
+            sglang_per_token_group_quant_fp8(xs_iso[i % 2], 128, column_major_scales=True)
+        else:
+            iso.time(lambda: sglang_per_token_group_quant_fp8(xs_iso[i % 2], 128, column_major_scales=True))
+    torch.cuda.synchronize()
+    quant_big_gbs = round(group_quant_bytes(m, layers[big][1]) / (iso.total_ms() / iso.count()) / 1e6, 1)
+    del xs_iso
+    traffic = None
+    tfile = ROOT / "profiles" / "headline_traffic.json"
+    if tfile.exists():
+        traffic = json.loads(tfile.read_text()).get("gemm_hbm_bytes_per_launch_avg")
     gemm_tflops = flops_step / (gemm_ms * 1e-3) / 1e12
     quant_gbs = qbytes_step / (quant_ms * 1e-3) / 1e9
     props = torch.cuda.get_device_properties(dev)
@@ -202,20 +233,24 @@ def run_headline(args):
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(gemm_tflops / PEAK_FP8_TFLOPS, 4),
-            "traffic": None,
+            "traffic": traffic,
             "avg_launch_ms": round(gemm_ms / len(layers), 4),
             "flops_per_launch_avg": flops_step / len(layers),
         },
         "quant": {
             "kernel": "sgl_per_token_group_quant_fp8 (group_quant_kernel)",
             "bound": "hbm",
-            "achieved": round(quant_gbs, 1),
+            "launch": f"A[4096,{layers[big][1]}] bf16 -> e4m3fn + fp32 scales (largest of the step)",
+            "achieved": quant_big_gbs,
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
-            "frac": round(quant_gbs / PEAK_HBM_GBS, 4),
-            "avg_launch_ms": round(quant_ms / len(layers), 4),
-            "bytes_per_launch_avg": qbytes_step / len(layers),
+            "frac": round(quant_big_gbs / PEAK_HBM_GBS, 4),
+            "bytes_per_launch": group_quant_bytes(m, layers[big][1]),
+            "measured": "10 back-to-back launches on 2 alternating inputs, events on the launch stream",
+            "same_launch_inside_the_step_GBs": quant_in_step_gbs,
+            "all_launches_inside_the_step_GBs": round(quant_gbs, 1),
         },
+        "per_shape": per_shape,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
     }
@@ -354,7 +389,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-rows", type=int, default=256, help="activation rows in the CPU-baseline sample")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="activation rows in the CPU-baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (reference point for the rocprofv3 byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
     ap.add_argument("--iters", type=int, default=20)
