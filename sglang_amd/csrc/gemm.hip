@@ -53,6 +53,8 @@ struct GemmArgs {
 // s_waitcnt immediate: wait until at most `vm` vector-memory loads are outstanding
 // and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
 constexpr int waitcnt_vm_lgkm0(int vm) { return (vm & 0xf) | (((vm >> 4) & 3) << 14) | (7 << 4); }
+// ... and one that waits for LDS / scalar-memory operations only
+constexpr int waitcnt_lgkm0_only() { return 0xf | (3 << 14) | (7 << 4); }
 
 // Global -> LDS copies written as assembly (16 or 4 bytes per lane; lane l lands at
 // lds_dst + l * size).  The decode kernel keeps several stages of such copies in flight and
@@ -180,16 +182,18 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
   }
 }
 
-// Epilogue of the 256 x 256 kernel for 16-bit outputs: every wave converts its
-// accumulators (scales and bias applied) and drops them into a 256 x 512-byte image of
-// the C tile in LDS, then the block writes the image out in rows, 16 bytes per lane, so
-// that a wavefront store covers two full 512-byte row segments instead of sixteen
-// 32-byte pieces.  Chunk c (16 bytes) of row r sits at chunk position c ^ (r & 31).
-// The caller guarantees that nobody reads the stage buffers any more.
+// Epilogue of the 256 x 256 kernel for 16-bit outputs, in two halves of 128 rows: the
+// waves that own the half convert their accumulators (scales and bias applied) and drop
+// them into a 128 x 512-byte image in one stage buffer, then all eight waves write the
+// image out in rows, 16 bytes per lane, so that a wavefront store covers two full 512-byte
+// row segments instead of sixteen 32-byte pieces.  Chunk c (16 bytes) of row r sits at
+// chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
+// next tile's first K block.  The caller has made sure nobody reads `img` any more; on
+// return every wave has passed a barrier after its last read of `img`.
 template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
-SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* smem, int m0, int n0, int wm, int wn,
+SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, int m0, int n0, int wm, int wn,
                                int r16, int g, int lane, int wave) {
-  constexpr int TM = MI * 16, TN = NI * 16;
+  constexpr int TN = NI * 16;
   float bv[NI][4], sbv[NI][4];
   if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
 #pragma unroll
@@ -208,49 +212,60 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* sm
       }
     }
   }
-#pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int ml = wm * TM + i * 16 + r16;
-    float sam = 1.f;
-    if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) sam = (m0 + ml < p.M) ? p.sa[m0 + ml] : 0.f;
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      float o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[j][e] * sam, bv[j][e]);
-        else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam, sbv[j][e] * acc[i][j][e], bv[j][e]);
-        else o[e] = acc[i][j][e];
-      }
-      const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
-      char* dst = smem + ml * 512 + ((chunk ^ (ml & 31)) * 16) + (g & 1) * 8;
-      if constexpr (OUT_DT == SGLQ_BF16) {
-        typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
-        *reinterpret_cast<bf4*>(dst) = bf4{(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
-      } else {
-        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-        *reinterpret_cast<h4*>(dst) = h4{(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
-      }
-    }
-  }
-  __syncthreads();
-  // 256 rows, 8 waves: wave w writes rows 32 w .. 32 w + 31, two rows per store instruction
   const int c = lane & 31;
   const int n = n0 + c * 8;
   char* out = reinterpret_cast<char*>(p.out);
-#pragma unroll 4
-  for (int it = 0; it < 16; ++it) {
-    const int ml = wave * 32 + it * 2 + (lane >> 5);
-    const int m = m0 + ml;
-    const v4i v = *reinterpret_cast<const v4i*>(smem + ml * 512 + ((c ^ (ml & 31)) * 16));
-    if (m < p.M) {
-      char* row = out + ((int64_t)m * p.ldo + n) * 2;
-      if (n + 8 <= p.N) {
-        *reinterpret_cast<v4i*>(row) = v;
-      } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
-        *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[0], (uint32_t)v[1]};
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    if (wm == half) {  // wave-uniform
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int ml = i * 16 + r16;  // row inside the half
+        float sam = 1.f;
+        if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
+          const int m = m0 + half * 128 + ml;
+          sam = (m < p.M) ? p.sa[m] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          float o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[j][e] * sam, bv[j][e]);
+            else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam, sbv[j][e] * acc[i][j][e], bv[j][e]);
+            else o[e] = acc[i][j][e];
+          }
+          const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
+          char* dst = img + ml * 512 + ((chunk ^ (ml & 31)) * 16) + (g & 1) * 8;
+          if constexpr (OUT_DT == SGLQ_BF16) {
+            typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+            *reinterpret_cast<bf4*>(dst) = bf4{(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
+          } else {
+            typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+            *reinterpret_cast<h4*>(dst) = h4{(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
+          }
+        }
       }
     }
+    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
+    __builtin_amdgcn_s_barrier();
+    // 128 rows, 8 waves: wave w writes rows 16 w .. 16 w + 15, two rows per store instruction
+#pragma unroll 4
+    for (int it = 0; it < 8; ++it) {
+      const int ml = wave * 16 + it * 2 + (lane >> 5);
+      const int m = m0 + half * 128 + ml;
+      const v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
+      if (m < p.M) {
+        char* row = out + ((int64_t)m * p.ldo + n) * 2;
+        if (n + 8 <= p.N) {
+          *reinterpret_cast<v4i*>(row) = v;
+        } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
+          *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[0], (uint32_t)v[1]};
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());  // my reads of the image are complete
+    __builtin_amdgcn_s_barrier();
   }
 }
 
@@ -430,6 +445,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   constexpr int STAGE_BYTES = (BM + BN) * 128;
   constexpr int NLOAD = (BM + BN) / 8 / NW;  // 8 one-KiB copies per wave per stage: 4 of A, 4 of B
   constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
 
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
 
@@ -437,10 +453,6 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int r16 = lane & 15, g = lane >> 4;
-
-  int tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
 
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
@@ -453,8 +465,8 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   // scalar operand (K is a multiple of 128 for this kernel).
   const int l8 = lane >> 3;
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
-  const uint32_t off_a = (uint32_t)(m0 + wave * 8 + l8) * p.lda + c16;
-  const uint32_t off_b = (uint32_t)(n0 + wave * 8 + l8) * p.ldb + c16;
+  const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
+  uint32_t off_a = 0, off_b = 0;  // of the tile whose copies are being issued
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
   auto issue_load = [&](int j, int stage, int k0) {
     const bool is_a = j < NLOAD / 2;
@@ -470,67 +482,60 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   const int lane_off1 = lane_off0 ^ 16;
   const int a_base = (wm * TM) * 128;
   const int b_base = (BM + wn * TN) * 128;
-
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
-  acc_t acc[MI][NI];
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
-
-  // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].
-  // A lane owns row r16 of each of the wave's 16-row fragments; rows past M read
-  // as zero through the buffer's extent (they are never stored).
-  const int nkb = p.K >> 7;
-  float sfa_cur[MI];
-  float sfb_cur = 0.f, sfb_next = 0.f;
-  __amdgpu_buffer_rsrc_t rs = ra;
-  uint32_t sfa_off = 0;
-  int sfa_frag = 0, sfa_step = 0, nb = 0;
-  if constexpr (KIND == KIND_FP8_BLOCK) {
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
-    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
-    const int nblocks = (p.N + 127) >> 7;
-    nb = (n0 + wn * TN) >> 7;
-    if (nb >= nblocks) nb = nblocks - 1;
-    nb = __builtin_amdgcn_readfirstlane(nb);
-    const int mrow = m0 + wm * TM + r16;
-    // a row past M must not alias a valid element of another K block: send it out of range
-    sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
-    sfa_frag = (int)(16 * p.sa_stride_m * 4);
-    sfa_step = (int)(p.sa_stride_k * 4);
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      const bool ok = mrow + i * 16 < p.M;
-      sfa_cur[i] = __builtin_bit_cast(
-          float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok ? sfa_off + i * sfa_frag : OOB, 0, 0));
-    }
-    sfb_cur = p.sb[nb * p.sb_stride_n];
-  }
-  // validity of fragment i's row for the scale prefetch, as a bit mask
-  uint32_t sfa_ok = 0;
-  if constexpr (KIND == KIND_FP8_BLOCK) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i) sfa_ok |= (m0 + wm * TM + r16 + i * 16 < p.M ? 1u : 0u) << i;
-  }
-
   auto read_frag = [&](const char* q) -> v8i {
     v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
     v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-#pragma unroll
-  for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
-  __builtin_amdgcn_s_waitcnt(0);
-  __builtin_amdgcn_s_barrier();
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
 
-  // One K step.  more_tag = another step follows: its copies and scales are issued here,
-  // in the shadow of the MFMAs, so that no wave spends issue slots on them while the
-  // MFMA pipe is idle.
-  auto k_step = [&](int kb, auto more_tag) {
-    constexpr bool more = decltype(more_tag)::value;
-    const int cur = kb & 1;
+  // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].
+  // A lane owns row r16 of each of the wave's 16-row fragments; rows past M read
+  // as zero through the out-of-range offset (they are never stored).
+  const int nkb = p.K >> 7;
+  float sfa_cur[MI];
+  float sfb_cur = 0.f, sfb_next = 0.f;
+  __amdgpu_buffer_rsrc_t rs = ra;
+  uint32_t sfa_off = 0, sfa_ok = 0;
+  int sfa_frag = 0, sfa_step = 0, nb = 0;
+  if constexpr (BLOCK) {
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    sfa_frag = (int)(16 * p.sa_stride_m * 4);
+    sfa_step = (int)(p.sa_stride_k * 4);
+  }
+  // Addressing of the tile whose copies and scales are issued from now on.
+  auto set_tile = [&](int m0, int n0) {
+    off_a = (uint32_t)(m0 + row_in_tile) * p.lda + c16;
+    off_b = (uint32_t)(n0 + row_in_tile) * p.ldb + c16;
+    if constexpr (BLOCK) {
+      const int nblocks = (p.N + 127) >> 7;
+      nb = (n0 + wn * TN) >> 7;
+      if (nb >= nblocks) nb = nblocks - 1;
+      nb = __builtin_amdgcn_readfirstlane(nb);
+      const int mrow = m0 + wm * TM + r16;
+      // a row past M must not alias a valid element of another K block: send it out of range
+      sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
+      sfa_ok = 0;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sfa_ok |= (mrow + i * 16 < p.M ? 1u : 0u) << i;
+    }
+  };
+  auto load_sfa = [&](int i, int kb) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
+  };
+
+  // One K step on stage `cur`.  With a `pre_tag`, the copies (into the other stage) and the
+  // scales of K block `kn` of the tile that set_tile named last are issued here, in the
+  // shadow of the MFMAs, so that no wave spends issue slots on them while the MFMA pipe is
+  // idle: that is the next K block of this tile, or, in a tile's last step (`last_tag`),
+  // the first K block of the block's next tile.
+  auto k_step = [&](int cur, int kn, auto pre_tag, auto last_tag) {
+    constexpr bool pre = decltype(pre_tag)::value;
+    constexpr bool last = decltype(last_tag)::value;
     const char* st = smem + cur * STAGE_BYTES;
     v8i bf[NI];
     bf[0] = read_frag(st + b_base);
@@ -544,19 +549,19 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       v8i a_nxt = a_cur;
-      if constexpr (KIND == KIND_FP8_BLOCK) {
+      if constexpr (BLOCK) {
         sc_prev = sc;
         sc = sfa_cur[i] * sfb_cur;
       }
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
         const int idx = i * NI + j;
-        if constexpr (KIND == KIND_FP8_BLOCK) {
+        if constexpr (BLOCK) {
           const v4f z = {0.f, 0.f, 0.f, 0.f};
           v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, z, 0, 0, 0, 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
           if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
-          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
             const float s_use = (pi == i) ? sc : sc_prev;
@@ -565,72 +570,113 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
             acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
             acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
           }
-          if (more && idx == NLOAD) sfb_next = p.sb[(kb + 1) * p.sb_stride_k + nb * p.sb_stride_n];
+          if (pre && idx == NLOAD) sfb_next = p.sb[kn * p.sb_stride_k + nb * p.sb_stride_n];
           // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
-          if (more && j == 1 && i >= 1)
-            sfa_cur[i - 1] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rs, ((sfa_ok >> (i - 1)) & 1) ? sfa_off + (i - 1) * sfa_frag : OOB,
-                                                            (kb + 1) * sfa_step, 0));
+          if (pre && j == 1 && i >= 1) sfa_cur[i - 1] = load_sfa(i - 1, kn);
           part_prev = part;
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, acc[i][j], 0, 0, 0, 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
           if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
-          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
         } else {
           const v4i b0 = {bf[j][0], bf[j][1], bf[j][2], bf[j][3]}, b1 = {bf[j][4], bf[j][5], bf[j][6], bf[j][7]};
           const v4i a0 = {a_cur[0], a_cur[1], a_cur[2], a_cur[3]}, a1 = {a_cur[4], a_cur[5], a_cur[6], a_cur[7]};
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
           if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
-          if (more && idx < NLOAD) issue_load(idx, cur ^ 1, (kb + 1) * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
       a_cur = a_nxt;
     }
-    if constexpr (KIND == KIND_FP8_BLOCK) {
+    if constexpr (BLOCK) {
       acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
       acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
       acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
-      if constexpr (more) {
-        sfa_cur[MI - 1] = __builtin_bit_cast(
-            float, __builtin_amdgcn_raw_buffer_load_b32(rs, ((sfa_ok >> (MI - 1)) & 1) ? sfa_off + (MI - 1) * sfa_frag : OOB,
-                                                        (kb + 1) * sfa_step, 0));
+      if constexpr (pre) {
+        sfa_cur[MI - 1] = load_sfa(MI - 1, kn);
         sfb_cur = sfb_next;
       }
     }
-    if constexpr (more) {
-      // The next stage's copies were the first eight vector-memory loads of this step
-      // and loads retire in order, so it is enough to wait until at most the
-      // SCALE_LOADS_AFTER_COPIES younger ones (activation-scale refills, none for the
-      // other kinds) are still in flight; lgkmcnt(0) covers this wave's LDS reads of the
-      // stage that the next step overwrites.  A bare s_barrier: the waits above are
-      // the only ordering needed, a fence would drain the scale refills as well.
-      constexpr int SCALE_LOADS_AFTER_COPIES = (KIND == KIND_FP8_BLOCK) ? MI - 1 : 0;
+    if constexpr (!last) {
+      // The next stage's copies were the first eight vector-memory loads of this step and
+      // vector-memory operations retire in order, so it is enough to wait until at most the
+      // SCALE_LOADS_AFTER_COPIES younger ones (activation-scale refills, none for the other
+      // kinds) are still in flight; lgkmcnt(0) covers this wave's LDS reads of the stage
+      // that the next step overwrites.  A bare s_barrier: the waits above are the only
+      // ordering needed, a fence would drain the scale refills as well.
+      constexpr int SCALE_LOADS_AFTER_COPIES = BLOCK ? MI - 1 : 0;
       __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(SCALE_LOADS_AFTER_COPIES));
+      __builtin_amdgcn_s_barrier();
+    } else {
+      // Last K block of a tile: wait for everything, so that the epilogue's stores are the
+      // only vector-memory operations in flight when the next tile starts.  After the
+      // barrier the next tile's first K block is visible to every wave and nobody reads
+      // this stage any more (it becomes the epilogue's staging buffer).
+      __builtin_amdgcn_s_waitcnt(0);
       __builtin_amdgcn_s_barrier();
     }
   };
-  for (int kb = 0; kb + 1 < nkb; ++kb) k_step(kb, std::true_type{});
-  k_step(nkb - 1, std::false_type{});
 
-  if constexpr (KIND == KIND_I8_RAW) {
-    epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
-  } else {
-    // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
-    const bool aligned = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-    if (aligned) {
-      __syncthreads();  // every wave is done with the last stage: the buffers become the C image
-      epilogue_via_lds<KIND, OUT_DT, MI, NI>(p, acc, smem, m0, n0, wm, wn, r16, g, lane, wave);
+  // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
+  const int total = p.tiles_m * p.tiles_n;
+  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+  int tile = blockIdx.x;
+  int tm, tn;
+  tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+  int m0 = tm * BM, n0 = tn * BN;
+  int par = 0;  // stage that holds K block 0 of the current tile
+
+  set_tile(m0, n0);
+#pragma unroll
+  for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
+  if constexpr (BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
+    sfb_cur = p.sb[nb * p.sb_stride_n];
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
+
+  while (true) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+    for (int kb = 0; kb + 1 < nkb; ++kb) k_step((kb + par) & 1, kb + 1, std::true_type{}, std::false_type{});
+
+    const int next_tile = tile + (int)gridDim.x;
+    const bool has_next = next_tile < total;
+    const int last_stage = (nkb - 1 + par) & 1;
+    const int cm0 = m0, cn0 = n0;
+    // The tile's last step always prefetches: past the block's last tile it is pointed at
+    // rows beyond M and N, which the buffer bounds turn into zero fill without memory traffic.
+    tile_of_block(has_next ? next_tile : 0, p.tiles_m, p.tiles_n, tm, tn);
+    m0 = has_next ? tm * BM : p.tiles_m * BM;
+    n0 = has_next ? tn * BN : p.tiles_n * BN;
+    set_tile(m0, n0);  // the current tile issues no more copies or scale loads
+    k_step(last_stage, 0, std::true_type{}, std::true_type{});
+
+    if constexpr (KIND == KIND_I8_RAW) {
+      epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
     } else {
-      epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
+      if (aligned_out)
+        epilogue_via_lds<KIND, OUT_DT, MI, NI>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g, lane,
+                                               wave);
+      else
+        epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
     }
+    if (!has_next) break;
+    tile = next_tile;
+    par = last_stage ^ 1;
   }
 }
-
 
 // ---------------------------------------------------------------------------
 // Decode kernel (M <= 64): the weight matrix is streamed once from HBM, so the
@@ -802,6 +848,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------
 static bool g_use_dma = true;
 
+// Compute units of the current device (cached; a multiple of 8 keeps the persistent
+// kernel's tile walk on one XCD per block).
+static int num_cus() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached = n >= 8 ? (n / 8) * 8 : n;
+  }
+  return cached;
+}
+
 static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
 
 template <int KIND, int OUT_DT>
@@ -843,7 +901,10 @@ static void launch_big(GemmArgs& p, hipStream_t st) {
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 255) / 256;
   p.splits = 1;
-  gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(512), 0, st>>>(p);
+  // persistent: one block per CU walks the tiles blockIdx, blockIdx + gridDim, ...
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int blocks = tiles < num_cus() ? tiles : num_cus();
+  gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
 }
 
 template <int KIND, int OUT_DT>
@@ -888,7 +949,11 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
-  if ((p.K & 127) == 0 && (g_force_tile == 256 || (g_force_tile == 0 && g_use_dma && p.M > 1024))) {
+  // Measured crossover: the 256 x 256 kernel wins once its tiles cover more than half of
+  // the 256 CUs (e.g. 144 tiles at M = 4096, N = 2112; 192 at M = 512, N = 24576); with
+  // fewer tiles the 128 x 128 kernel with split-K keeps more CUs busy.
+  const int big_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
+  if ((p.K & 127) == 0 && (g_force_tile == 256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && big_tiles >= 140))) {
     launch_big<KIND, OUT_DT>(p, st);
     return;
   }
