@@ -182,7 +182,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
   }
 }
 
-// Epilogue of the 256 x 256 kernel for 16-bit outputs, in two halves of 128 rows: the
+// Epilogue of the 256-row kernels for 16-bit outputs, in two halves of 128 rows: the
 // waves that own the half convert their accumulators (scales and bias applied) and drop
 // them into a 128 x 512-byte image in one stage buffer, then all eight waves write the
 // image out in rows, 16 bytes per lane, so that a wavefront store covers two full 512-byte
@@ -190,7 +190,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 // chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
-template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
+template <int KIND, int OUT_DT, int MI, int NI, int BN, typename acc_t>
 SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, int m0, int n0, int wm, int wn,
                                int r16, int g, int lane, int wave) {
   constexpr int TN = NI * 16;
@@ -217,10 +217,10 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   char* out = reinterpret_cast<char*>(p.out);
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    if (wm == half) {  // wave-uniform
+    if (((wm * MI * 16) >> 7) == half) {  // wave-uniform: a wave's rows lie in one half
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        const int ml = i * 16 + r16;  // row inside the half
+        const int ml = ((wm * MI * 16) & 127) + i * 16 + r16;  // row inside the half
         float sam = 1.f;
         if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
           const int m = m0 + half * 128 + ml;
@@ -255,7 +255,7 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
       const int ml = wave * 16 + it * 2 + (lane >> 5);
       const int m = m0 + half * 128 + ml;
       const v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
-      if (m < p.M) {
+      if (m < p.M && c * 8 < BN) {
         char* row = out + ((int64_t)m * p.ldo + n) * 2;
         if (n + 8 <= p.N) {
           *reinterpret_cast<v4i*>(row) = v;
@@ -667,8 +667,272 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g, lane,
                                                wave);
+      else
+        epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+    }
+    if (!has_next) break;
+    tile = next_tile;
+    par = last_stage ^ 1;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 256 x (32 NI) kernel, NI = 6, 7 or 8 (tile widths 192, 224, 256): the same
+// persistent, two-stage structure as the 256 x 256 kernel with the roles of the
+// operands exchanged.  The eight waves form a 4 (M) x 2 (N) grid; a wave keeps its
+// four activation fragments of the K step in registers and streams its NI weight
+// fragments one ahead.  The tile width is chosen on the host so that the tile count
+// fills whole rounds of the chip's CUs: 7168 columns are 32 tiles of 224 (two full
+// rounds at M = 4096) instead of 28 tiles of 256 (one full round and a 3/4 one).
+// A wave's columns can straddle two 128-column scale blocks, so the weight scale is
+// selected per fragment.
+// ---------------------------------------------------------------------------
+template <int KIND, int OUT_DT, int NI>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
+  constexpr int BM = 256, NW = 8, WAVES_N = 2, MI = 4;
+  constexpr int TM = MI * 16, TN = NI * 16, BN = WAVES_N * TN;
+  constexpr int STAGE_BYTES = 512 * 128;  // stage pitch; only (BM + BN) rows are filled
+  constexpr int NCOPY = (BM + BN) / 8;    // one-KiB copies per stage: 32 of A, BN / 8 of B
+  constexpr int NLOAD = (NCOPY + NW - 1) / NW;
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
+
+  // Copy j of this wave is copy c = wave + 8 j of the stage and fills stage rows 8 c .. 8 c + 7
+  // (c < 32: activation rows, else weight rows); lane l brings row l / 8 of those, chunk
+  // (l % 8) ^ swz(row).  swz depends on l / 8 and the parity of the wave only, so all A copies
+  // (and all B copies) of a wave share one per-lane offset and differ by a multiple of 64 rows.
+  // Rows past M / N fall beyond the buffer's extent and read as zero; the K offset travels in
+  // the scalar operand (K is a multiple of 128 for this kernel).
+  const int l8 = lane >> 3;
+  const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
+  const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
+  uint32_t off_a = 0, off_b = 0;  // of the tile whose copies are being issued
+  const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
+  auto issue_load = [&](int j, int stage, int k0) {
+    const bool is_a = j < 4;
+    const int c = wave + j * NW;
+    if (c >= NCOPY) return;  // wave-uniform; only the last copy of a 224-wide tile
+    char* dst = smem + stage * STAGE_BYTES + c * 1024;
+    const uint32_t off = is_a ? off_a + (uint32_t)j * step_a : off_b + (uint32_t)(j - 4) * step_b;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(is_a ? ra : rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0,
+                                             0, 0);
+  };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  const int a_base = (wm * TM) * 128;
+  const int b_base = (BM + wn * TN) * 128;
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
+
+  // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].  A lane owns
+  // row r16 of each of the wave's 16-row activation fragments.  The wave's weight fragments
+  // 0 .. jsw - 1 lie in scale block nb_lo, the others in nb_lo + 1.
+  const int nkb = p.K >> 7;
+  float sfa_cur[MI], sfa_nxt[MI];
+  float sfb_lo = 0.f, sfb_hi = 0.f, sfb_lo_nxt = 0.f, sfb_hi_nxt = 0.f;
+  __amdgpu_buffer_rsrc_t rs = ra;
+  uint32_t sfa_off = 0, sfa_ok = 0;
+  int sfa_frag = 0, sfa_step = 0, nb_lo = 0, nb_hi = 0, jsw = NI, jsw_nxt = NI;
+  if constexpr (BLOCK) {
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    sfa_frag = (int)(16 * p.sa_stride_m * 4);
+    sfa_step = (int)(p.sa_stride_k * 4);
+  }
+  // Addressing of the tile whose copies and scales are issued from now on.
+  auto set_tile = [&](int m0, int n0) {
+    off_a = (uint32_t)(m0 + row_in_tile) * p.lda + c16;
+    off_b = (uint32_t)(n0 + row_in_tile) * p.ldb + c16;
+    if constexpr (BLOCK) {
+      const int nblocks = (p.N + 127) >> 7;
+      const int nw = n0 + wn * TN;
+      nb_lo = nw >> 7;
+      jsw_nxt = ((nb_lo + 1) * 128 - nw) >> 4;
+      nb_hi = nb_lo + 1;
+      if (nb_lo >= nblocks) nb_lo = nblocks - 1;
+      if (nb_hi >= nblocks) nb_hi = nblocks - 1;
+      nb_lo = __builtin_amdgcn_readfirstlane(nb_lo);
+      nb_hi = __builtin_amdgcn_readfirstlane(nb_hi);
+      jsw_nxt = __builtin_amdgcn_readfirstlane(jsw_nxt);
+      const int mrow = m0 + wm * TM + r16;
+      // a row past M must not alias a valid element of another K block: send it out of range
+      sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
+      sfa_ok = 0;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sfa_ok |= (mrow + i * 16 < p.M ? 1u : 0u) << i;
+    }
+  };
+  auto load_sfa = [&](int i, int kb) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
+  };
+
+  // One K step on stage `cur`.  With a `pre_tag`, the copies (into the other stage) and the
+  // scales of K block `kn` of the tile that set_tile named last are issued here, in the
+  // shadow of the MFMAs: that is the next K block of this tile, or, in a tile's last step
+  // (`last_tag`), the first K block of the block's next tile.
+  auto k_step = [&](int cur, int kn, auto pre_tag, auto last_tag) {
+    constexpr bool pre = decltype(pre_tag)::value;
+    constexpr bool last = decltype(last_tag)::value;
+    const char* st = smem + cur * STAGE_BYTES;
+    v8i af[MI];
+    af[0] = read_frag(st + a_base);
+    v8i b_cur = read_frag(st + b_base);
+#pragma unroll
+    for (int i = 1; i < MI; ++i) af[i] = read_frag(st + a_base + i * 16 * 128);
+    float sc = 0.f, sc_prev = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4f part_prev = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      v8i b_nxt = b_cur;
+      float sfb_j = 0.f;
+      if constexpr (BLOCK) sfb_j = j < jsw ? sfb_lo : sfb_hi;  // wave-uniform
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int idx = j * MI + i;
+        if constexpr (BLOCK) {
+          const v4f z = {0.f, 0.f, 0.f, 0.f};
+          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], z, 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
+          sc_prev = sc;
+          sc = sfa_cur[i] * sfb_j;
+          if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
+            const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
+            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], sc_prev, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], sc_prev, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], sc_prev, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], sc_prev, acc[pi][pj][3]);
+          }
+          if (pre && idx == NLOAD) {
+            sfb_lo_nxt = p.sb[kn * p.sb_stride_k + nb_lo * p.sb_stride_n];
+            sfb_hi_nxt = p.sb[kn * p.sb_stride_k + nb_hi * p.sb_stride_n];
+          }
+          if (pre && idx >= NLOAD && idx < NLOAD + MI) sfa_nxt[idx - NLOAD] = load_sfa(idx - NLOAD, kn);
+          part_prev = part;
+        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
+        } else {
+          const v4i b0 = {b_cur[0], b_cur[1], b_cur[2], b_cur[3]}, b1 = {b_cur[4], b_cur[5], b_cur[6], b_cur[7]};
+          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]}, a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
+          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      b_cur = b_nxt;
+    }
+    if constexpr (BLOCK) {
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+      if constexpr (pre) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) sfa_cur[i] = sfa_nxt[i];
+        sfb_lo = sfb_lo_nxt;
+        sfb_hi = sfb_hi_nxt;
+        jsw = jsw_nxt;
+      }
+    }
+    if constexpr (!last) {
+      // The next stage's copies were the first vector-memory loads of this step and
+      // vector-memory operations retire in order, so it is enough to wait until at most the
+      // SCALE_LOADS_AFTER_COPIES younger ones (activation-scale loads, none for the other
+      // kinds) are still in flight; lgkmcnt(0) covers this wave's LDS reads of the stage
+      // that the next step overwrites.  A bare s_barrier: the waits above are the only
+      // ordering needed, a fence would drain the scale loads as well.
+      constexpr int SCALE_LOADS_AFTER_COPIES = BLOCK ? MI : 0;
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(SCALE_LOADS_AFTER_COPIES));
+      __builtin_amdgcn_s_barrier();
+    } else {
+      // Last K block of a tile: wait for everything, so that the epilogue's stores are the
+      // only vector-memory operations in flight when the next tile starts.  After the
+      // barrier the next tile's first K block is visible to every wave and nobody reads
+      // this stage any more (it becomes the epilogue's staging buffer).
+      __builtin_amdgcn_s_waitcnt(0);
+      __builtin_amdgcn_s_barrier();
+    }
+  };
+
+  // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
+  const int total = p.tiles_m * p.tiles_n;
+  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+  int tile = blockIdx.x;
+  int tm, tn;
+  tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+  int m0 = tm * BM, n0 = tn * BN;
+  int par = 0;  // stage that holds K block 0 of the current tile
+
+  set_tile(m0, n0);
+#pragma unroll
+  for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
+  if constexpr (BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
+    sfb_lo = p.sb[nb_lo * p.sb_stride_n];
+    sfb_hi = p.sb[nb_hi * p.sb_stride_n];
+    jsw = jsw_nxt;
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
+
+  while (true) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+    for (int kb = 0; kb + 1 < nkb; ++kb) k_step((kb + par) & 1, kb + 1, std::true_type{}, std::false_type{});
+
+    const int next_tile = tile + (int)gridDim.x;
+    const bool has_next = next_tile < total;
+    const int last_stage = (nkb - 1 + par) & 1;
+    const int cm0 = m0, cn0 = n0;
+    // The tile's last step always prefetches: past the block's last tile it is pointed at
+    // rows beyond M and N, which the buffer bounds turn into zero fill without memory traffic.
+    tile_of_block(has_next ? next_tile : 0, p.tiles_m, p.tiles_n, tm, tn);
+    m0 = has_next ? tm * BM : p.tiles_m * BM;
+    n0 = has_next ? tn * BN : p.tiles_n * BN;
+    set_tile(m0, n0);  // the current tile issues no more copies or scale loads
+    k_step(last_stage, 0, std::true_type{}, std::true_type{});
+
+    if constexpr (KIND == KIND_I8_RAW) {
+      epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+    } else {
+      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
+      if (aligned_out)
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g,
+                                                   lane, wave);
       else
         epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
     }
@@ -894,7 +1158,9 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   if (splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
-static int g_force_tile = 0;  // test hook: 0 = heuristic, 128 = always the 128x128 kernel, 256 = always 256x256
+// test hook: 0 = heuristic, 64 = the M <= 64 kernel where it applies, 128 = the 128 x 128 kernel,
+// 256 = the 256 x 256 kernel, 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide
+static int g_force_tile = 0;
 
 template <int KIND, int OUT_DT>
 static void launch_big(GemmArgs& p, hipStream_t st) {
@@ -905,6 +1171,34 @@ static void launch_big(GemmArgs& p, hipStream_t st) {
   const int tiles = p.tiles_m * p.tiles_n;
   const int blocks = tiles < num_cus() ? tiles : num_cus();
   gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+}
+
+template <int KIND, int OUT_DT, int NI>
+static void launch_wide(GemmArgs& p, hipStream_t st) {
+  p.tiles_m = (p.M + 255) / 256;
+  p.tiles_n = (p.N + 32 * NI - 1) / (32 * NI);
+  p.splits = 1;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int blocks = tiles < num_cus() ? tiles : num_cus();
+  gemm_wide_kernel<KIND, OUT_DT, NI><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+}
+
+// Tile width of the 256-row kernels.  Every CU works through ceil(tiles / CUs) tiles, each
+// costing in proportion to its width: take the width with the least rounds x width (7168
+// columns at M = 4096: 2 x 224 against 2 x 256; 2112 columns: 1 x 192 against 1 x 256).
+static int pick_tile_width(const GemmArgs& p) {
+  const int tiles_m = (p.M + 255) / 256;
+  int best = 256;
+  int64_t best_cost = 0;
+  for (int bn = 256; bn >= 192; bn -= 32) {
+    const int tiles = tiles_m * ((p.N + bn - 1) / bn);
+    const int64_t cost = (int64_t)((tiles + num_cus() - 1) / num_cus()) * bn;
+    if (bn == 256 || cost < best_cost) {
+      best = bn;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 template <int KIND, int OUT_DT>
@@ -953,8 +1247,13 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // the 256 CUs (e.g. 144 tiles at M = 4096, N = 2112; 192 at M = 512, N = 24576); with
   // fewer tiles the 128 x 128 kernel with split-K keeps more CUs busy.
   const int big_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
-  if ((p.K & 127) == 0 && (g_force_tile == 256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && big_tiles >= 140))) {
-    launch_big<KIND, OUT_DT>(p, st);
+  const bool forced_256 = g_force_tile == 256 || g_force_tile == 192 || g_force_tile == 224 || g_force_tile == 257;
+  if ((p.K & 127) == 0 && (forced_256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && big_tiles >= 140))) {
+    const int width = g_force_tile == 0 ? pick_tile_width(p) : g_force_tile;
+    if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
+    else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
+    else if (width == 257) launch_wide<KIND, OUT_DT, 8>(p, st);
+    else launch_big<KIND, OUT_DT>(p, st);
     return;
   }
   if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, ws_bytes, st);

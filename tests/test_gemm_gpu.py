@@ -37,7 +37,8 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
-@pytest.fixture(params=[0, 128, 256], ids=["tile_auto", "tile128", "tile256"])  # tile_auto sends M <= 64 to the decode kernel
+# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide)
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257], ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -51,7 +52,7 @@ def tile(request):
 def test_int8_accumulators_bit_exact(gpu, load_path, tile, mnk):
     from sglang_amd.sgl_kernel import int8_mm_i32
 
-    if tile == 256 and not load_path:
+    if tile >= 192 and not load_path:
         pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
     say("int8 acc", mnk, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
@@ -103,7 +104,7 @@ def make_block_case(m, n, k, seed, outliers=False):
 def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
-    if tile == 256 and not load_path:
+    if tile >= 192 and not load_path:
         pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
     say("fp8_blockwise", mnk, out_dtype, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
