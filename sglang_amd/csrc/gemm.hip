@@ -679,25 +679,30 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------
-// 256 x (32 NI) kernel, NI = 6, 7 or 8 (tile widths 192, 224, 256): the same
-// persistent, two-stage structure as the 256 x 256 kernel with the roles of the
-// operands exchanged.  The eight waves form a 4 (M) x 2 (N) grid; a wave keeps its
-// four activation fragments of the K step in registers and streams its NI weight
-// fragments one ahead.  The tile width is chosen on the host so that the tile count
-// fills whole rounds of the chip's CUs: 7168 columns are 32 tiles of 224 (two full
-// rounds at M = 4096) instead of 28 tiles of 256 (one full round and a 3/4 one).
-// A wave's columns can straddle two 128-column scale blocks, so the weight scale is
-// selected per fragment.
+// 256 x 256 kernel, software-pipelined across K steps (K >= 384).  Same tile, wave grid
+// and LDS layout as gemm_big_kernel; what differs is where the step barrier sits and what
+// is in registers when a step starts:
+//   * the barrier of step u comes before its last activation fragment's four MFMAs (MFMA
+//     28 of 32).  By then every wave has issued and completed all its LDS reads of step
+//     u's stage, and the copies of K block u + 1 have landed in the other stage.
+//   * behind MFMAs 28..31 a wave reads the first fragments of block u + 1 (each weight
+//     fragment right after its last use, plus the first activation fragment) and issues
+//     the four activation copies of block u + 2 into the stage that just became free; the
+//     four weight copies of block u + 2 follow behind MFMAs 0..3 of step u + 1.
+// So a step starts with its operands in registers and four MFMAs queued behind the
+// barrier, instead of every wave waiting for ten LDS reads right after it.  The sequence
+// of blocks runs across tile boundaries (the block's next tile follows the last K block
+// of the current one); only the activation copies behind the last step of a tile are
+// deferred to the next tile's first step, because the freed stage stages the C tile.
 // ---------------------------------------------------------------------------
-template <int KIND, int OUT_DT, int NI>
-__global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
-  constexpr int BM = 256, NW = 8, WAVES_N = 2, MI = 4;
-  constexpr int TM = MI * 16, TN = NI * 16, BN = WAVES_N * TN;
-  constexpr int STAGE_BYTES = 512 * 128;  // stage pitch; only (BM + BN) rows are filled
-  constexpr int NCOPY = (BM + BN) / 8;    // one-KiB copies per stage: 32 of A, BN / 8 of B
-  constexpr int NLOAD = (NCOPY + NW - 1) / NW;
+template <int KIND, int OUT_DT>
+__global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
+  constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
+  constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
+  constexpr int STAGE_BYTES = (BM + BN) * 128;
   constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
   constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  static_assert(NI == 4 && MI == 8, "the copy schedule below is written for 4 x 8 fragments");
 
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
 
@@ -709,26 +714,32 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
 
-  // Copy j of this wave is copy c = wave + 8 j of the stage and fills stage rows 8 c .. 8 c + 7
-  // (c < 32: activation rows, else weight rows); lane l brings row l / 8 of those, chunk
-  // (l % 8) ^ swz(row).  swz depends on l / 8 and the parity of the wave only, so all A copies
-  // (and all B copies) of a wave share one per-lane offset and differ by a multiple of 64 rows.
-  // Rows past M / N fall beyond the buffer's extent and read as zero; the K offset travels in
-  // the scalar operand (K is a multiple of 128 for this kernel).
+  // Copy j (0..3) of a wave fills activation rows 8 (wave + 8 j) .. + 7 of the stage, and
+  // the same rows of the weight half; lane l brings row l / 8 of those, chunk
+  // (l % 8) ^ swz(row).  swz depends on l / 8 and the parity of the wave only, so the four
+  // copies share one per-lane offset and differ by a multiple of 64 rows.  Rows past M / N
+  // fall beyond the buffer's extent and read as zero; the K offset travels in the scalar
+  // operand.
   const int l8 = lane >> 3;
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
   const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
-  uint32_t off_a = 0, off_b = 0;  // of the tile whose copies are being issued
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
-  auto issue_load = [&](int j, int stage, int k0) {
-    const bool is_a = j < 4;
-    const int c = wave + j * NW;
-    if (c >= NCOPY) return;  // wave-uniform; only the last copy of a 224-wide tile
-    char* dst = smem + stage * STAGE_BYTES + c * 1024;
-    const uint32_t off = is_a ? off_a + (uint32_t)j * step_a : off_b + (uint32_t)(j - 4) * step_b;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(is_a ? ra : rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0,
-                                             0, 0);
+  // off_a: tile of the block after the current one (copies issued in a tile's first step);
+  // off_a2: tile of the block two after the current one (copies issued behind MFMAs 28..31);
+  // off_b: tile of the block after the current one.
+  uint32_t off_a = 0, off_a2 = 0, off_b = 0;
+  auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
+    char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
+                                             off + (uint32_t)j * step_a, k0, 0, 0);
   };
+  auto copy_b = [&](int j, int stage, int k0) {
+    char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16,
+                                             off_b + (uint32_t)j * step_b, k0, 0, 0);
+  };
+  auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
+  auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
 
   const int sw = (r16 & 7) ^ (r16 >> 3);
   const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
@@ -743,37 +754,34 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 
   using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
   acc_t acc[MI][NI];
+  v8i bf[NI];  // the step's weight fragments
+  v8i a_cur;   // the activation fragment the next MFMAs use
 
-  // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].  A lane owns
-  // row r16 of each of the wave's 16-row activation fragments.  The wave's weight fragments
-  // 0 .. jsw - 1 lie in scale block nb_lo, the others in nb_lo + 1.
+  // Block scales of the block after the current one (addressing switches to the next tile
+  // together with off_b).  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a
+  // lane owns row r16 of each of the wave's 16-row fragments.
   const int nkb = p.K >> 7;
-  float sfa_cur[MI], sfa_nxt[MI];
-  float sfb_lo = 0.f, sfb_hi = 0.f, sfb_lo_nxt = 0.f, sfb_hi_nxt = 0.f;
-  __amdgpu_buffer_rsrc_t rs = ra;
+  float sfa_cur[MI];
+  float sfb_cur = 0.f, sfb_next = 0.f;
+  __amdgpu_buffer_rsrc_t rs = ra, rsb = ra;
   uint32_t sfa_off = 0, sfa_ok = 0;
-  int sfa_frag = 0, sfa_step = 0, nb_lo = 0, nb_hi = 0, jsw = NI, jsw_nxt = NI;
+  int sfa_frag = 0, sfa_step = 0, sfb_step = 0, sfb_col = 0;
   if constexpr (BLOCK) {
     const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
     rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    const int nblocks = (p.N + 127) >> 7;
+    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
+    rsb = make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sfa_frag = (int)(16 * p.sa_stride_m * 4);
     sfa_step = (int)(p.sa_stride_k * 4);
+    sfb_step = (int)(p.sb_stride_k * 4);
   }
-  // Addressing of the tile whose copies and scales are issued from now on.
-  auto set_tile = [&](int m0, int n0) {
-    off_a = (uint32_t)(m0 + row_in_tile) * p.lda + c16;
-    off_b = (uint32_t)(n0 + row_in_tile) * p.ldb + c16;
+  auto set_scales = [&](int m0, int n0) {
     if constexpr (BLOCK) {
       const int nblocks = (p.N + 127) >> 7;
-      const int nw = n0 + wn * TN;
-      nb_lo = nw >> 7;
-      jsw_nxt = ((nb_lo + 1) * 128 - nw) >> 4;
-      nb_hi = nb_lo + 1;
-      if (nb_lo >= nblocks) nb_lo = nblocks - 1;
-      if (nb_hi >= nblocks) nb_hi = nblocks - 1;
-      nb_lo = __builtin_amdgcn_readfirstlane(nb_lo);
-      nb_hi = __builtin_amdgcn_readfirstlane(nb_hi);
-      jsw_nxt = __builtin_amdgcn_readfirstlane(jsw_nxt);
+      int nb = (n0 + wn * TN) >> 7;
+      if (nb >= nblocks) nb = nblocks - 1;
+      sfb_col = __builtin_amdgcn_readfirstlane((int)(nb * p.sb_stride_n * 4));
       const int mrow = m0 + wm * TM + r16;
       // a row past M must not alias a valid element of another K block: send it out of range
       sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
@@ -786,101 +794,96 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
                                          rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
   };
+  // one dword, the same for every lane: a vector load, so that it is counted with the others
+  auto load_sfb = [&](int kb) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsb, (uint32_t)sfb_col, kb * sfb_step, 0));
+  };
 
-  // One K step on stage `cur`.  With a `pre_tag`, the copies (into the other stage) and the
-  // scales of K block `kn` of the tile that set_tile named last are issued here, in the
-  // shadow of the MFMAs: that is the next K block of this tile, or, in a tile's last step
-  // (`last_tag`), the first K block of the block's next tile.
-  auto k_step = [&](int cur, int kn, auto pre_tag, auto last_tag) {
-    constexpr bool pre = decltype(pre_tag)::value;
+  // One K step: block u sits in stage `cur` and its first fragments are in bf / a_cur.
+  // kn: index, inside its tile, of block u + 1 (weight copies, scales, and in a tile's first
+  // step the activation copies); kn2: that of block u + 2 (activation copies, off_a2).
+  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
+    constexpr bool first = decltype(first_tag)::value;
     constexpr bool last = decltype(last_tag)::value;
     const char* st = smem + cur * STAGE_BYTES;
-    v8i af[MI];
-    af[0] = read_frag(st + a_base);
-    v8i b_cur = read_frag(st + b_base);
-#pragma unroll
-    for (int i = 1; i < MI; ++i) af[i] = read_frag(st + a_base + i * 16 * 128);
+    const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
-    __builtin_amdgcn_sched_barrier(0);
-
     v4f part_prev = {0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      v8i b_nxt = b_cur;
-      float sfb_j = 0.f;
-      if constexpr (BLOCK) sfb_j = j < jsw ? sfb_lo : sfb_hi;  // wave-uniform
+    for (int i = 0; i < MI; ++i) {
+      v8i a_nxt = a_cur;
+      if constexpr (BLOCK) {
+        sc_prev = sc;
+        sc = sfa_cur[i] * sfb_cur;
+      }
+      if (i == MI - 1) {
+        // Vector-memory operations retire in order.  Younger than the last copy of block
+        // u + 1 (issued behind MFMA 3, or MFMA 7 in a tile's first step) are only this step's
+        // scale loads: the weight scale (behind MFMA 8) and the activation-scale refills
+        // behind MFMAs 5, 9, .., 25.  lgkmcnt(0): this wave's LDS reads of stage `cur` are
+        // complete.  A bare s_barrier: these waits are all the ordering that is needed.
+        constexpr int YOUNGER = BLOCK ? (first ? 6 : 7) : 0;
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(YOUNGER));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const int idx = j * MI + i;
+      for (int j = 0; j < NI; ++j) {
+        const int idx = i * NI + j;
+        v4f part = {0.f, 0.f, 0.f, 0.f};
         if constexpr (BLOCK) {
           const v4f z = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], z, 0, 0, 0, 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
-          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
-          sc_prev = sc;
-          sc = sfa_cur[i] * sfb_j;
-          if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
-            const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
-            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], sc_prev, acc[pi][pj][0]);
-            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], sc_prev, acc[pi][pj][1]);
-            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], sc_prev, acc[pi][pj][2]);
-            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], sc_prev, acc[pi][pj][3]);
-          }
-          if (pre && idx == NLOAD) {
-            sfb_lo_nxt = p.sb[kn * p.sb_stride_k + nb_lo * p.sb_stride_n];
-            sfb_hi_nxt = p.sb[kn * p.sb_stride_k + nb_hi * p.sb_stride_n];
-          }
-          if (pre && idx >= NLOAD && idx < NLOAD + MI) sfa_nxt[idx - NLOAD] = load_sfa(idx - NLOAD, kn);
-          part_prev = part;
+          part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, z, 0, 0, 0, 0, 0, 0);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
-          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
-          const v4i b0 = {b_cur[0], b_cur[1], b_cur[2], b_cur[3]}, b1 = {b_cur[4], b_cur[5], b_cur[6], b_cur[7]};
-          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]}, a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
+          const v4i b0 = {bf[j][0], bf[j][1], bf[j][2], bf[j][3]};
+          const v4i a0 = {a_cur[0], a_cur[1], a_cur[2], a_cur[3]};
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          if (i == 0 && j + 1 < NI) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
-          if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!IS_FP8) {
+          const v4i b1 = {bf[j][4], bf[j][5], bf[j][6], bf[j][7]};
+          const v4i a1 = {a_cur[4], a_cur[5], a_cur[6], a_cur[7]};
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (i + 1 < MI) {
+          if (j == 0) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
+        } else {
+          // weight fragment j has had its last use in this step: refill it from block u + 1
+          bf[j] = read_frag(sn + b_base + j * 16 * 128);
+          if (j == 0) a_nxt = read_frag(sn + a_base);
+          if (!last) copy_a(j, cur, kn2 * 128, off_a2);
+        }
+        if (idx < 4) copy_b(idx, cur ^ 1, kn * 128);
+        if (first && idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+        if constexpr (BLOCK) {
+          if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
+            const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
+            const float s_use = (pi == i) ? sc : sc_prev;
+            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], s_use, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], s_use, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
+          }
+          if (idx == 8) sfb_next = load_sfb(kn);
+          // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
+          if (j == 1 && i >= 1) sfa_cur[i - 1] = load_sfa(i - 1, kn);
+          part_prev = part;
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      b_cur = b_nxt;
+      a_cur = a_nxt;
     }
     if constexpr (BLOCK) {
       acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
       acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
       acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
-      if constexpr (pre) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i) sfa_cur[i] = sfa_nxt[i];
-        sfb_lo = sfb_lo_nxt;
-        sfb_hi = sfb_hi_nxt;
-        jsw = jsw_nxt;
-      }
-    }
-    if constexpr (!last) {
-      // The next stage's copies were the first vector-memory loads of this step and
-      // vector-memory operations retire in order, so it is enough to wait until at most the
-      // SCALE_LOADS_AFTER_COPIES younger ones (activation-scale loads, none for the other
-      // kinds) are still in flight; lgkmcnt(0) covers this wave's LDS reads of the stage
-      // that the next step overwrites.  A bare s_barrier: the waits above are the only
-      // ordering needed, a fence would drain the scale loads as well.
-      constexpr int SCALE_LOADS_AFTER_COPIES = BLOCK ? MI : 0;
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(SCALE_LOADS_AFTER_COPIES));
-      __builtin_amdgcn_s_barrier();
-    } else {
-      // Last K block of a tile: wait for everything, so that the epilogue's stores are the
-      // only vector-memory operations in flight when the next tile starts.  After the
-      // barrier the next tile's first K block is visible to every wave and nobody reads
-      // this stage any more (it becomes the epilogue's staging buffer).
-      __builtin_amdgcn_s_waitcnt(0);
-      __builtin_amdgcn_s_barrier();
+      sfa_cur[MI - 1] = load_sfa(MI - 1, kn);
+      sfb_cur = sfb_next;
     }
   };
 
@@ -893,18 +896,23 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   int m0 = tm * BM, n0 = tn * BN;
   int par = 0;  // stage that holds K block 0 of the current tile
 
-  set_tile(m0, n0);
+  off_a = off_a2 = a_offset(m0);
+  off_b = b_offset(n0);
+  set_scales(m0, n0);
 #pragma unroll
-  for (int j = 0; j < NLOAD; ++j) issue_load(j, 0, 0);
+  for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) copy_b(j, 0, 0);
   if constexpr (BLOCK) {
 #pragma unroll
     for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
-    sfb_lo = p.sb[nb_lo * p.sb_stride_n];
-    sfb_hi = p.sb[nb_hi * p.sb_stride_n];
-    jsw = jsw_nxt;
+    sfb_cur = load_sfb(0);
   }
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int j = 0; j < NI; ++j) bf[j] = read_frag(smem + b_base + j * 16 * 128);
+  a_cur = read_frag(smem + a_base);
 
   while (true) {
 #pragma unroll
@@ -912,32 +920,341 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
-    for (int kb = 0; kb + 1 < nkb; ++kb) k_step((kb + par) & 1, kb + 1, std::true_type{}, std::false_type{});
-
+    // The block's next tile; past its last tile the prefetches are pointed at rows beyond M
+    // and N, which the buffer bounds turn into zero fill without memory traffic.
     const int next_tile = tile + (int)gridDim.x;
     const bool has_next = next_tile < total;
-    const int last_stage = (nkb - 1 + par) & 1;
-    const int cm0 = m0, cn0 = n0;
-    // The tile's last step always prefetches: past the block's last tile it is pointed at
-    // rows beyond M and N, which the buffer bounds turn into zero fill without memory traffic.
     tile_of_block(has_next ? next_tile : 0, p.tiles_m, p.tiles_n, tm, tn);
-    m0 = has_next ? tm * BM : p.tiles_m * BM;
-    n0 = has_next ? tn * BN : p.tiles_n * BN;
-    set_tile(m0, n0);  // the current tile issues no more copies or scale loads
-    k_step(last_stage, 0, std::true_type{}, std::true_type{});
+    const int nm0 = has_next ? tm * BM : p.tiles_m * BM;
+    const int nn0 = has_next ? tn * BN : p.tiles_n * BN;
 
+    // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
+    const uint32_t off_a_next = a_offset(nm0);
+    k_step(par, 1, 2, std::true_type{}, std::false_type{});
+    for (int kb = 1; kb + 1 < nkb; ++kb) {
+      const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
+      off_a2 = pen ? off_a_next : off_a2;
+      k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
+    }
+    // last K block: the weight copies and the scales issued now belong to the next tile
+    const int last_stage = (nkb - 1 + par) & 1;
+    off_b = b_offset(nn0);
+    set_scales(nm0, nn0);
+    k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
+    off_a = off_a2;
+
+    // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
+    // nothing is being copied into it, so it stages the C tile.
     if constexpr (KIND == KIND_I8_RAW) {
-      epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+      epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g,
-                                                   lane, wave);
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, m0, n0, wm, wn, r16, g, lane,
+                                                   wave);
       else
-        epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+        epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     }
     if (!has_next) break;
     tile = next_tile;
+    m0 = nm0;
+    n0 = nn0;
+    par = last_stage ^ 1;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 256 x (32 NI) kernel, NI = 6, 7 or 8 (tile widths 192, 224, 256), K >= 384: the same
+// persistent, pipelined two-stage structure as gemm_pipe_kernel with the roles of the
+// operands exchanged.  The eight waves form a 4 (M) x 2 (N) grid; a wave keeps its four
+// activation fragments of the K step in registers and streams its NI weight fragments one
+// ahead.  The tile width is chosen on the host so that the tile count fills whole rounds of
+// the chip's CUs: 7168 columns are 32 tiles of 224 (two full rounds at M = 4096) instead
+// of 28 tiles of 256 (one full round and a 3/4 one).  A wave's columns can straddle two
+// 128-column scale blocks, so the weight scale is selected per fragment.
+// ---------------------------------------------------------------------------
+template <int KIND, int OUT_DT, int NI>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
+  constexpr int BM = 256, NW = 8, WAVES_N = 2, MI = 4;
+  constexpr int TM = MI * 16, TN = NI * 16, BN = WAVES_N * TN;
+  constexpr int STAGE_BYTES = 512 * 128;  // stage pitch; only (BM + BN) rows are filled
+  constexpr int NB = BN / 8;              // one-KiB weight copies per stage
+  constexpr int NBW = (NB + NW - 1) / NW; // ... per wave (the last one only for waves < NB % 8)
+  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
+
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
+
+  // Copy j of a wave fills activation rows 8 (wave + 8 j) .. + 7 of the stage, or the same
+  // rows of the weight part; lane l brings row l / 8 of those, chunk (l % 8) ^ swz(row).
+  // swz depends on l / 8 and the parity of the wave only, so a wave's copies share one
+  // per-lane offset and differ by a multiple of 64 rows.  Rows past M / N fall beyond the
+  // buffer's extent and read as zero; the K offset travels in the scalar operand.  A
+  // weight copy past the tile's width (224-wide tiles: the fourth copy of waves 4..7) is
+  // sent out of range as well and zero-fills stage rows that nobody reads.
+  const int l8 = lane >> 3;
+  const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
+  const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
+  const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
+  const bool last_b_ok = wave + (NBW - 1) * NW < NB;
+  // off_a: tile of the block after the current one (copies issued in a tile's first step);
+  // off_a2: tile of the block two after the current one (copies behind the last MFMAs);
+  // off_b: tile of the block after the current one.
+  uint32_t off_a = 0, off_a2 = 0, off_b = 0;
+  auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
+    char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
+                                             off + (uint32_t)j * step_a, k0, 0, 0);
+  };
+  auto copy_b = [&](int j, int stage, int k0) {
+    char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
+    uint32_t off = off_b + (uint32_t)j * step_b;
+    if (j == NBW - 1 && NB % NW != 0) off = last_b_ok ? off : OOB;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0, 0, 0);
+  };
+  auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
+  auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  const int a_base = (wm * TM) * 128;
+  const int b_base = (BM + wn * TN) * 128;
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[MI][NI];
+  v8i af[MI];  // the step's activation fragments
+  v8i b_cur;   // the weight fragment the next MFMAs use
+
+  // Block scales of the block after the current one (addressing switches to the next tile
+  // together with off_b).  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a
+  // lane owns row r16 of each of the wave's 16-row activation fragments.  The wave's weight
+  // fragments 0 .. jsw - 1 lie in one 128-column scale block, the others in the next.
+  const int nkb = p.K >> 7;
+  float sfa_cur[MI], sfa_nxt[MI];
+  float sfb_lo = 0.f, sfb_hi = 0.f, sfb_lo_nxt = 0.f, sfb_hi_nxt = 0.f;
+  __amdgpu_buffer_rsrc_t rs = ra, rsb = ra;
+  uint32_t sfa_off = 0, sfa_ok = 0;
+  int sfa_frag = 0, sfa_step = 0, sfb_step = 0, sfb_col_lo = 0, sfb_col_hi = 0, jsw = NI, jsw_nxt = NI;
+  if constexpr (BLOCK) {
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
+    const int nblocks = (p.N + 127) >> 7;
+    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
+    rsb = make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
+    sfa_frag = (int)(16 * p.sa_stride_m * 4);
+    sfa_step = (int)(p.sa_stride_k * 4);
+    sfb_step = (int)(p.sb_stride_k * 4);
+  }
+  auto set_scales = [&](int m0, int n0) {
+    if constexpr (BLOCK) {
+      const int nblocks = (p.N + 127) >> 7;
+      const int nw = n0 + wn * TN;
+      int nb_lo = nw >> 7;
+      jsw_nxt = __builtin_amdgcn_readfirstlane(((nb_lo + 1) * 128 - nw) >> 4);
+      int nb_hi = nb_lo + 1;
+      if (nb_lo >= nblocks) nb_lo = nblocks - 1;
+      if (nb_hi >= nblocks) nb_hi = nblocks - 1;
+      sfb_col_lo = __builtin_amdgcn_readfirstlane((int)(nb_lo * p.sb_stride_n * 4));
+      sfb_col_hi = __builtin_amdgcn_readfirstlane((int)(nb_hi * p.sb_stride_n * 4));
+      const int mrow = m0 + wm * TM + r16;
+      // a row past M must not alias a valid element of another K block: send it out of range
+      sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
+      sfa_ok = 0;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sfa_ok |= (mrow + i * 16 < p.M ? 1u : 0u) << i;
+    }
+  };
+  auto load_sfa = [&](int i, int kb) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
+  };
+  // one dword, the same for every lane: a vector load, so that it is counted with the others
+  auto load_sfb = [&](int col, int kb) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsb, (uint32_t)col, kb * sfb_step, 0));
+  };
+
+  // One K step: block u sits in stage `cur`, its activation fragments and first weight
+  // fragment are in af / b_cur.  kn: index, inside its tile, of block u + 1 (weight copies,
+  // scales, and in a tile's first step the activation copies); kn2: that of block u + 2
+  // (activation copies, off_a2).  The step's barrier comes before the last weight
+  // fragment's four MFMAs; behind those the wave reads the first fragments of block u + 1
+  // and issues the activation copies of block u + 2 into the stage that just became free.
+  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
+    constexpr bool first = decltype(first_tag)::value;
+    constexpr bool last = decltype(last_tag)::value;
+    const char* st = smem + cur * STAGE_BYTES;
+    const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
+    float sc = 0.f, sc_prev = 0.f;
+    v4f part_prev = {0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      v8i b_nxt = b_cur;
+      float sfb_j = 0.f;
+      if constexpr (BLOCK) sfb_j = j < jsw ? sfb_lo : sfb_hi;  // wave-uniform
+      if (j == NI - 1) {
+        // Vector-memory operations retire in order.  Younger than the last copy of block
+        // u + 1 (issued behind MFMA 3, or MFMA 7 in a tile's first step) are only this step's
+        // six scale loads (behind MFMAs 8..12).  lgkmcnt(0): this wave's LDS reads of stage
+        // `cur` are complete.  A bare s_barrier: these waits are all the ordering needed.
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(BLOCK ? 6 : 0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int idx = j * MI + i;
+        v4f part = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (BLOCK) {
+          const v4f z = {0.f, 0.f, 0.f, 0.f};
+          part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], z, 0, 0, 0, 0, 0, 0);
+        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+        } else {
+          const v4i b0 = {b_cur[0], b_cur[1], b_cur[2], b_cur[3]};
+          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!IS_FP8) {
+          const v4i b1 = {b_cur[4], b_cur[5], b_cur[6], b_cur[7]};
+          const v4i a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (j + 1 < NI) {
+          if (i == 0) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
+        } else {
+          // activation fragment i has had its last use in this step: refill it from block u + 1
+          af[i] = read_frag(sn + a_base + i * 16 * 128);
+          if (i == 0) b_nxt = read_frag(sn + b_base);
+          if (!last) copy_a(i, cur, kn2 * 128, off_a2);
+        }
+        if (idx < NBW) copy_b(idx, cur ^ 1, kn * 128);
+        if (first && idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+        if constexpr (BLOCK) {
+          sc_prev = sc;
+          sc = sfa_cur[i] * sfb_j;
+          if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
+            const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
+            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], sc_prev, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], sc_prev, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], sc_prev, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], sc_prev, acc[pi][pj][3]);
+          }
+          if (idx == 8) {
+            sfb_lo_nxt = load_sfb(sfb_col_lo, kn);
+            sfb_hi_nxt = load_sfb(sfb_col_hi, kn);
+          }
+          if (idx >= 9 && idx < 9 + MI) sfa_nxt[idx - 9] = load_sfa(idx - 9, kn);
+          part_prev = part;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      b_cur = b_nxt;
+    }
+    if constexpr (BLOCK) {
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) sfa_cur[i] = sfa_nxt[i];
+      sfb_lo = sfb_lo_nxt;
+      sfb_hi = sfb_hi_nxt;
+      jsw = jsw_nxt;
+    }
+  };
+
+  // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
+  const int total = p.tiles_m * p.tiles_n;
+  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+  int tile = blockIdx.x;
+  int tm, tn;
+  tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+  int m0 = tm * BM, n0 = tn * BN;
+  int par = 0;  // stage that holds K block 0 of the current tile
+
+  off_a = off_a2 = a_offset(m0);
+  off_b = b_offset(n0);
+  set_scales(m0, n0);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
+#pragma unroll
+  for (int j = 0; j < NBW; ++j) copy_b(j, 0, 0);
+  if constexpr (BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
+    sfb_lo = load_sfb(sfb_col_lo, 0);
+    sfb_hi = load_sfb(sfb_col_hi, 0);
+    jsw = jsw_nxt;
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < MI; ++i) af[i] = read_frag(smem + a_base + i * 16 * 128);
+  b_cur = read_frag(smem + b_base);
+
+  while (true) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+    // The block's next tile; past its last tile the prefetches are pointed at rows beyond M
+    // and N, which the buffer bounds turn into zero fill without memory traffic.
+    const int next_tile = tile + (int)gridDim.x;
+    const bool has_next = next_tile < total;
+    tile_of_block(has_next ? next_tile : 0, p.tiles_m, p.tiles_n, tm, tn);
+    const int nm0 = has_next ? tm * BM : p.tiles_m * BM;
+    const int nn0 = has_next ? tn * BN : p.tiles_n * BN;
+
+    // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
+    const uint32_t off_a_next = a_offset(nm0);
+    k_step(par, 1, 2, std::true_type{}, std::false_type{});
+    for (int kb = 1; kb + 1 < nkb; ++kb) {
+      const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
+      off_a2 = pen ? off_a_next : off_a2;
+      k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
+    }
+    // last K block: the weight copies and the scales issued now belong to the next tile
+    const int last_stage = (nkb - 1 + par) & 1;
+    off_b = b_offset(nn0);
+    set_scales(nm0, nn0);
+    k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
+    off_a = off_a2;
+
+    // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
+    // nothing is being copied into it, so it stages the C tile.
+    if constexpr (KIND == KIND_I8_RAW) {
+      epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+    } else {
+      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
+      if (aligned_out)
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, m0, n0, wm, wn, r16, g, lane,
+                                                   wave);
+      else
+        epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+    }
+    if (!has_next) break;
+    tile = next_tile;
+    m0 = nm0;
+    n0 = nn0;
     par = last_stage ^ 1;
   }
 }
@@ -1159,7 +1476,8 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 }
 
 // test hook: 0 = heuristic, 64 = the M <= 64 kernel where it applies, 128 = the 128 x 128 kernel,
-// 256 = the 256 x 256 kernel, 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide
+// 256 = the plain 256 x 256 kernel, 258 = the pipelined one (K >= 384, else the plain one),
+// 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258)
 static int g_force_tile = 0;
 
 template <int KIND, int OUT_DT>
@@ -1170,7 +1488,9 @@ static void launch_big(GemmArgs& p, hipStream_t st) {
   // persistent: one block per CU walks the tiles blockIdx, blockIdx + gridDim, ...
   const int tiles = p.tiles_m * p.tiles_n;
   const int blocks = tiles < num_cus() ? tiles : num_cus();
-  gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  // the pipelined kernel needs three K blocks; 256 forces the plain one (test hook)
+  if (g_force_tile != 256 && p.K >= 384) gemm_pipe_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  else gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
 }
 
 template <int KIND, int OUT_DT, int NI>
@@ -1247,9 +1567,10 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // the 256 CUs (e.g. 144 tiles at M = 4096, N = 2112; 192 at M = 512, N = 24576); with
   // fewer tiles the 128 x 128 kernel with split-K keeps more CUs busy.
   const int big_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
-  const bool forced_256 = g_force_tile == 256 || g_force_tile == 192 || g_force_tile == 224 || g_force_tile == 257;
+  const bool forced_256 = g_force_tile == 256 || g_force_tile == 258 || g_force_tile == 192 || g_force_tile == 224 || g_force_tile == 257;
   if ((p.K & 127) == 0 && (forced_256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && big_tiles >= 140))) {
-    const int width = g_force_tile == 0 ? pick_tile_width(p) : g_force_tile;
+    int width = g_force_tile == 0 ? pick_tile_width(p) : g_force_tile;
+    if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
     else if (width == 257) launch_wide<KIND, OUT_DT, 8>(p, st);

@@ -37,8 +37,8 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
-# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide)
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257], ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256"])
+# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258], ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256"])
 def tile(request):
     from sglang_amd import _lib
 
