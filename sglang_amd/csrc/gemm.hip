@@ -680,20 +680,28 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 
 // ---------------------------------------------------------------------------
 // 256 x 256 kernel, software-pipelined across K steps (K >= 384).  Same tile, wave grid
-// and LDS layout as gemm_big_kernel; what differs is where the step barrier sits and what
-// is in registers when a step starts:
-//   * the barrier of step u comes before its last activation fragment's four MFMAs (MFMA
-//     28 of 32).  By then every wave has issued and completed all its LDS reads of step
-//     u's stage, and the copies of K block u + 1 have landed in the other stage.
-//   * behind MFMAs 28..31 a wave reads the first fragments of block u + 1 (each weight
-//     fragment right after its last use, plus the first activation fragment) and issues
-//     the four activation copies of block u + 2 into the stage that just became free; the
-//     four weight copies of block u + 2 follow behind MFMAs 0..3 of step u + 1.
-// So a step starts with its operands in registers and four MFMAs queued behind the
-// barrier, instead of every wave waiting for ten LDS reads right after it.  The sequence
-// of blocks runs across tile boundaries (the block's next tile follows the last K block
-// of the current one); only the activation copies behind the last step of a tile are
-// deferred to the next tile's first step, because the freed stage stages the C tile.
+// and LDS layout as gemm_big_kernel; what differs is what is in registers when a step
+// starts and how far ahead the copies run.  With u the running index of the K block:
+//   * step u starts with block u's four weight fragments and first activation fragment in
+//     registers.  Barrier 1, behind MFMA 3: every wave holds block u's weights in registers,
+//     so the weight half of block u's stage is free and receives the weight copies of block
+//     u + 2 (behind MFMAs 4..7): they have 1 3/4 steps to land.
+//   * barrier 2, before the last activation fragment's four MFMAs (28..31): every wave has
+//     completed its LDS reads of block u's activations, and block u + 1 has landed.  Behind
+//     MFMAs 28..31 a wave reads the first fragments of block u + 1 (each weight fragment
+//     right after its last use) and issues the activation copies of block u + 2 into the
+//     half that just became free (one step to land).
+//   * the block scales travel through LDS like the operands: per K block one dword per
+//     activation row (four 64-row copies, waves 0..3) and the tile's two weight scales (wave
+//     4), issued with the activation copies and read into registers behind MFMAs 28..31.
+//     Vector-memory instructions are the scarce issue resource of this loop (a CU's 64
+//     one-KiB copies per step already keep its address unit busy half of the time); loading
+//     the scales per fragment and per wave took as many instructions again.
+// A CU needs about a stage's worth of bytes in flight to cover the memory latency of a
+// step; a plain two-stage ring has less than that most of the time.  The sequence of
+// blocks runs across tile boundaries (the block's next tile follows the last K block of
+// the current one); only the copies behind a tile's last step are deferred to the next
+// tile's first step, because the freed stage stages the C tile.
 // ---------------------------------------------------------------------------
 template <int KIND, int OUT_DT>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
@@ -704,7 +712,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
   static_assert(NI == 4 && MI == 8, "the copy schedule below is written for 4 x 8 fragments");
 
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+  constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -724,19 +733,18 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
   const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
-  // off_a: tile of the block after the current one (copies issued in a tile's first step);
-  // off_a2: tile of the block two after the current one (copies issued behind MFMAs 28..31);
-  // off_b: tile of the block after the current one.
-  uint32_t off_a = 0, off_a2 = 0, off_b = 0;
+  // off_a / off_b: tile of the block after the current one (copies deferred to a tile's first
+  // step); off_a2 / off_b2: tile of the block two after the current one.
+  uint32_t off_a = 0, off_a2 = 0, off_b = 0, off_b2 = 0;
   auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
     char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
                                              off + (uint32_t)j * step_a, k0, 0, 0);
   };
-  auto copy_b = [&](int j, int stage, int k0) {
+  auto copy_b = [&](int j, int stage, int k0, uint32_t off) {
     char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16,
-                                             off_b + (uint32_t)j * step_b, k0, 0, 0);
+                                             off + (uint32_t)j * step_b, k0, 0, 0);
   };
   auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
   auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
@@ -757,51 +765,50 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   v8i bf[NI];  // the step's weight fragments
   v8i a_cur;   // the activation fragment the next MFMAs use
 
-  // Block scales of the block after the current one (addressing switches to the next tile
-  // together with off_b).  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a
-  // lane owns row r16 of each of the wave's 16-row fragments.
+  // Block scales.  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a lane owns
+  // row r16 of each of the wave's 16-row fragments.  Every wave issues one 4-byte-per-lane
+  // copy per K block: waves 0..3 the activation scales of tile rows 64 w + lane, wave 4 the
+  // two weight scales of the tile's two 128-column blocks (lanes 0 and 1), waves 5..7 nothing
+  // (all lanes out of range; kept so that the instruction stream has no branch).
+  // sc_voff / sc_voff2: per-lane source offsets for the tile of block u + 1 / u + 2.
   const int nkb = p.K >> 7;
   float sfa_cur[MI];
-  float sfb_cur = 0.f, sfb_next = 0.f;
-  __amdgpu_buffer_rsrc_t rs = ra, rsb = ra;
-  uint32_t sfa_off = 0, sfa_ok = 0;
-  int sfa_frag = 0, sfa_step = 0, sfb_step = 0, sfb_col = 0;
+  float sfb_cur = 0.f;
+  __amdgpu_buffer_rsrc_t rsc = ra;
+  uint32_t sc_voff = OOB, sc_voff2 = OOB;
+  int sc_step = 0;
+  const int sc_dst = 2 * STAGE_BYTES + wave * 256;  // waves 5..7 land behind the used part
+  const int sfa_rd = 2 * STAGE_BYTES + (wm * TM + r16) * 4;
+  const int sfb_rd = 2 * STAGE_BYTES + 1024 + (wn >> 1) * 4;
   if constexpr (BLOCK) {
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
-    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
     const int nblocks = (p.N + 127) >> 7;
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
-    rsb = make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
-    sfa_frag = (int)(16 * p.sa_stride_m * 4);
-    sfa_step = (int)(p.sa_stride_k * 4);
-    sfb_step = (int)(p.sb_stride_k * 4);
+    rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
+    sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
   }
-  auto set_scales = [&](int m0, int n0) {
-    if constexpr (BLOCK) {
-      const int nblocks = (p.N + 127) >> 7;
-      int nb = (n0 + wn * TN) >> 7;
-      if (nb >= nblocks) nb = nblocks - 1;
-      sfb_col = __builtin_amdgcn_readfirstlane((int)(nb * p.sb_stride_n * 4));
-      const int mrow = m0 + wm * TM + r16;
-      // a row past M must not alias a valid element of another K block: send it out of range
-      sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
-      sfa_ok = 0;
-#pragma unroll
-      for (int i = 0; i < MI; ++i) sfa_ok |= (mrow + i * 16 < p.M ? 1u : 0u) << i;
+  auto scale_offset = [&](int m0, int n0) -> uint32_t {
+    if (wave < 4) {
+      const int row = m0 + wave * 64 + lane;
+      return row < p.M ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
     }
+    const int nblocks = (p.N + 127) >> 7;
+    int nb = (n0 >> 7) + lane;
+    if (nb >= nblocks) nb = nblocks - 1;
+    return (wave == 4 && lane < 2) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
   };
-  auto load_sfa = [&](int i, int kb) -> float {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                         rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
+  auto copy_scales = [&](int buf, int kb, uint32_t voff) {
+    char* dst = smem + buf * SCALE_BYTES + sc_dst;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, voff, kb * sc_step, 0, 0);
   };
-  // one dword, the same for every lane: a vector load, so that it is counted with the others
-  auto load_sfb = [&](int kb) -> float {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsb, (uint32_t)sfb_col, kb * sfb_step, 0));
+  auto read_sfa = [&](int buf, int i) -> float {
+    return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfa_rd + i * 64);
   };
+  auto read_sfb = [&](int buf) -> float { return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfb_rd); };
 
   // One K step: block u sits in stage `cur` and its first fragments are in bf / a_cur.
-  // kn: index, inside its tile, of block u + 1 (weight copies, scales, and in a tile's first
-  // step the activation copies); kn2: that of block u + 2 (activation copies, off_a2).
+  // kn: index, inside its tile, of block u + 1 (scales, and the copies deferred to a tile's
+  // first step); kn2: that of block u + 2 (off_a2 / off_b2).
   auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
     constexpr bool first = decltype(first_tag)::value;
     constexpr bool last = decltype(last_tag)::value;
@@ -817,13 +824,19 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         sc_prev = sc;
         sc = sfa_cur[i] * sfb_cur;
       }
+      if (i == 1 && !last) {
+        // barrier 1: MFMAs 0..3 have consumed this wave's weight fragments, so its LDS reads
+        // of block u's weights are complete; behind the barrier that holds for every wave.
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (i == MI - 1) {
-        // Vector-memory operations retire in order.  Younger than the last copy of block
-        // u + 1 (issued behind MFMA 3, or MFMA 7 in a tile's first step) are only this step's
-        // scale loads: the weight scale (behind MFMA 8) and the activation-scale refills
-        // behind MFMAs 5, 9, .., 25.  lgkmcnt(0): this wave's LDS reads of stage `cur` are
-        // complete.  A bare s_barrier: these waits are all the ordering that is needed.
-        constexpr int YOUNGER = BLOCK ? (first ? 6 : 7) : 0;
+        // barrier 2.  Vector-memory operations retire in order; block u + 1's last copy is
+        // the activation copy behind MFMA 31 of the step before (MFMA 11 of this step in a
+        // tile's first step).  Younger than it are only the four weight copies of block u + 2,
+        // which stay in flight.  lgkmcnt(0): this wave's LDS reads of block u's activations
+        // and scales are complete.  A bare s_barrier: these waits are all the ordering needed.
+        constexpr int YOUNGER = last ? 0 : 4;
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(YOUNGER));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -856,9 +869,23 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           bf[j] = read_frag(sn + b_base + j * 16 * 128);
           if (j == 0) a_nxt = read_frag(sn + a_base);
           if (!last) copy_a(j, cur, kn2 * 128, off_a2);
+          if constexpr (BLOCK) {
+            // scales i < 7 had their last use when fragment 7's scale was formed; sfa_cur[7] and
+            // sfb_cur are dead as well: `sc` holds their product
+            sfa_cur[2 * j] = read_sfa(cur ^ 1, 2 * j);
+            sfa_cur[2 * j + 1] = read_sfa(cur ^ 1, 2 * j + 1);
+            if (j == 0) sfb_cur = read_sfb(cur ^ 1);
+            if (j == 0 && !last) copy_scales(cur, kn2, sc_voff2);
+          }
         }
-        if (idx < 4) copy_b(idx, cur ^ 1, kn * 128);
-        if (first && idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+        if constexpr (first) {
+          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b);
+          if (idx >= 8 && idx < 12) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
+          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
+          if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2);
+        } else if constexpr (!last) {
+          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2);
+        }
         if constexpr (BLOCK) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
@@ -868,9 +895,6 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
             acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
             acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
           }
-          if (idx == 8) sfb_next = load_sfb(kn);
-          // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
-          if (j == 1 && i >= 1) sfa_cur[i - 1] = load_sfa(i - 1, kn);
           part_prev = part;
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -882,8 +906,6 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
       acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
-      sfa_cur[MI - 1] = load_sfa(MI - 1, kn);
-      sfb_cur = sfb_next;
     }
   };
 
@@ -897,22 +919,23 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   int par = 0;  // stage that holds K block 0 of the current tile
 
   off_a = off_a2 = a_offset(m0);
-  off_b = b_offset(n0);
-  set_scales(m0, n0);
+  off_b = off_b2 = b_offset(n0);
+  if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0);
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_b(j, 0, 0);
-  if constexpr (BLOCK) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
-    sfb_cur = load_sfb(0);
-  }
+  for (int j = 0; j < 4; ++j) copy_b(j, 0, 0, off_b);
+  if constexpr (BLOCK) copy_scales(0, 0, sc_voff);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int j = 0; j < NI; ++j) bf[j] = read_frag(smem + b_base + j * 16 * 128);
   a_cur = read_frag(smem + a_base);
+  if constexpr (BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_cur[i] = read_sfa(0, i);
+    sfb_cur = read_sfb(0);
+  }
 
   while (true) {
 #pragma unroll
@@ -929,19 +952,23 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     const int nn0 = has_next ? tn * BN : p.tiles_n * BN;
 
     // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
-    const uint32_t off_a_next = a_offset(nm0);
+    const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
+    uint32_t sc_voff_next = OOB;
+    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
     k_step(par, 1, 2, std::true_type{}, std::false_type{});
     for (int kb = 1; kb + 1 < nkb; ++kb) {
       const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
       off_a2 = pen ? off_a_next : off_a2;
+      off_b2 = pen ? off_b_next : off_b2;
+      sc_voff2 = pen ? sc_voff_next : sc_voff2;
       k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
     }
-    // last K block: the weight copies and the scales issued now belong to the next tile
+    // last K block: its copies (the next tile's second block) wait for the next tile's first step
     const int last_stage = (nkb - 1 + par) & 1;
-    off_b = b_offset(nn0);
-    set_scales(nm0, nn0);
     k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
     off_a = off_a2;
+    off_b = off_b2;
+    sc_voff = sc_voff2;
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
