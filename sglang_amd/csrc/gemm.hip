@@ -998,7 +998,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 // ahead.  The tile width is chosen on the host so that the tile count fills whole rounds of
 // the chip's CUs: 7168 columns are 32 tiles of 224 (two full rounds at M = 4096) instead
 // of 28 tiles of 256 (one full round and a 3/4 one).  A wave's columns can straddle two
-// 128-column scale blocks, so the weight scale is selected per fragment.
+// 128-column scale blocks, so the weight scale is selected per fragment.  Here the
+// activation half of a stage is the one that is free early (barrier 1, behind MFMA 3: all
+// four activation fragments are in registers) and is refilled two K blocks ahead; the
+// weight copies of block u + 2 follow behind the last weight fragment's MFMAs.
 // ---------------------------------------------------------------------------
 template <int KIND, int OUT_DT, int NI>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
@@ -1011,7 +1014,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
   static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
 
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+  constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1033,18 +1037,17 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
   const bool last_b_ok = wave + (NBW - 1) * NW < NB;
-  // off_a: tile of the block after the current one (copies issued in a tile's first step);
-  // off_a2: tile of the block two after the current one (copies behind the last MFMAs);
-  // off_b: tile of the block after the current one.
-  uint32_t off_a = 0, off_a2 = 0, off_b = 0;
+  // off_a / off_b: tile of the block after the current one (copies deferred to a tile's first
+  // step); off_a2 / off_b2: tile of the block two after the current one.
+  uint32_t off_a = 0, off_a2 = 0, off_b = 0, off_b2 = 0;
   auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
     char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
                                              off + (uint32_t)j * step_a, k0, 0, 0);
   };
-  auto copy_b = [&](int j, int stage, int k0) {
+  auto copy_b = [&](int j, int stage, int k0, uint32_t off_tile) {
     char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
-    uint32_t off = off_b + (uint32_t)j * step_b;
+    uint32_t off = off_tile + (uint32_t)j * step_b;
     if (j == NBW - 1 && NB % NW != 0) off = last_b_ok ? off : OOB;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0, 0, 0);
   };
@@ -1067,60 +1070,63 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   v8i af[MI];  // the step's activation fragments
   v8i b_cur;   // the weight fragment the next MFMAs use
 
-  // Block scales of the block after the current one (addressing switches to the next tile
-  // together with off_b).  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a
-  // lane owns row r16 of each of the wave's 16-row activation fragments.  The wave's weight
-  // fragments 0 .. jsw - 1 lie in one 128-column scale block, the others in the next.
+  // Block scales.  Row m of K block kb sits at sfa[m * stride_m + kb * stride_k]; a lane owns
+  // row r16 of each of the wave's 16-row activation fragments.  Every wave issues one
+  // 4-byte-per-lane copy per K block: waves 0..3 the activation scales of tile rows
+  // 64 w + lane, wave 4 the weight scales of the (up to three) 128-column blocks the tile
+  // touches (lanes 0..2), waves 5..7 nothing (all lanes out of range; kept so that the
+  // instruction stream has no branch).  sc_voff / sc_voff2: per-lane source offsets for the
+  // tile of block u + 1 / u + 2.  The wave's weight fragments 0 .. jsw - 1 lie in scale
+  // block sb_lo of the tile's blocks, the others in sb_lo + 1.
   const int nkb = p.K >> 7;
-  float sfa_cur[MI], sfa_nxt[MI];
-  float sfb_lo = 0.f, sfb_hi = 0.f, sfb_lo_nxt = 0.f, sfb_hi_nxt = 0.f;
-  __amdgpu_buffer_rsrc_t rs = ra, rsb = ra;
-  uint32_t sfa_off = 0, sfa_ok = 0;
-  int sfa_frag = 0, sfa_step = 0, sfb_step = 0, sfb_col_lo = 0, sfb_col_hi = 0, jsw = NI, jsw_nxt = NI;
+  float sfa_cur[MI];
+  float sfb_lo = 0.f, sfb_hi = 0.f;
+  __amdgpu_buffer_rsrc_t rsc = ra;
+  uint32_t sc_voff = OOB, sc_voff2 = OOB;
+  int sc_step = 0, jsw = NI;
+  // jsw / sfb read offset of the tile whose scales are read next (two tiles can be in flight:
+  // the values for the tile of block u + 1 are needed when its scales are read)
+  int jsw_nxt = NI, sfb_rd_nxt = 0;
+  const int sc_dst = 2 * STAGE_BYTES + wave * 256;  // waves 5..7 land behind the used part
+  const int sfa_rd = 2 * STAGE_BYTES + (wm * TM + r16) * 4;
   if constexpr (BLOCK) {
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
-    rs = make_rsrc(p.sa, (uint32_t)(sfa_elems * 4));
     const int nblocks = (p.N + 127) >> 7;
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
-    rsb = make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
-    sfa_frag = (int)(16 * p.sa_stride_m * 4);
-    sfa_step = (int)(p.sa_stride_k * 4);
-    sfb_step = (int)(p.sb_stride_k * 4);
+    rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
+    sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
   }
-  auto set_scales = [&](int m0, int n0) {
-    if constexpr (BLOCK) {
-      const int nblocks = (p.N + 127) >> 7;
-      const int nw = n0 + wn * TN;
-      int nb_lo = nw >> 7;
-      jsw_nxt = __builtin_amdgcn_readfirstlane(((nb_lo + 1) * 128 - nw) >> 4);
-      int nb_hi = nb_lo + 1;
-      if (nb_lo >= nblocks) nb_lo = nblocks - 1;
-      if (nb_hi >= nblocks) nb_hi = nblocks - 1;
-      sfb_col_lo = __builtin_amdgcn_readfirstlane((int)(nb_lo * p.sb_stride_n * 4));
-      sfb_col_hi = __builtin_amdgcn_readfirstlane((int)(nb_hi * p.sb_stride_n * 4));
-      const int mrow = m0 + wm * TM + r16;
-      // a row past M must not alias a valid element of another K block: send it out of range
-      sfa_off = mrow < p.M ? (uint32_t)(mrow * p.sa_stride_m * 4) : OOB;
-      sfa_ok = 0;
-#pragma unroll
-      for (int i = 0; i < MI; ++i) sfa_ok |= (mrow + i * 16 < p.M ? 1u : 0u) << i;
+  auto scale_offset = [&](int m0, int n0) -> uint32_t {
+    if (wave < 4) {
+      const int row = m0 + wave * 64 + lane;
+      return row < p.M ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
     }
+    const int nblocks = (p.N + 127) >> 7;
+    int nb = (n0 >> 7) + lane;
+    if (nb >= nblocks) nb = nblocks - 1;
+    return (wave == 4 && lane < 3) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
   };
-  auto load_sfa = [&](int i, int kb) -> float {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                         rs, ((sfa_ok >> i) & 1) ? sfa_off + i * sfa_frag : OOB, kb * sfa_step, 0));
+  // where this wave's columns start inside the tile's scale blocks
+  auto set_scale_split = [&](int n0) {
+    const int nw = n0 + wn * TN;
+    const int nb_lo = nw >> 7;
+    jsw_nxt = __builtin_amdgcn_readfirstlane(((nb_lo + 1) * 128 - nw) >> 4);
+    sfb_rd_nxt = __builtin_amdgcn_readfirstlane(2 * STAGE_BYTES + 1024 + (nb_lo - (n0 >> 7)) * 4);
   };
-  // one dword, the same for every lane: a vector load, so that it is counted with the others
-  auto load_sfb = [&](int col, int kb) -> float {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsb, (uint32_t)col, kb * sfb_step, 0));
+  auto copy_scales = [&](int buf, int kb, uint32_t voff) {
+    char* dst = smem + buf * SCALE_BYTES + sc_dst;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, voff, kb * sc_step, 0, 0);
+  };
+  auto read_sfa = [&](int buf, int i) -> float {
+    return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfa_rd + i * 64);
+  };
+  auto read_sfb = [&](int buf, int which) -> float {
+    return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfb_rd_nxt + which * 4);
   };
 
   // One K step: block u sits in stage `cur`, its activation fragments and first weight
-  // fragment are in af / b_cur.  kn: index, inside its tile, of block u + 1 (weight copies,
-  // scales, and in a tile's first step the activation copies); kn2: that of block u + 2
-  // (activation copies, off_a2).  The step's barrier comes before the last weight
-  // fragment's four MFMAs; behind those the wave reads the first fragments of block u + 1
-  // and issues the activation copies of block u + 2 into the stage that just became free.
+  // fragment are in af / b_cur.  kn: index, inside its tile, of block u + 1 (the copies
+  // deferred to a tile's first step); kn2: that of block u + 2 (off_a2 / off_b2).
   auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
     constexpr bool first = decltype(first_tag)::value;
     constexpr bool last = decltype(last_tag)::value;
@@ -1134,12 +1140,21 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       v8i b_nxt = b_cur;
       float sfb_j = 0.f;
       if constexpr (BLOCK) sfb_j = j < jsw ? sfb_lo : sfb_hi;  // wave-uniform
+      if (j == 1 && !last) {
+        // barrier 1: MFMAs 0..3 have consumed this wave's activation fragments, so its LDS
+        // reads of block u's activations are complete; behind the barrier that holds for
+        // every wave and the activation half of the stage is free.
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (j == NI - 1) {
-        // Vector-memory operations retire in order.  Younger than the last copy of block
-        // u + 1 (issued behind MFMA 3, or MFMA 7 in a tile's first step) are only this step's
-        // six scale loads (behind MFMAs 8..12).  lgkmcnt(0): this wave's LDS reads of stage
-        // `cur` are complete.  A bare s_barrier: these waits are all the ordering needed.
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(BLOCK ? 6 : 0));
+        // barrier 2.  Vector-memory operations retire in order; block u + 1's last copy is a
+        // weight copy behind the last MFMAs of the step before (or a deferred one behind MFMA
+        // 11 of a tile's first step).  Younger than it are only the four activation copies of
+        // block u + 2, which stay in flight.  lgkmcnt(0): this wave's LDS reads of block u's
+        // weights and scales are complete.  A bare s_barrier: these waits are all the
+        // ordering that is needed.
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(last ? 0 : 4));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1164,19 +1179,34 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (BLOCK) {
+          sc_prev = sc;
+          sc = sfa_cur[i] * sfb_j;
+        }
         if (j + 1 < NI) {
           if (i == 0) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
         } else {
           // activation fragment i has had its last use in this step: refill it from block u + 1
           af[i] = read_frag(sn + a_base + i * 16 * 128);
           if (i == 0) b_nxt = read_frag(sn + b_base);
-          if (!last) copy_a(i, cur, kn2 * 128, off_a2);
+          if (!last && i < NBW) copy_b(i, cur, kn2 * 128, off_b2);
+          if constexpr (BLOCK) {
+            // so has its scale (`sc` holds the product), and the weight scales (`sfb_j`)
+            sfa_cur[i] = read_sfa(cur ^ 1, i);
+            if (i == 0) sfb_lo = read_sfb(cur ^ 1, 0);
+            if (i == 1) sfb_hi = read_sfb(cur ^ 1, 1);
+            if (i == 0 && !last) copy_scales(cur, kn2, sc_voff2);
+          }
         }
-        if (idx < NBW) copy_b(idx, cur ^ 1, kn * 128);
-        if (first && idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+        if constexpr (first) {
+          if (idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+          if (idx >= 8 && idx < 8 + NBW) copy_b(idx - 8, cur ^ 1, kn * 128, off_b);
+          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
+          if (idx >= 12 && idx < 16) copy_a(idx - 12, cur, kn2 * 128, off_a2);
+        } else if constexpr (!last) {
+          if (idx >= 4 && idx < 8) copy_a(idx - 4, cur, kn2 * 128, off_a2);
+        }
         if constexpr (BLOCK) {
-          sc_prev = sc;
-          sc = sfa_cur[i] * sfb_j;
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
             acc[pi][pj][0] = __builtin_fmaf(part_prev[0], sc_prev, acc[pi][pj][0]);
@@ -1184,11 +1214,6 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
             acc[pi][pj][2] = __builtin_fmaf(part_prev[2], sc_prev, acc[pi][pj][2]);
             acc[pi][pj][3] = __builtin_fmaf(part_prev[3], sc_prev, acc[pi][pj][3]);
           }
-          if (idx == 8) {
-            sfb_lo_nxt = load_sfb(sfb_col_lo, kn);
-            sfb_hi_nxt = load_sfb(sfb_col_hi, kn);
-          }
-          if (idx >= 9 && idx < 9 + MI) sfa_nxt[idx - 9] = load_sfa(idx - 9, kn);
           part_prev = part;
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -1200,10 +1225,6 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
       acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
-#pragma unroll
-      for (int i = 0; i < MI; ++i) sfa_cur[i] = sfa_nxt[i];
-      sfb_lo = sfb_lo_nxt;
-      sfb_hi = sfb_hi_nxt;
       jsw = jsw_nxt;
     }
   };
@@ -1218,24 +1239,28 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   int par = 0;  // stage that holds K block 0 of the current tile
 
   off_a = off_a2 = a_offset(m0);
-  off_b = b_offset(n0);
-  set_scales(m0, n0);
+  off_b = off_b2 = b_offset(n0);
+  if constexpr (BLOCK) {
+    sc_voff = sc_voff2 = scale_offset(m0, n0);
+    set_scale_split(n0);
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
 #pragma unroll
-  for (int j = 0; j < NBW; ++j) copy_b(j, 0, 0);
-  if constexpr (BLOCK) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i) sfa_cur[i] = load_sfa(i, 0);
-    sfb_lo = load_sfb(sfb_col_lo, 0);
-    sfb_hi = load_sfb(sfb_col_hi, 0);
-    jsw = jsw_nxt;
-  }
+  for (int j = 0; j < NBW; ++j) copy_b(j, 0, 0, off_b);
+  if constexpr (BLOCK) copy_scales(0, 0, sc_voff);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int i = 0; i < MI; ++i) af[i] = read_frag(smem + a_base + i * 16 * 128);
   b_cur = read_frag(smem + b_base);
+  if constexpr (BLOCK) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) sfa_cur[i] = read_sfa(0, i);
+    sfb_lo = read_sfb(0, 0);
+    sfb_hi = read_sfb(0, 1);
+    jsw = jsw_nxt;
+  }
 
   while (true) {
 #pragma unroll
@@ -1252,19 +1277,25 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const int nn0 = has_next ? tn * BN : p.tiles_n * BN;
 
     // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
-    const uint32_t off_a_next = a_offset(nm0);
+    const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
+    uint32_t sc_voff_next = OOB;
+    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
     k_step(par, 1, 2, std::true_type{}, std::false_type{});
     for (int kb = 1; kb + 1 < nkb; ++kb) {
       const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
       off_a2 = pen ? off_a_next : off_a2;
+      off_b2 = pen ? off_b_next : off_b2;
+      sc_voff2 = pen ? sc_voff_next : sc_voff2;
       k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
     }
-    // last K block: the weight copies and the scales issued now belong to the next tile
+    // last K block: the scales read behind its last MFMAs are the next tile's; its copies (the
+    // next tile's second block) wait for the next tile's first step
     const int last_stage = (nkb - 1 + par) & 1;
-    off_b = b_offset(nn0);
-    set_scales(nm0, nn0);
+    if constexpr (BLOCK) set_scale_split(nn0);
     k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
     off_a = off_a2;
+    off_b = off_b2;
+    sc_voff = sc_voff2;
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
