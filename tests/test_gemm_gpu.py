@@ -37,8 +37,10 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
-# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258], ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256"])
+# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel,
+# 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 16, 32],
+                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "stream16", "stream32"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -52,7 +54,7 @@ def tile(request):
 def test_int8_accumulators_bit_exact(gpu, load_path, tile, mnk):
     from sglang_amd.sgl_kernel import int8_mm_i32
 
-    if tile >= 192 and not load_path:
+    if (tile >= 192 or tile in (16, 32)) and not load_path:
         pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
     say("int8 acc", mnk, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
@@ -104,7 +106,7 @@ def make_block_case(m, n, k, seed, outliers=False):
 def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
-    if tile >= 192 and not load_path:
+    if (tile >= 192 or tile in (16, 32)) and not load_path:
         pytest.skip("the 256x256 kernel only has the direct-to-LDS path")
     say("fp8_blockwise", mnk, out_dtype, "direct" if load_path else "regs", "tile", tile)
     m, n, k = mnk
@@ -229,6 +231,51 @@ def test_decode_kernel_split_k(gpu, splits, mnk):
     acc_ref = O.int8_mm_i32(a8, w8.t())
     acc = int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()
     assert torch.equal(acc, acc_ref)
+    sa8 = sa * 0.01
+    ref = O.int8_scaled_mm(a8, w8.t(), sa8, sb, torch.bfloat16, bias)
+    out = int8_scaled_mm(a8.to(gpu), w8.to(gpu).t(), sa8.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
+def stream_rows(request):
+    from sglang_amd import _lib
+
+    _lib.load().sglq_debug_force_tile(request.param)
+    yield request.param
+    _lib.load().sglq_debug_force_tile(0)
+
+
+@pytest.mark.parametrize("mnk", [(1, 128, 512), (1, 7168, 2048), (7, 2112, 7168), (16, 264, 640), (17, 136, 1024), (32, 4096, 512),
+                                 (8, 48, 16384), (3, 24, 896)])
+def test_decode_kernel_full_k(gpu, stream_rows, mnk):
+    """M <= 32 with enough weight rows runs on the kernel whose blocks own all of K and add
+    their four waves' partial sums in LDS (forced here for small N as well): every kind,
+    N not a multiple of the block's rows, K blocks not a multiple of four."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32, int8_scaled_mm
+
+    say("full-K decode kernel", mnk, "rows per block", stream_rows)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m * n + k, outliers=True)
+    ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.float16)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    g = torch.Generator().manual_seed(m + n)
+    sa = torch.rand((m, 1), generator=g) * 0.05 + 0.01
+    sb = torch.rand((n, 1), generator=g) * 0.001 + 0.0005
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16)
+    ref = O.fp8_scaled_mm(xq, wq.t(), sa, sb, torch.float32, bias, acc_dtype=torch.float64)
+    out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    a8, w8 = rand_i8((m, k), 3), rand_i8((n, k), 4)
+    if m > 1:
+        a8[1] = -128
+        w8[n - 1] = -128
+    acc = int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()
+    assert torch.equal(acc, O.int8_mm_i32(a8, w8.t()))
     sa8 = sa * 0.01
     ref = O.int8_scaled_mm(a8, w8.t(), sa8, sb, torch.bfloat16, bias)
     out = int8_scaled_mm(a8.to(gpu), w8.to(gpu).t(), sa8.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
