@@ -57,6 +57,16 @@ int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* outpu
                                     int64_t s_stride_row, int64_t s_stride_col, float eps, float int8_min,
                                     float int8_max, void* stream);
 
+/* Replaces torch.ops.sgl_kernel.sgl_per_tensor_quant_fp8
+ * (sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:96-123; schema
+ * common_extension.cc:126-127): one scale for the whole tensor of num_elements
+ * elements.  is_static == 0: *output_s must be zero on entry (the reference's
+ * caller allocates it with zeros, fp8_kernel.py:1252) and receives
+ * max|x| / 448 through an atomic max; is_static != 0: *output_s is read only.
+ * Codes are max(min(x * (1 / *output_s), 448), -448) rounded to e4m3fn. */
+int sglq_per_tensor_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                              int64_t num_elements, int is_static, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
  * (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:166-227; schema
  * common_extension.cc:129-130), zero rows giving zero codes as in the

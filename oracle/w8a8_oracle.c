@@ -135,6 +135,21 @@ void oracle_token_quant_fp8(const void* x, int dtype, int64_t rows, int64_t cols
   }
 }
 
+/* per_tensor_quant_fp8.cu:10-123.  is_static == 0: *s = max|x| / 448 first (:44). */
+void oracle_tensor_quant_fp8(const void* x, int dtype, int64_t n, int is_static, uint8_t* q, float* s) {
+  if (!is_static) {
+    float amax = 0.f; /* :13 */
+    for (int64_t j = 0; j < n; ++j) amax = fmaxf(amax, fabsf(load_elem(x, dtype, j)));
+    *s = amax / 448.0f;
+  }
+  float inv = 1.0f / *s; /* :56 */
+  for (int64_t j = 0; j < n; ++j) {
+    float v = load_elem(x, dtype, j) * inv;
+    v = fmaxf(fminf(v, 448.0f), -448.0f); /* :70; fminf(NaN, 448) = 448 */
+    q[j] = oracle_e4m3fn_encode(v);
+  }
+}
+
 static float e4m3fn_decode(uint8_t c) {
   int e = (c >> 3) & 0xf;
   int m = c & 7;

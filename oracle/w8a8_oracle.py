@@ -187,6 +187,26 @@ def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q.to(FP8), scale
 
 
+def per_tensor_quant_fp8(x: torch.Tensor, scale: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-123.
+
+    Dynamic (scale is None): scale = max|x| / 448 (:44, the maximum over the blocks'
+    `max / 448` equals the divide of the overall maximum: the divide is monotonic).
+    Then, for both modes: inv = 1 / scale (:56); q = max(min(x * inv, 448), -448)
+    (:70,:88) -> e4m3fn RNE.  fminf / fmaxf return their non-NaN operand, so the
+    NaN of 0 * inf (all-zero tensor, dynamic) becomes +448."""
+    xf = x.to(torch.float32)
+    if scale is None:
+        scale = (xf.abs().amax() / torch.tensor(FP8_E4M3_MAX, dtype=torch.float32)).reshape(1)
+    else:
+        scale = scale.to(torch.float32).reshape(1)
+    inv = torch.tensor(1.0, dtype=torch.float32) / scale
+    v = xf * inv
+    v = torch.where(torch.isnan(v), torch.full_like(v, FP8_E4M3_MAX), torch.minimum(v, torch.tensor(FP8_E4M3_MAX)))
+    v = torch.maximum(v, torch.tensor(-FP8_E4M3_MAX))
+    return v.to(FP8), scale
+
+
 # ---------------------------------------------------------------------------
 # a4  block-scaled FP8 GEMM
 # ---------------------------------------------------------------------------

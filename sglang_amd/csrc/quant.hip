@@ -362,6 +362,82 @@ __global__ __launch_bounds__(256) void token_quant_generic_kernel(const char* __
 }
 
 // ---------------------------------------------------------------------------
+// Per-tensor FP8 quantization (sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu): one scale
+// for the whole tensor.  Dynamic mode runs tensor_absmax_kernel first: every block folds
+// its share of the input into one abs-max, divides by 448 and merges it into *s with an
+// unsigned integer atomic max on the float's bit pattern (non-negative floats order like
+// their bits; *s must be zero on entry, as the reference's caller allocates it).  Both
+// modes then run tensor_quant_kernel: q = max(min(x * (1 / *s), 448), -448) -> e4m3fn.
+// VEC = false: element-wise accesses, for buffers that are not 16-byte aligned.
+// ---------------------------------------------------------------------------
+template <int DT>
+SGLQ_DEV float load_elem(const char* x, int64_t idx) {
+  if constexpr (DT == SGLQ_BF16) return u2f((uint32_t)reinterpret_cast<const uint16_t*>(x)[idx] << 16);
+  else if constexpr (DT == SGLQ_FP16) return (float)reinterpret_cast<const _Float16*>(x)[idx];
+  else return reinterpret_cast<const float*>(x)[idx];
+}
+
+template <int DT, bool VEC>
+__global__ __launch_bounds__(256) void tensor_absmax_kernel(const char* __restrict__ x, float* __restrict__ s, int64_t n) {
+  __shared__ uint32_t red[4];
+  const int64_t nchunks = VEC ? (n >> 3) : 0;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  uint32_t mb = 0;
+  int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; c + 3 * stride < nchunks; c += 4 * stride) {  // four independent loads in flight per lane
+    Chunk8<DT> ch[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ch[u].load(x + (c + u * stride) * Chunk8<DT>::kBytes);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) mb = umax(mb, ch[u].amax_bits());
+  }
+  for (; c < nchunks; c += stride) {
+    Chunk8<DT> ch;
+    ch.load(x + c * Chunk8<DT>::kBytes);
+    mb = umax(mb, ch.amax_bits());
+  }
+  for (int64_t j = (nchunks << 3) + (int64_t)blockIdx.x * 256 + threadIdx.x; j < n; j += stride)
+    mb = umax(mb, f2u(load_elem<DT>(x, j)) & 0x7fffffffu);
+  mb = wave_umax(mb);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mb;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mb = umax(umax(red[0], red[1]), umax(red[2], red[3]));
+    const uint32_t mine = f2u(u2f(mb) / 448.0f);  // per_tensor_quant_fp8.cu:44
+    // Atomics on one address serialise in L2 (about 12 ns each, measured): skip the update when the
+    // value already there is not smaller.  It only ever grows, so a stale read costs an atomic, never a result.
+    unsigned int* sp = reinterpret_cast<unsigned int*>(s);
+    if (mine > __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(sp, mine);
+  }
+}
+
+SGLQ_DEV float clamp_like_fminf_fmaxf(float v) {
+  // fminf / fmaxf return the non-NaN operand: NaN (0 * inf, all-zero tensor in dynamic mode)
+  // becomes +448 as in per_tensor_quant_fp8.cu:70; fmed3 would not do that.
+  return __builtin_fmaxf(__builtin_fminf(v, 448.0f), -448.0f);
+}
+
+template <int DT, bool VEC>
+__global__ __launch_bounds__(256) void tensor_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
+                                                           const float* __restrict__ s, int64_t n) {
+  const float inv = 1.0f / *s;  // per_tensor_quant_fp8.cu:56
+  const int64_t nchunks = VEC ? (n >> 3) : 0;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += stride) {
+    Chunk8<DT> ch;
+    ch.load(x + c * Chunk8<DT>::kBytes);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = clamp_like_fminf_fmaxf(ch.get(i) * inv);
+    *reinterpret_cast<v2u*>(q + c * 8) = Fp8Pack::pack(v);
+  }
+  for (int64_t j = (nchunks << 3) + (int64_t)blockIdx.x * 256 + threadIdx.x; j < n; j += stride) {
+    const float y = clamp_like_fminf_fmaxf(load_elem<DT>(x, j) * inv);
+    q[j] = (char)(cvt_pk_e4m3<false>(y, y, 0) & 0xffu);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Host-side dispatch
 // ---------------------------------------------------------------------------
 static int check_launch(const char* what) {
@@ -512,6 +588,56 @@ static int token_quant_entry(const char* name, const void* input, int in_dtype, 
   return SGLQ_EUNSUPPORTED;
 }
 
+template <int DT>
+static void launch_tensor_quant(const void* x, void* q, float* s, int64_t n, bool is_static, hipStream_t st) {
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
+  const int64_t work = vec ? (n + 7) / 8 : n;
+  int64_t blocks = (work + 255) / 256;
+  if (blocks > 4096) blocks = 4096;  // grid-stride beyond that: 16 blocks per CU
+  if (blocks < 1) blocks = 1;
+  int64_t max_blocks = (work + 1023) / 1024;  // the abs-max pass: four chunks per lane and trip, one atomic per block
+  if (max_blocks > 1024) max_blocks = 1024;
+  if (max_blocks < 1) max_blocks = 1;
+  const dim3 grid((uint32_t)blocks), grid_max((uint32_t)max_blocks), block(256);
+  const char* xc = static_cast<const char*>(x);
+  char* qc = static_cast<char*>(q);
+  if (vec) {
+    if (!is_static) tensor_absmax_kernel<DT, true><<<grid_max, block, 0, st>>>(xc, s, n);
+    tensor_quant_kernel<DT, true><<<grid, block, 0, st>>>(xc, qc, s, n);
+  } else {
+    if (!is_static) tensor_absmax_kernel<DT, false><<<grid_max, block, 0, st>>>(xc, s, n);
+    tensor_quant_kernel<DT, false><<<grid, block, 0, st>>>(xc, qc, s, n);
+  }
+}
+
+static int tensor_quant_entry(const void* input, int in_dtype, void* output_q, float* output_s, int64_t num_elements,
+                              int is_static, void* stream) {
+  const char* name = "sgl_per_tensor_quant_fp8";
+  if (num_elements < 0) {
+    set_error("%s: negative element count", name);
+    return SGLQ_EINVAL;
+  }
+  if (!output_s) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_elements > 0 && (!input || !output_q)) {
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_elements == 0) return SGLQ_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (in_dtype) {
+    case SGLQ_BF16: launch_tensor_quant<SGLQ_BF16>(input, output_q, output_s, num_elements, is_static != 0, st); break;
+    case SGLQ_FP16: launch_tensor_quant<SGLQ_FP16>(input, output_q, output_s, num_elements, is_static != 0, st); break;
+    case SGLQ_FP32: launch_tensor_quant<SGLQ_FP32>(input, output_q, output_s, num_elements, is_static != 0, st); break;
+    default:
+      set_error("%s: input dtype must be bf16, fp16 or fp32", name);
+      return SGLQ_EUNSUPPORTED;
+  }
+  return check_launch(name);
+}
+
 }  // namespace sglq
 
 extern "C" int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
@@ -542,4 +668,9 @@ extern "C" int sglq_per_token_quant_int8(const void* input, int in_dtype, void* 
                                          void* row_sum, int64_t num_tokens, int64_t hidden, void* stream) {
   return sglq::token_quant_entry<sglq::MODE_INT8>("per_token_quant_int8", input, in_dtype, output_q, output_s,
                                                   row_sum, num_tokens, hidden, stream);
+}
+
+extern "C" int sglq_per_tensor_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                         int64_t num_elements, int is_static, void* stream) {
+  return sglq::tensor_quant_entry(input, in_dtype, output_q, output_s, num_elements, is_static, stream);
 }

@@ -6,7 +6,9 @@ from __future__ import annotations
 
 import torch
 
-from ..sgl_kernel import sgl_per_token_group_quant_fp8, sgl_per_token_quant_fp8
+from typing import Optional
+
+from ..sgl_kernel import sgl_per_tensor_quant_fp8, sgl_per_token_group_quant_fp8, sgl_per_token_quant_fp8
 
 # gfx950 implements the OCP formats: e4m3fn with maximum 448 (fp8_kernel.py:71-85
 # selects the fnuz/224 variant only for gfx94x).
@@ -75,3 +77,31 @@ def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
     x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
     sgl_per_token_quant_fp8(x, x_q, x_s)
     return x_q, x_s
+
+
+def scaled_fp8_quant(
+    input: torch.Tensor,
+    scale: Optional[torch.Tensor] = None,
+    num_token_padding: Optional[int] = None,
+    use_per_token_if_dynamic: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """fp8_kernel.py:1233-1266 (the sgl_kernel branch): per-token dynamic, per-tensor
+    dynamic (scale starts at zero, the op merges max|x| / 448 into it) or per-tensor
+    static quantization of a 2-D tensor; rows past input's are left unwritten."""
+    assert input.ndim == 2, f"Expected 2D input tensor, got {input.ndim}D"
+    shape = input.shape
+    if num_token_padding:
+        shape = (max(num_token_padding, input.shape[0]), shape[1])
+    output = torch.empty(shape, device=input.device, dtype=fp8_dtype)
+    q = output[: input.shape[0]]
+    if scale is None:
+        if use_per_token_if_dynamic:
+            scale = torch.empty((shape[0], 1), device=input.device, dtype=torch.float32)
+            sgl_per_token_quant_fp8(input, q, scale[: input.shape[0]])
+        else:
+            scale = torch.zeros(1, device=input.device, dtype=torch.float32)
+            sgl_per_tensor_quant_fp8(input, q, scale, is_static=False)
+    else:
+        assert scale.numel() == 1, f"Expected scalar scale, got numel={scale.numel()}"
+        sgl_per_tensor_quant_fp8(input, q, scale, is_static=True)
+    return output, scale

@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
-from .fp8_kernel import per_token_group_quant_fp8, sglang_per_token_quant_fp8
+from .fp8_kernel import per_token_group_quant_fp8, scaled_fp8_quant, sglang_per_token_quant_fp8
 
 
 def w8a8_block_fp8_linear(
@@ -47,11 +47,15 @@ def apply_fp8_linear(
     apply_fp8_linear that ends in fp8_scaled_mm (fp8_utils.py:693,720-733).
 
     weight is the [K, N] transposed view, weight_scale one fp32 per output channel."""
-    if input_scale is not None:
-        raise NotImplementedError("static activation scales are not built")
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[1]]
-    qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
+    if input_scale is not None:
+        # static per-tensor activation scale (scaled_fp8_quant, fp8_utils.py:569-573); the GEMM
+        # takes one scale per row, so the scalar is repeated
+        qinput, x_scale = scaled_fp8_quant(input_2d, input_scale)
+        x_scale = x_scale.reshape(1, 1).expand(input_2d.shape[0], 1).contiguous()
+    else:
+        qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
     assert weight_scale.numel() == weight.shape[1], "cutlass w8a8 fp8 sgl-kernel only supports per-channel scale"
     output = fp8_scaled_mm(qinput, weight, x_scale, weight_scale, out_dtype=input.dtype, bias=bias)
     return output.view(*output_shape)

@@ -8,6 +8,7 @@ from .gemm import (
     int8_scaled_mm,
     sgl_per_token_group_quant_fp8,
     sgl_per_token_group_quant_int8,
+    sgl_per_tensor_quant_fp8,
     sgl_per_token_quant_fp8,
 )
 
@@ -18,5 +19,6 @@ __all__ = [
     "int8_scaled_mm",
     "sgl_per_token_group_quant_fp8",
     "sgl_per_token_group_quant_int8",
+    "sgl_per_tensor_quant_fp8",
     "sgl_per_token_quant_fp8",
 ]

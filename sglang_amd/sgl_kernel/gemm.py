@@ -118,6 +118,17 @@ def check_token_quant_fp8(input, output_q, output_s, require_cuda=True):
     _check(input.size(1) % 8 == 0, f"Hidden dimension must be divisible by 8, but got {input.size(1)}")
 
 
+def check_tensor_quant_fp8(input, output_q, output_s, require_cuda=True):
+    """per_tensor_quant_fp8.cu:96-99 (CHECK_INPUT: CUDA and contiguous) plus what the kernels assume."""
+    for name, t in (("input", input), ("output_q", output_q), ("output_s", output_s)):
+        if require_cuda:
+            _check(t.is_cuda, f"{name} must be a CUDA tensor")
+        _check(t.is_contiguous(), f"{name} must be contiguous")
+    _check(input.dtype in DTYPE_CODE, "input must be Float, Half or BFloat16")
+    _check(output_q.dtype == FP8 and output_q.numel() == input.numel(), "output_q must be Float8_e4m3fn with input's element count")
+    _check(output_s.dtype == torch.float32 and output_s.numel() >= 1, "output_s must hold one Float32")
+
+
 # ---------------------------------------------------------------------------
 # op implementations (CUDA dispatch key = ROCm device tensors)
 # ---------------------------------------------------------------------------
@@ -210,6 +221,17 @@ def _sgl_per_token_quant_fp8_impl(input, output_q, output_s):
     _lib.check(rc, "sgl_per_token_quant_fp8")
 
 
+def _sgl_per_tensor_quant_fp8_impl(input, output_q, output_s, is_static):
+    check_tensor_quant_fp8(input, output_q, output_s)
+    if input.numel() == 0:
+        return
+    lib = _lib.load()
+    rc = lib.sglq_per_tensor_quant_fp8(
+        input.data_ptr(), DTYPE_CODE[input.dtype], output_q.data_ptr(), output_s.data_ptr(), input.numel(),
+        1 if is_static else 0, _lib.stream_ptr(input.device))
+    _lib.check(rc, "sgl_per_tensor_quant_fp8")
+
+
 _SCHEMAS = {
     # sgl-kernel/csrc/common_extension.cc:101-130
     "int8_scaled_mm": "(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? bias) -> Tensor",
@@ -218,6 +240,7 @@ _SCHEMAS = {
     "sgl_per_token_group_quant_fp8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s, int group_size, float eps, float fp8_min, float fp8_max, bool scale_ue8m0) -> ()",
     "sgl_per_token_group_quant_int8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s, int group_size, float eps, float int8_min, float int8_max) -> ()",
     "sgl_per_token_quant_fp8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s) -> ()",
+    "sgl_per_tensor_quant_fp8": "(Tensor input, Tensor(a!) output_q, Tensor(b!) output_s, bool is_static) -> ()",
 }
 _IMPLS = {
     "int8_scaled_mm": _int8_scaled_mm_impl,
@@ -226,6 +249,7 @@ _IMPLS = {
     "sgl_per_token_group_quant_fp8": _sgl_per_token_group_quant_fp8_impl,
     "sgl_per_token_group_quant_int8": _sgl_per_token_group_quant_int8_impl,
     "sgl_per_token_quant_fp8": _sgl_per_token_quant_fp8_impl,
+    "sgl_per_tensor_quant_fp8": _sgl_per_tensor_quant_fp8_impl,
 }
 
 _library = torch.library.Library("sgl_kernel", "FRAGMENT")
@@ -280,6 +304,11 @@ def sgl_per_token_group_quant_int8(
 
 def sgl_per_token_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
     torch.ops.sgl_kernel.sgl_per_token_quant_fp8.default(input, output_q, output_s)
+
+
+def sgl_per_tensor_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor, is_static: bool) -> None:
+    """sgl-kernel/python/sgl_kernel/gemm.py:129-137."""
+    torch.ops.sgl_kernel.sgl_per_tensor_quant_fp8.default(input, output_q, output_s, is_static)
 
 
 def int8_mm_i32(mat_a: torch.Tensor, mat_b: torch.Tensor) -> torch.Tensor:

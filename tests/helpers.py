@@ -39,6 +39,15 @@ def c_token_quant_fp8(lib, x: torch.Tensor):
     return q, s.reshape(rows, 1)
 
 
+def c_tensor_quant_fp8(lib, x: torch.Tensor, scale=None):
+    x = x.contiguous()
+    q = torch.empty(x.shape, dtype=torch.uint8)
+    s = torch.zeros(1, dtype=torch.float32) if scale is None else scale.clone().float().reshape(1)
+    lib.oracle_tensor_quant_fp8(raw_ptr(x), DT[x.dtype], ctypes.c_int64(x.numel()), ctypes.c_int(0 if scale is None else 1),
+                                raw_ptr(q), raw_ptr(s))
+    return q, s
+
+
 def fp8_bits(t: torch.Tensor) -> torch.Tensor:
     return t.view(torch.uint8)
 

@@ -160,5 +160,10 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == 1 and b"multiple of 16" in lib.sglq_last_error()
     rc = lib.sglq_fp8_blockwise_scaled_mm(p, 128, p, 128, p, 1, 4, p, 1, 1, p, 8, 2, 4, 8, 128, None, 0, None)
     assert rc == 1 and b"out_dtype" in lib.sglq_last_error()
+    rc = lib.sglq_per_tensor_quant_fp8(p, 7, p, p, 16, 0, None)
+    assert rc == 2 and b"dtype" in lib.sglq_last_error()
+    rc = lib.sglq_per_tensor_quant_fp8(p, 0, p, None, 16, 0, None)
+    assert rc == 1 and b"scale" in lib.sglq_last_error()
+    assert lib.sglq_per_tensor_quant_fp8(None, 0, None, p, 0, 1, None) == 0
     # empty problems are a no-op
     assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0

@@ -9,7 +9,8 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_bits_equal, c_group_quant_fp8, c_token_quant_fp8, c_token_quant_int8, fp8_bits
+from helpers import (assert_bits_equal, c_group_quant_fp8, c_tensor_quant_fp8, c_token_quant_fp8, c_token_quant_int8,
+                     fp8_bits)
 from oracle import w8a8_oracle as O
 
 FP8 = torch.float8_e4m3fn
@@ -199,6 +200,41 @@ def test_token_fp8_closed_form():
     q, s = O.per_token_quant_fp8(x)
     assert_bits_equal(s, scale.reshape(9, 1), "scale")
     assert torch.equal(q.float(), O.e4m3fn_decode(codes))
+
+
+# ------------------------------------------------------------------ f2 fp8 per tensor
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_tensor_fp8_quant_vs_c_and_formula(c_oracle, dtype):
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn((37, 203), generator=g) * 3).to(dtype)
+    for scale in (None, torch.tensor([0.0123])):
+        q, s = O.per_tensor_quant_fp8(x, scale)
+        qc, sc = c_tensor_quant_fp8(c_oracle, x, scale)
+        assert_bits_equal(s, sc, "scale")
+        assert_bits_equal(fp8_bits(q), qc, "codes")
+        # the reference test's formula (sgl-kernel/tests/test_per_tensor_quant_fp8.py:28-35)
+        want = (x.float() * s.reciprocal()).clamp(-448, 448).to(FP8)
+        assert_bits_equal(q, want, "codes vs reference-test formula")
+    q, s = O.per_tensor_quant_fp8(x)
+    assert s.item() == (x.float().abs().max() / 448).item()
+    assert float(q.float().abs().max()) == 448.0
+
+
+def test_tensor_fp8_closed_form_and_zero_tensor(c_oracle):
+    # x = value(code) * 2^e with a +-448 present: scale is 2^e exactly, its inverse too, so the codes come back
+    x, codes, scale = make_closed_form_groups(1, 1, group=512, seed=12)
+    q, s = O.per_tensor_quant_fp8(x)
+    assert_bits_equal(s, scale.reshape(1), "scale")
+    assert torch.equal(q.float(), O.e4m3fn_decode(codes))
+    # static scale of 2^-3: codes of x / 2^-3
+    q, s = O.per_tensor_quant_fp8(torch.tensor([[0.5, -1.0, 100.0, 0.0]]), torch.tensor([0.125]))
+    assert q.float().tolist() == [[4.0, -8.0, 448.0, 0.0]]
+    # all-zero tensor, dynamic: scale 0, 0 * inf = NaN, fminf / fmaxf turn it into +448 (per_tensor_quant_fp8.cu:70)
+    z = torch.zeros(3, 8)
+    q, s = O.per_tensor_quant_fp8(z)
+    qc, sc = c_tensor_quant_fp8(c_oracle, z)
+    assert s.item() == 0.0 and sc.item() == 0.0
+    assert fp8_bits(q).unique().tolist() == [0x7E] and qc.unique().tolist() == [0x7E]
 
 
 # ------------------------------------------------------------------ GEMMs

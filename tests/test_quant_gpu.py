@@ -170,6 +170,78 @@ def test_token_quant_fp8_bit_exact(gpu, dtype, shape):
     assert_bits_equal(q, q_ref, "codes")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 8), (3, 7), (128, 512), (512, 4096), (33, 1003), (2048, 14336)])
+def test_tensor_quant_fp8_bit_exact(gpu, dtype, shape):
+    """sgl_per_tensor_quant_fp8, dynamic and static, against the oracle bit for bit (shapes of
+    sgl-kernel/tests/test_per_tensor_quant_fp8.py:40-43 plus lengths that are not a multiple of 8)."""
+    from sglang_amd.quantization.fp8_kernel import scaled_fp8_quant
+
+    say("tensor_quant", dtype, shape)
+    m, k = shape
+    x = (O.gen_activation(m, k, seed=m + 3 * k, outliers=True).float() * 1.7).to(dtype)
+    q_ref, s_ref = O.per_tensor_quant_fp8(x)
+    q, s = scaled_fp8_quant(x.to(gpu))
+    assert_bits_equal(s, s_ref, "dynamic scale")
+    assert_bits_equal(q, q_ref, "dynamic codes")
+    static = torch.tensor([0.0371], dtype=torch.float32)
+    q_ref, _ = O.per_tensor_quant_fp8(x, static)
+    q, s = scaled_fp8_quant(x.to(gpu), static.to(gpu))
+    assert_bits_equal(q, q_ref, "static codes")
+    assert s.item() == static.item()
+
+
+def test_tensor_quant_fp8_unaligned_zero_and_padding(gpu):
+    from sglang_amd.quantization.fp8_kernel import scaled_fp8_quant
+    from sglang_amd.sgl_kernel import sgl_per_tensor_quant_fp8
+
+    # a view that starts 2 bytes into an allocation: the element-wise kernels
+    base = O.gen_activation(5, 1001, seed=9).to(torch.bfloat16).flatten()
+    xg = base.to(gpu)[1:]
+    q = torch.empty(xg.numel() + 1, dtype=FP8, device=gpu)[1:]
+    s = torch.zeros(1, dtype=torch.float32, device=gpu)
+    sgl_per_tensor_quant_fp8(xg, q, s, False)
+    q_ref, s_ref = O.per_tensor_quant_fp8(base[1:])
+    assert_bits_equal(s, s_ref, "scale, unaligned")
+    assert_bits_equal(q, q_ref, "codes, unaligned")
+    # all-zero tensor, dynamic: scale 0 and the +448 codes of the reference's fminf / fmaxf clamp
+    z = torch.zeros((4, 64), dtype=torch.float16, device=gpu)
+    q, s = scaled_fp8_quant(z)
+    assert s.item() == 0.0 and fp8_bits(q).unique().tolist() == [0x7E]
+    # the scale is merged with an atomic max: a larger value already in the buffer survives
+    x = torch.ones((2, 16), dtype=torch.bfloat16, device=gpu)
+    q = torch.empty((2, 16), dtype=FP8, device=gpu)
+    s = torch.full((1,), 2.0, dtype=torch.float32, device=gpu)
+    sgl_per_tensor_quant_fp8(x, q, s, False)
+    assert s.item() == 2.0 and q.float().unique().tolist() == [0.5]
+    # num_token_padding only enlarges the output
+    x = O.gen_activation(3, 64, seed=1).to(torch.bfloat16)
+    q, s = scaled_fp8_quant(x.to(gpu), num_token_padding=17)
+    assert q.shape == (17, 64)
+    q_ref, s_ref = O.per_tensor_quant_fp8(x)
+    assert_bits_equal(q[:3], q_ref, "codes, padded output")
+    # per-token dynamic branch of the same helper
+    q, s = scaled_fp8_quant(x.to(gpu), use_per_token_if_dynamic=True)
+    q_ref, s_ref = O.per_token_quant_fp8(x)
+    assert_bits_equal(q, q_ref, "per-token codes")
+    assert_bits_equal(s, s_ref, "per-token scales")
+
+
+def test_tensor_quant_full_size_properties(gpu):
+    """8192 x 16384 (the largest activation of the configurations): quantizing the dequantized
+    tensor with the same static scale reproduces the codes; the maximum code is 448."""
+    from sglang_amd.quantization.fp8_kernel import scaled_fp8_quant
+
+    g = torch.Generator(device=gpu).manual_seed(7)
+    x = torch.randn((8192, 16384), generator=g, device=gpu, dtype=torch.bfloat16)
+    q, s = scaled_fp8_quant(x)
+    assert s.item() == (x.float().abs().max() / 448).item()
+    assert float(q[:64].float().abs().max()) <= 448.0 and int((fp8_bits(q) & 0x7F).max()) == 0x7E
+    deq = (q.float() * s).to(torch.float32)
+    q2, _ = scaled_fp8_quant(deq, s)
+    assert torch.equal(fp8_bits(q2), fp8_bits(q))
+
+
 def test_quant_empty_inputs(gpu):
     from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_quant_fp8
     from sglang_amd.quantization.int8_kernel import per_token_quant_int8
