@@ -143,6 +143,8 @@ def run_headline(args):
         layers.append((n, k, make_activation(m, k, 2000 + i, dev), wq, ws))
     torch.cuda.synchronize()
 
+    kernel_of = {}
+
     def step(tq=None, tg=None):
         for li, (n, k, x, wq, ws) in enumerate(layers):
             if tq is None:
@@ -151,6 +153,7 @@ def run_headline(args):
             else:
                 xq, xs = tq[li].time(lambda: sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True))
                 tg[li].time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+                kernel_of[li] = _lib.load().sglq_debug_last_gemm_kernel().decode()
 
     if args.calibrate_copy:
         src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
@@ -182,7 +185,7 @@ def run_headline(args):
     per_shape = []
     for (n, k, *_), a, b in zip(layers, tq, tg):
         qm, gm = a.total_ms() / args.steps, b.total_ms() / args.steps
-        per_shape.append({"N": n, "K": k, "quant_us": round(qm * 1e3, 1),
+        per_shape.append({"N": n, "K": k, "gemm_kernel": kernel_of.get(len(per_shape), ""), "quant_us": round(qm * 1e3, 1),
                           "quant_GBs": round(group_quant_bytes(m, k) / qm / 1e6, 1),
                           "gemm_us": round(gm * 1e3, 1), "gemm_TFLOPs": round(2.0 * m * n * k / gm / 1e9, 1)})
     big = max(range(len(layers)), key=lambda i: layers[i][1])  # the launch with the most activation bytes
@@ -199,10 +202,18 @@ def run_headline(args):
     torch.cuda.synchronize()
     quant_big_gbs = round(group_quant_bytes(m, layers[big][1]) / (iso.total_ms() / iso.count()) / 1e6, 1)
     del xs_iso
-    traffic = None
+    # the dominant kernel: the GEMM launch that takes the largest share of the step
+    dom = max(range(len(layers)), key=lambda i: tg[i].total_ms())
+    dom_n, dom_k = layers[dom][0], layers[dom][1]
+    dom_ms = tg[dom].total_ms() / tg[dom].count()
+    dom_flops = 2.0 * m * dom_n * dom_k
+    dom_tflops = dom_flops / (dom_ms * 1e-3) / 1e12
+    traffic = traffic_all = None
     tfile = ROOT / "profiles" / "headline_traffic.json"
     if tfile.exists():
-        traffic = json.loads(tfile.read_text()).get("gemm_hbm_bytes_per_launch_avg")
+        tj = json.loads(tfile.read_text())
+        traffic = tj.get("hbm_bytes_per_launch", {}).get(f"{dom_n}x{dom_k}")
+        traffic_all = tj.get("gemm_hbm_bytes_per_launch_avg")
     gemm_tflops = flops_step / (gemm_ms * 1e-3) / 1e12
     quant_gbs = qbytes_step / (quant_ms * 1e-3) / 1e9
     props = torch.cuda.get_device_properties(dev)
@@ -227,15 +238,23 @@ def run_headline(args):
             "value_is": "sum of 2MNK over the 5 GEMMs / wall time of the whole step (quant kernels included)",
         },
         "roofline": {
-            "kernel": "fp8_blockwise_scaled_mm (gemm_kernel<FP8_BLOCK>)",
+            "kernel": f"fp8_blockwise_scaled_mm: sglq::{kernel_of.get(dom, '')} (block-scaled FP8, bf16 out) on "
+                      f"{m} x {dom_n} x {dom_k}, the launch with the largest share of the step",
             "bound": "mfma",
-            "achieved": round(gemm_tflops, 2),
+            "achieved": round(dom_tflops, 2),
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(gemm_tflops / PEAK_FP8_TFLOPS, 4),
+            "frac": round(dom_tflops / PEAK_FP8_TFLOPS, 4),
             "traffic": traffic,
-            "avg_launch_ms": round(gemm_ms / len(layers), 4),
-            "flops_per_launch_avg": flops_step / len(layers),
+            "avg_launch_ms": round(dom_ms, 4),
+            "flops_per_launch": dom_flops,
+            "all_gemm_launches_of_the_step": {
+                "achieved": round(gemm_tflops, 2),
+                "frac": round(gemm_tflops / PEAK_FP8_TFLOPS, 4),
+                "avg_launch_ms": round(gemm_ms / len(layers), 4),
+                "flops_per_launch_avg": flops_step / len(layers),
+                "traffic_per_launch_avg": traffic_all,
+            },
         },
         "quant": {
             "kernel": "sgl_per_token_group_quant_fp8 (group_quant_kernel)",

@@ -129,12 +129,18 @@ int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, c
  * copy global memory straight into LDS with buffer loads, zero stages the same
  * bytes through registers.  Both must give identical results. */
 void sglq_debug_set_direct_lds(int on);
-/* Test hook: 0 = choose the GEMM tile by shape (default), 128 / 256 = always use
- * the 128x128 / 256x256 kernel. */
+/* Test hook: 0 = choose the GEMM kernel and tile by shape (default); 16 / 32 = the M <= 32
+ * kernel whose blocks own 16 / 32 weight rows and all of K; 64 = the M <= 64 split-K kernel;
+ * 128 = the 128x128 kernel; 256 = the plain 256x256 kernel; 258 = the pipelined 256x256
+ * kernel; 192 / 224 / 257 = the pipelined 4x2-wave kernel with tiles 192 / 224 / 256 wide.
+ * A kernel that does not apply to the shape falls through to the next one that does. */
 void sglq_debug_force_tile(int tile);
 /* Test hook: > 0 fixes the split-K factor of the M <= 64 kernels (0 = by shape);
  * with sglq_debug_force_tile(64 / 128 / 256): 64 = always the M <= 64 kernel where it applies. */
 void sglq_debug_force_splits(int splits);
+/* Test and measurement hook: name of the GEMM kernel that the calling thread's last GEMM
+ * call launched ("" before the first call); the string is static. */
+const char* sglq_debug_last_gemm_kernel(void);
 
 #ifdef __cplusplus
 }

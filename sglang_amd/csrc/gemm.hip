@@ -1667,6 +1667,7 @@ static int num_cus() {
 }
 
 static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
+static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
 
 template <int KIND, int OUT_DT>
 static void launch_reduce(GemmArgs& p, hipStream_t st);
@@ -1695,6 +1696,7 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   if (splits < 1) splits = 1;
   p.splits = splits;
   dim3 grid((uint32_t)(tiles * splits)), block(WAVES_M * WAVES_N * 64);
+  g_last_kernel = splits > 1 ? "gemm_kernel+splitk_reduce_kernel" : "gemm_kernel";
   if (g_use_dma) gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, true><<<grid, block, 0, st>>>(p);
   else gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, false><<<grid, block, 0, st>>>(p);
   if (splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
@@ -1714,8 +1716,13 @@ static void launch_big(GemmArgs& p, hipStream_t st) {
   const int tiles = p.tiles_m * p.tiles_n;
   const int blocks = tiles < num_cus() ? tiles : num_cus();
   // the pipelined kernel needs three K blocks; 256 forces the plain one (test hook)
-  if (g_force_tile != 256 && p.K >= 384) gemm_pipe_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
-  else gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  if (g_force_tile != 256 && p.K >= 384) {
+    g_last_kernel = "gemm_pipe_kernel";
+    gemm_pipe_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  } else {
+    g_last_kernel = "gemm_big_kernel";
+    gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  }
 }
 
 template <int KIND, int OUT_DT, int NI>
@@ -1725,6 +1732,7 @@ static void launch_wide(GemmArgs& p, hipStream_t st) {
   p.splits = 1;
   const int tiles = p.tiles_m * p.tiles_n;
   const int blocks = tiles < num_cus() ? tiles : num_cus();
+  g_last_kernel = NI == 6 ? "gemm_wide_kernel<6>" : NI == 7 ? "gemm_wide_kernel<7>" : "gemm_wide_kernel<8>";
   gemm_wide_kernel<KIND, OUT_DT, NI><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
 }
 
@@ -1754,6 +1762,7 @@ static void launch_reduce(GemmArgs& p, hipStream_t st) {
 
 template <int KIND, int MI, int OUT_DT>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
+  g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
   gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits)), dim3(256), 0, st>>>(p);
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
@@ -1801,6 +1810,7 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   p.tiles_m = 1;
   p.tiles_n = (p.N + 16 * nib - 1) / (16 * nib);
   const dim3 grid((uint32_t)p.tiles_n), block(256);
+  g_last_kernel = nib == 1 ? "gemm_stream_kernel<16 rows>" : "gemm_stream_kernel<32 rows>";
   if (p.M <= 16) {
     if (nib == 1) gemm_stream_kernel<KIND, 1, 1, OUT_DT><<<grid, block, 0, st>>>(p);
     else gemm_stream_kernel<KIND, 1, 2, OUT_DT><<<grid, block, 0, st>>>(p);
@@ -1909,6 +1919,7 @@ using namespace sglq;
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
+extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel; }
 
 extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                                             int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
