@@ -104,6 +104,21 @@ int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int6
                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                  int64_t workspace_bytes, void* stream);
 
+/* Replaces w8a8_block_int8_matmul, a Triton kernel in the reference
+ * (python/sglang/srt/layers/quantization/int8_kernel.py:212-425; there is no
+ * sgl_kernel C++ op): out[m,n] = sum_kb float(sum_{k in block kb} a[m,k] b[k,n])
+ * * sfa[m,kb] * sfb[kb, n/128], the int32 block sums exact, fp32 accumulation over
+ * kb, one rounding to out_dtype (Half or BFloat16).  Arguments as
+ * sglq_fp8_blockwise_scaled_mm with int8 operands; the reference passes the
+ * weight as stored, [N, K] row-major (= b with ldb = K), its scales
+ * [N/128, K/128] (sfb_stride_k = 1, sfb_stride_n = K/128) and row-major
+ * activation scales [M, K/128] (sfa_stride_m = K/128, sfa_stride_k = 1). */
+int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                  int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                  int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                  int64_t workspace_bytes, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.int8_scaled_mm
  * (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; schema common_extension.cc:101-104).
  * out = float(acc) * (scales_b[n] * scales_a[m]) + bias[n], acc exact int32.

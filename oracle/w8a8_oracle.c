@@ -185,6 +185,25 @@ void oracle_fp8_blockwise_mm(const uint8_t* a, const uint8_t* bt, const float* s
     }
 }
 
+/* int8_kernel.py:273-296 (w8a8_block_int8_matmul), evaluated in double:
+ * C[m,n] = sum_kb (sum_{k in kb} a[m,k] * bt[n,k]) * sfa[m,kb] * sfb[n/128, kb];
+ * a [M,K], bt [N,K], sfa [M,KB], sfb [NB,KB], all row-major. */
+void oracle_int8_blockwise_mm(const int8_t* a, const int8_t* bt, const float* sfa, const float* sfb,
+                              int64_t M, int64_t N, int64_t K, double* out) {
+  int64_t KB = (K + 127) / 128;
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      double acc = 0.0;
+      for (int64_t kb = 0; kb < KB; ++kb) {
+        int64_t p = 0;
+        int64_t k1 = (kb + 1) * 128 < K ? (kb + 1) * 128 : K;
+        for (int64_t k = kb * 128; k < k1; ++k) p += (int64_t)a[m * K + k] * (int64_t)bt[n * K + k];
+        acc += (double)p * (double)sfa[m * KB + kb] * (double)sfb[(n / 128) * KB + kb];
+      }
+      out[m * N + n] = acc;
+    }
+}
+
 /* int8_gemm_kernel.cu: int8 x int8 -> int32 accumulators, exact. */
 void oracle_int8_mm_i32(const int8_t* a, const int8_t* bt, int64_t M, int64_t N, int64_t K, int32_t* out) {
   for (int64_t m = 0; m < M; ++m)

@@ -245,6 +245,51 @@ def fp8_blockwise_scaled_mm(
 # ---------------------------------------------------------------------------
 # a5  INT8 scaled GEMM
 # ---------------------------------------------------------------------------
+def w8a8_block_int8_matmul(
+    a: torch.Tensor,
+    b_nk: torch.Tensor,
+    scales_a: torch.Tensor,
+    scales_b: torch.Tensor,
+    out_dtype: torch.dtype,
+    acc_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """python/sglang/srt/layers/quantization/int8_kernel.py:273-296 (the Triton kernel's loop):
+
+    C[m,n] = sum_kb float(sum_{k in kb} A[m,k] B[n,k]) * As[m,kb] * Bs[n//128, kb],
+
+    a int8 [M,K]; b_nk int8 [N,K]; scales_a [M, ceil(K/128)]; scales_b [ceil(N/128), ceil(K/128)].
+    The int32 block sums are exact (at most 128 * 128^2 < 2^24)."""
+    m, k = a.shape
+    n, k2 = b_nk.shape
+    assert k == k2
+    kb = (k + 127) // 128
+    af = a.to(torch.float64)
+    bf = b_nk.to(torch.float64)
+    sa = scales_a.to(acc_dtype)
+    sb_full = scales_b.to(acc_dtype).repeat_interleave(128, dim=0)[:n, :]  # [N, kb]
+    out = torch.zeros((m, n), dtype=acc_dtype)
+    for i in range(kb):
+        ks = slice(i * 128, min((i + 1) * 128, k))
+        p = (af[:, ks] @ bf[:, ks].t()).to(acc_dtype)  # exact
+        out += p * sa[:, i : i + 1] * sb_full[:, i].reshape(1, n)  # (dot * a_s) * b_s as :293
+    return out.to(out_dtype)
+
+
+def block_quant_weight_int8(w: torch.Tensor, block: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Harness-side block quantization of a weight to int8 (not on the measured path):
+    scale = absmax_block / 127 (0 -> 1), q = round-half-even(w / scale), scales [ceil(N/128), ceil(K/128)]."""
+    n, k = w.shape
+    nb, kb = (n + block - 1) // block, (k + block - 1) // block
+    wp = torch.zeros((nb * block, kb * block), dtype=torch.float32)
+    wp[:n, :k] = w.float()
+    blocks = wp.reshape(nb, block, kb, block)
+    amax = blocks.abs().amax(dim=(1, 3))
+    scale = amax / 127.0
+    scale = torch.where(scale == 0, torch.ones_like(scale), scale)
+    q = torch.round(blocks / scale[:, None, :, None]).clamp(-127, 127).reshape(nb * block, kb * block)[:n, :k]
+    return q.to(torch.int8).contiguous(), scale.contiguous()
+
+
 def int8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """Exact INT32 accumulators of int8 [M,K] x int8 [K,N]
     (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:38-153, ElementAccumulator int32).

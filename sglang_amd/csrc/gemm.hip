@@ -29,6 +29,11 @@ constexpr int KIND_FP8_BLOCK = 0;   // a4: sum_kb P_kb * sfa[m,kb] * sfb[kb,n/12
 constexpr int KIND_FP8_ROWCOL = 1;  // a6: sa[m] * (sb[n] * acc) + bias[n]
 constexpr int KIND_I8_ROWCOL = 2;   // a5: float(acc) * (sb[n] * sa[m]) + bias[n]
 constexpr int KIND_I8_RAW = 3;      // INT32 accumulators
+constexpr int KIND_I8_BLOCK = 4;    // block-scaled INT8: sum_kb float(P_kb) * sfa[m,kb] * sfb[kb,n/128]
+
+constexpr bool is_block(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_I8_BLOCK; }
+constexpr bool fp8_operands(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_FP8_ROWCOL; }
+constexpr bool float_acc(int kind) { return fp8_operands(kind) || kind == KIND_I8_BLOCK; }
 
 constexpr uint32_t OOB = 0x80000000u;  // offset beyond any buffer this library accepts
 
@@ -82,6 +87,28 @@ SGLQ_DEV uint32_t lds_addr(const void* p) {
 
 SGLQ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
+// One 128-byte K block of a block-scaled kind: the product of a weight and an activation
+// fragment from a zero accumulator.  FP8: one MFMA, fp32 result.  INT8: two MFMAs, exact
+// int32 result, returned as its bit pattern so that the conversion to float can wait until
+// the result is folded into the accumulator (block_value) instead of stalling on the MFMA.
+template <int KIND>
+SGLQ_DEV v4f block_mfma(const v8i& w, const v8i& a) {
+  if constexpr (KIND == KIND_I8_BLOCK) {
+    const v4i w0 = {w[0], w[1], w[2], w[3]}, w1 = {w[4], w[5], w[6], w[7]};
+    const v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
+    v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, a0, v4i{0, 0, 0, 0}, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, a1, t, 0, 0, 0);
+    return __builtin_bit_cast(v4f, t);
+  } else {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+  }
+}
+template <int KIND>
+SGLQ_DEV float block_value(float raw) {
+  if constexpr (KIND == KIND_I8_BLOCK) return (float)__builtin_bit_cast(int, raw);
+  else return raw;
+}
+
 template <int OUT_DT>
 SGLQ_DEV void store4(void* out, int64_t idx, float v0, float v1, float v2, float v3) {
   if constexpr (OUT_DT == SGLQ_BF16) {
@@ -133,7 +160,7 @@ SGLQ_DEV void finish4(const GemmArgs& p, int m, int n, const acc_t& a, float sam
   const int64_t idx = (int64_t)m * p.ldo + n;
   if constexpr (KIND == KIND_I8_RAW) {
     *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = a;
-  } else if constexpr (KIND == KIND_FP8_BLOCK) {
+  } else if constexpr (is_block(KIND)) {
     store4<OUT_DT>(p.out, idx, a[0], a[1], a[2], a[3]);
   } else {
     float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
@@ -279,9 +306,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
   constexpr int MI = TM / 16, NI = TN / 16;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
   constexpr int NLOAD = (BM + BN) / 8 / NW;  // 1 KiB copies per wave per stage
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool IS_FP8 = fp8_operands(KIND);
   static_assert((BM + BN) % (8 * NW) == 0 && TM % 16 == 0 && TN % 16 == 0, "tile shape");
-  static_assert(KIND != KIND_FP8_BLOCK || (128 % TN == 0), "a wave must stay inside one 128-wide scale block");
+  static_assert(!is_block(KIND) || (128 % TN == 0), "a wave must stay inside one 128-wide scale block");
 
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
 
@@ -341,7 +368,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
   const int a_base = (wm * TM) * 128;
   const int b_base = (BM + wn * TN) * 128;
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -355,7 +382,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
   float sfb_next = 0.f;
   int sfa_row[MI];
   int nb = 0;
-  if constexpr (KIND == KIND_FP8_BLOCK) {
+  if constexpr (is_block(KIND)) {
     const int nblocks = (p.N + 127) >> 7;
     nb = (n0 + wn * TN) >> 7;
     if (nb >= nblocks) nb = nblocks - 1;
@@ -377,7 +404,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     if (kb + 1 < nkb) issue_loads(cur ^ 1, (kb + 1) * 128);
 
     float sc[MI];
-    if constexpr (KIND == KIND_FP8_BLOCK) {
+    if constexpr (is_block(KIND)) {
 #pragma unroll
       for (int i = 0; i < MI; ++i) sc[i] = sfa_next[i] * sfb_next;
       if (kb + 1 < nkb) {
@@ -408,13 +435,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
     for (int i = 0; i < MI; ++i) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
-        if constexpr (KIND == KIND_FP8_BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i], z, 0, 0, 0, 0, 0, 0);
-          acc[i][j][0] = __builtin_fmaf(part[0], sc[i], acc[i][j][0]);
-          acc[i][j][1] = __builtin_fmaf(part[1], sc[i], acc[i][j][1]);
-          acc[i][j][2] = __builtin_fmaf(part[2], sc[i], acc[i][j][2]);
-          acc[i][j][3] = __builtin_fmaf(part[3], sc[i], acc[i][j][3]);
+        if constexpr (is_block(KIND)) {
+          const v4f part = block_mfma<KIND>(bf[j], af[i]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(block_value<KIND>(part[e]), sc[i], acc[i][j][e]);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -447,8 +471,8 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
   constexpr int NLOAD = (BM + BN) / 8 / NW;  // 8 one-KiB copies per wave per stage: 4 of A, 4 of B
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
-  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  constexpr bool IS_FP8 = fp8_operands(KIND);
+  constexpr bool BLOCK = is_block(KIND);
 
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
 
@@ -491,7 +515,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NI];
 
   // Block scales: row m of K block kb sits at sfa[m * stride_m + kb * stride_k].
@@ -560,18 +584,17 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
       for (int j = 0; j < NI; ++j) {
         const int idx = i * NI + j;
         if constexpr (BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, z, 0, 0, 0, 0, 0, 0);
+          v4f part = block_mfma<KIND>(bf[j], a_cur);
           __builtin_amdgcn_sched_barrier(0);
           if (j == 0 && i + 1 < MI) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
           if (pre && idx < NLOAD) issue_load(idx, cur ^ 1, kn * 128);
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
             const float s_use = (pi == i) ? sc : sc_prev;
-            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], s_use, acc[pi][pj][0]);
-            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], s_use, acc[pi][pj][1]);
-            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
-            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
+            acc[pi][pj][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), s_use, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), s_use, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), s_use, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), s_use, acc[pi][pj][3]);
           }
           if (pre && idx == NLOAD) sfb_next = p.sb[kn * p.sb_stride_k + nb * p.sb_stride_n];
           // fragment i - 1's scale is dead once its last result is folded in (idx = 4 i): refill it
@@ -596,10 +619,10 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
       a_cur = a_nxt;
     }
     if constexpr (BLOCK) {
-      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
-      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
-      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
-      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
       if constexpr (pre) {
         sfa_cur[MI - 1] = load_sfa(MI - 1, kn);
         sfb_cur = sfb_next;
@@ -711,8 +734,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
   constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
-  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  constexpr bool IS_FP8 = fp8_operands(KIND);
+  constexpr bool BLOCK = is_block(KIND);
   static_assert(NI == 4 && MI == 8, "the copy schedule below is written for 4 x 8 fragments");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
@@ -763,7 +786,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NI];
   v8i bf[NI];  // the step's weight fragments
   v8i a_cur;   // the activation fragment the next MFMAs use
@@ -849,8 +872,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         const int idx = i * NI + j;
         v4f part = {0.f, 0.f, 0.f, 0.f};
         if constexpr (BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, z, 0, 0, 0, 0, 0, 0);
+          part = block_mfma<KIND>(bf[j], a_cur);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -859,7 +881,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!IS_FP8) {
+        if constexpr (!IS_FP8 && !BLOCK) {
           const v4i b1 = {bf[j][4], bf[j][5], bf[j][6], bf[j][7]};
           const v4i a1 = {a_cur[4], a_cur[5], a_cur[6], a_cur[7]};
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
@@ -893,10 +915,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
             const float s_use = (pi == i) ? sc : sc_prev;
-            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], s_use, acc[pi][pj][0]);
-            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], s_use, acc[pi][pj][1]);
-            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], s_use, acc[pi][pj][2]);
-            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], s_use, acc[pi][pj][3]);
+            acc[pi][pj][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), s_use, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), s_use, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), s_use, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), s_use, acc[pi][pj][3]);
           }
           part_prev = part;
         }
@@ -905,10 +927,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       a_cur = a_nxt;
     }
     if constexpr (BLOCK) {
-      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
-      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
-      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
-      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
     }
   };
 
@@ -1013,8 +1035,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   constexpr int STAGE_BYTES = 512 * 128;  // stage pitch; only (BM + BN) rows are filled
   constexpr int NB = BN / 8;              // one-KiB weight copies per stage
   constexpr int NBW = (NB + NW - 1) / NW; // ... per wave (the last one only for waves < NB % 8)
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
-  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  constexpr bool IS_FP8 = fp8_operands(KIND);
+  constexpr bool BLOCK = is_block(KIND);
   static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
@@ -1068,7 +1090,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NI];
   v8i af[MI];  // the step's activation fragments
   v8i b_cur;   // the weight fragment the next MFMAs use
@@ -1166,8 +1188,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         const int idx = j * MI + i;
         v4f part = {0.f, 0.f, 0.f, 0.f};
         if constexpr (BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], z, 0, 0, 0, 0, 0, 0);
+          part = block_mfma<KIND>(b_cur, af[i]);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -1176,7 +1197,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!IS_FP8) {
+        if constexpr (!IS_FP8 && !BLOCK) {
           const v4i b1 = {b_cur[4], b_cur[5], b_cur[6], b_cur[7]};
           const v4i a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
@@ -1212,10 +1233,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         if constexpr (BLOCK) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
-            acc[pi][pj][0] = __builtin_fmaf(part_prev[0], sc_prev, acc[pi][pj][0]);
-            acc[pi][pj][1] = __builtin_fmaf(part_prev[1], sc_prev, acc[pi][pj][1]);
-            acc[pi][pj][2] = __builtin_fmaf(part_prev[2], sc_prev, acc[pi][pj][2]);
-            acc[pi][pj][3] = __builtin_fmaf(part_prev[3], sc_prev, acc[pi][pj][3]);
+            acc[pi][pj][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc_prev, acc[pi][pj][0]);
+            acc[pi][pj][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc_prev, acc[pi][pj][1]);
+            acc[pi][pj][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc_prev, acc[pi][pj][2]);
+            acc[pi][pj][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc_prev, acc[pi][pj][3]);
           }
           part_prev = part;
         }
@@ -1224,10 +1245,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       b_cur = b_nxt;
     }
     if constexpr (BLOCK) {
-      acc[MI - 1][NI - 1][0] = __builtin_fmaf(part_prev[0], sc, acc[MI - 1][NI - 1][0]);
-      acc[MI - 1][NI - 1][1] = __builtin_fmaf(part_prev[1], sc, acc[MI - 1][NI - 1][1]);
-      acc[MI - 1][NI - 1][2] = __builtin_fmaf(part_prev[2], sc, acc[MI - 1][NI - 1][2]);
-      acc[MI - 1][NI - 1][3] = __builtin_fmaf(part_prev[3], sc, acc[MI - 1][NI - 1][3]);
+      acc[MI - 1][NI - 1][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc, acc[MI - 1][NI - 1][0]);
+      acc[MI - 1][NI - 1][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc, acc[MI - 1][NI - 1][1]);
+      acc[MI - 1][NI - 1][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc, acc[MI - 1][NI - 1][2]);
+      acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
       jsw = jsw_nxt;
     }
   };
@@ -1337,13 +1358,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int BN = 128, NI = 2;
   constexpr int AR = MI * 16 < 32 ? 32 : MI * 16;  // activation rows staged (at least one copy per wave)
   constexpr int ACW = AR / 32;                     // activation copies per wave per stage
-  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
+  constexpr bool BLOCK = is_block(KIND);
   constexpr int CPW = 4 + ACW + (BLOCK ? 1 : 0);   // vector-memory loads per wave per stage
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 1024 : 0;
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
   constexpr int NSTAGE = 3;  // 64-77 KiB of LDS: two blocks (eight waves) per CU
   constexpr int MAX_STEPS = 1024;                  // K blocks per split that the weight-scale table holds
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool IS_FP8 = fp8_operands(KIND);
 
   __shared__ __attribute__((aligned(1024))) char smem[NSTAGE * STAGE_BYTES];
   __shared__ float sfb_tab[BLOCK ? MAX_STEPS : 1];
@@ -1405,7 +1426,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -1445,10 +1466,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
         if constexpr (BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], z, 0, 0, 0, 0, 0, 0);
+          v4f part = block_mfma<KIND>(wf[j], af[i]);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], sc[i], acc[i][j][e]);
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(block_value<KIND>(part[e]), sc[i], acc[i][j][e]);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -1480,8 +1500,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 template <int KIND, int MI, int NIB, int OUT_DT>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
   constexpr int BN = NIB * 16, AR = MI * 16;
-  constexpr bool BLOCK = KIND == KIND_FP8_BLOCK;
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
+  constexpr bool BLOCK = is_block(KIND);
+  constexpr bool IS_FP8 = fp8_operands(KIND);
   constexpr int WC = BN / 8, AC = AR / 8;          // one-KiB copies per stage: weights, activations
   constexpr int CPW = WC + AC + (BLOCK ? 2 : 0);   // vector-memory loads per stage
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 512 : 0;
@@ -1553,7 +1573,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   acc_t acc[MI][NIB];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -1588,10 +1608,9 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
 #pragma unroll
       for (int j = 0; j < NIB; ++j) {
         if constexpr (BLOCK) {
-          const v4f z = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], z, 0, 0, 0, 0, 0, 0);
+          v4f part = block_mfma<KIND>(wf[j], af[i]);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], sc[i], acc[i][j][e]);
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(block_value<KIND>(part[e]), sc[i], acc[i][j][e]);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -1633,8 +1652,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
 // run of four consecutive n.
 template <int KIND, int OUT_DT>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
-  constexpr bool IS_FP8 = (KIND == KIND_FP8_BLOCK || KIND == KIND_FP8_ROWCOL);
-  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  constexpr bool IS_FP8 = fp8_operands(KIND);
+  using acc_t = typename std::conditional<float_acc(KIND), v4f, v4i>::type;
   const int n4 = p.N >> 2;
   const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (id >= (int64_t)p.M * n4) return;
@@ -1921,12 +1940,11 @@ extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
 extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel; }
 
-extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
-                                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
-                                            int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
-                                            int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
-                                            int64_t workspace_bytes, void* stream) {
-  const char* name = "fp8_blockwise_scaled_mm";
+template <int KIND>
+static int blockwise_entry(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                           int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb, int64_t sfb_stride_k,
+                           int64_t sfb_stride_n, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                           void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
@@ -1948,9 +1966,29 @@ extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const vo
   p.sb_stride_n = sfb_stride_n;
   p.ws = workspace;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (out_dtype == SGLQ_BF16) launch_kind<KIND_FP8_BLOCK, SGLQ_BF16>(p, workspace_bytes, st);
-  else launch_kind<KIND_FP8_BLOCK, SGLQ_FP16>(p, workspace_bytes, st);
+  if (out_dtype == SGLQ_BF16) launch_kind<KIND, SGLQ_BF16>(p, workspace_bytes, st);
+  else launch_kind<KIND, SGLQ_FP16>(p, workspace_bytes, st);
   return finish(name);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                            int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                            int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                            int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
+                                         sfb_stride_k, sfb_stride_n, out, ldo, out_dtype, M, N, K, workspace,
+                                         workspace_bytes, stream);
+}
+
+extern "C" int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                             int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                             int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                             int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                             int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_I8_BLOCK>("w8a8_block_int8_matmul", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
+                                        sfb_stride_k, sfb_stride_n, out, ldo, out_dtype, M, N, K, workspace,
+                                        workspace_bytes, stream);
 }
 
 static int rowcol_entry(const char* name, bool fp8, const void* a, int64_t lda, const void* b, int64_t ldb,

@@ -1,0 +1,28 @@
+"""apply_w8a8_block_int8_linear with the reference's call sequence
+(python/sglang/srt/layers/quantization/int8_utils.py:11-33)."""
+
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .int8_kernel import per_token_group_quant_int8, w8a8_block_int8_matmul
+
+
+def apply_w8a8_block_int8_linear(
+    input: torch.Tensor,
+    weight: torch.Tensor,
+    block_size: List[int],
+    weight_scale: torch.Tensor,
+    input_scale: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    assert input_scale is None
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    q_input, x_scale = per_token_group_quant_int8(input_2d, block_size[1])
+    output = w8a8_block_int8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
+    if bias is not None:
+        output = output + bias
+    return output.to(dtype=input.dtype).view(*output_shape)

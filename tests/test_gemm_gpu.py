@@ -119,6 +119,61 @@ def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
     torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
 
 
+def make_block_int8_case(m, n, k, seed):
+    x = O.gen_activation(m, k, seed=seed, outliers=True)
+    wq, ws = O.block_quant_weight_int8(O.gen_weight(n, k, seed=seed))
+    xq, xs = O.per_token_group_quant_8bit(x, 128, 1e-10, -128.0, 127.0, torch.int8)
+    return xq, xs, wq, ws
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (3, 256, 512), (5, 2112, 1536), (17, 7168, 2048), (127, 512, 7168), (128, 4096, 512),
+                                 (256, 2048, 7168), (512, 1536, 1024), (1024, 640, 2048)])
+def test_w8a8_block_int8_matmul(gpu, tile, mnk, out_dtype):
+    """Block-scaled INT8 (w8a8_block_int8_matmul, int8_kernel.py:339-425) on every GEMM kernel:
+    row-major activation scales, the weight and its scales as stored."""
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    say("block int8", mnk, out_dtype, "tile", tile)
+    m, n, k = mnk
+    xq, xs, wq, ws = make_block_int8_case(m, n, k, seed=m + n + k)
+    rows = sample_rows(m)
+    ref = O.w8a8_block_int8_matmul(xq[rows], wq, xs[rows], ws, torch.float32, acc_dtype=torch.float64)
+    out = w8a8_block_int8_matmul(xq.to(gpu), wq.to(gpu), xs.to(gpu), ws.to(gpu), [128, 128], out_dtype)
+    assert out.dtype == out_dtype and tuple(out.shape) == (m, n)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_w8a8_block_int8_unit_scales_exact_and_linear(gpu):
+    """Unit scales and small integers: exact whatever the summation order; then the glue
+    (per-token-group INT8 quant, GEMM, bias) against the oracle's same sequence."""
+    from sglang_amd.quantization.int8_kernel import per_token_group_quant_int8, w8a8_block_int8_matmul
+    from sglang_amd.quantization.int8_utils import apply_w8a8_block_int8_linear
+
+    say("block int8 exact integers + linear")
+    g = torch.Generator().manual_seed(6)
+    m, n, k = 300, 384, 1024
+    a = torch.randint(-8, 9, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-8, 9, (n, k), generator=g, dtype=torch.int8)
+    ref = a.double() @ w.double().t()
+    out = w8a8_block_int8_matmul(a.to(gpu), w.to(gpu), torch.ones((m, 8), device=gpu), torch.ones((3, 8), device=gpu),
+                                 [128, 128], torch.bfloat16).cpu()
+    assert torch.equal(out.double(), ref.to(torch.bfloat16).double())
+    x = O.gen_activation(40, 2048, seed=77, outliers=True)
+    wq, ws = O.block_quant_weight_int8(O.gen_weight(1536, 2048, seed=78))
+    bias = (torch.randn(1536, generator=g) * 0.1).to(torch.bfloat16)
+    xq_ref, xs_ref = O.per_token_group_quant_8bit(x, 128, 1e-10, -128.0, 127.0, torch.int8)
+    xq, xs = per_token_group_quant_int8(x.to(gpu), 128)
+    assert torch.equal(xq.cpu(), xq_ref) and torch.equal(xs.cpu(), xs_ref)
+    mm = O.w8a8_block_int8_matmul(xq_ref, wq, xs_ref, ws, torch.float32)
+    ref = mm + bias.float()
+    out = apply_w8a8_block_int8_linear(x.to(gpu).view(2, 20, 2048), wq.to(gpu), [128, 128], ws.to(gpu), bias=bias.to(gpu))
+    assert tuple(out.shape) == (2, 20, 1536) and out.dtype == torch.bfloat16
+    tol = 1e-2 + 1e-2 * ref.abs() + mm.abs() * 2.0**-8  # the GEMM output is rounded to bf16 before the bias is added
+    err = (out.cpu().view(40, 1536).float() - ref).abs()
+    assert bool((err <= tol).all()), f"max excess {(err - tol).max().item()}"
+
+
 def test_fp8_blockwise_unit_scales_is_plain_matmul(gpu):
     """All scales 1 and small integer-valued operands: every partial sum is an
     integer below 2^24, so the result is exact whatever the summation order."""

@@ -285,6 +285,44 @@ def test_blockwise_mm_vs_c_double_brute_force(c_oracle):
     torch.testing.assert_close(out.double(), deq_a @ deq_w.t(), rtol=1e-6, atol=1e-9)
 
 
+def test_block_int8_mm_pins(c_oracle):
+    """w8a8_block_int8_matmul: unit scales reduce to the exact integer product, one-hot rows select
+    scaled weight rows, a double-precision C brute force on N % 128 != 0 and K % 128 != 0, and the
+    reference test's block-wise dequantization (test/srt/quant/test_block_int8.py:40-92)."""
+    g = torch.Generator().manual_seed(21)
+    m, n, k = 4, 136, 320
+    a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int8)
+    a[0, :128] = -128
+    w[5, :128] = -128  # the extreme block sum 128 * 128^2 = 2^21 is exact
+    ones_a, ones_w = torch.ones(m, 3), torch.ones(2, 3)
+    out = O.w8a8_block_int8_matmul(a, w, ones_a, ones_w, torch.float32, acc_dtype=torch.float64)
+    assert torch.equal(out.double(), a.double() @ w.double().t())
+    sa = torch.rand((m, 3), generator=g) * 1e-2
+    sw = torch.rand((2, 3), generator=g) * 1e-3
+    onehot = torch.zeros((3, k), dtype=torch.int8)
+    onehot[0, 7], onehot[1, 200], onehot[2, 319] = 1, -2, 3
+    out = O.w8a8_block_int8_matmul(onehot, w, sa[:3], sw, torch.float32)
+    for r, (col, v) in enumerate(((7, 1), (200, -2), (319, 3))):
+        want = (w[:, col].float() * v) * sa[r, col // 128] * sw.repeat_interleave(128, dim=0)[:n, col // 128]
+        torch.testing.assert_close(out[r], want, rtol=1e-6, atol=0)
+    out = O.w8a8_block_int8_matmul(a, w, sa, sw, torch.float32, acc_dtype=torch.float64)
+    ref = torch.empty((m, n), dtype=torch.float64)
+    c_oracle.oracle_int8_blockwise_mm(
+        ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(w.data_ptr()), ctypes.c_void_p(sa.contiguous().data_ptr()),
+        ctypes.c_void_p(sw.contiguous().data_ptr()), ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+        ctypes.c_void_p(ref.data_ptr()))
+    torch.testing.assert_close(out.double(), ref, rtol=1e-6, atol=1e-9)  # the oracle rounds its result to fp32
+    deq_a = a.double() * sa.double().repeat_interleave(128, dim=1)[:, :k]
+    deq_w = w.double() * sw.double().repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)[:, :k]
+    torch.testing.assert_close(out.double(), deq_a @ deq_w.t(), rtol=1e-6, atol=1e-9)
+    # harness-side weight quantization round trip
+    wf = torch.randn((136, 300), generator=g)
+    q, s = O.block_quant_weight_int8(wf)
+    deq = q.float() * s.repeat_interleave(128, dim=0)[:136].repeat_interleave(128, dim=1)[:, :300]
+    assert float((deq - wf).abs().max()) <= float(s.max()) * 0.5 + 1e-7
+
+
 def test_int8_accumulators_exact(c_oracle):
     g = torch.Generator().manual_seed(8)
     a = torch.randint(-128, 128, (5, 4096), generator=g, dtype=torch.int8)
