@@ -12,7 +12,7 @@ quantization kernel's HBM figure, and a CPU baseline (the torch restatement of
 the same path, timed on a bounded row sample on the host cores).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --sweep gpurun_out/sweep.jsonl     # every configuration, one line per shape
+    python bench.py --sweep sweep.jsonl                # every configuration, one line per shape
 """
 import argparse
 import json
