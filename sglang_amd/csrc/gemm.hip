@@ -797,7 +797,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // two weight scales of the tile's two 128-column blocks (lanes 0 and 1), waves 5..7 nothing
   // (all lanes out of range; kept so that the instruction stream has no branch).
   // sc_voff / sc_voff2: per-lane source offsets for the tile of block u + 1 / u + 2.
-  const int nkb = p.K >> 7;
+  const int nkb_all = p.K >> 7;
+  const int nkb = nkb_all / p.splits;  // K blocks of one work unit (the host makes it divide)
   float sfa_cur[MI];
   float sfb_cur = 0.f;
   __amdgpu_buffer_rsrc_t rsc = ra;
@@ -808,8 +809,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   const int sfb_rd = 2 * STAGE_BYTES + 1024 + (wn >> 1) * 4;
   if constexpr (BLOCK) {
     const int nblocks = (p.N + 127) >> 7;
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
-    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb_all - 1) * p.sa_stride_k + 1;
+    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb_all - 1) * p.sb_stride_k + 1;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
   }
@@ -934,23 +935,33 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     }
   };
 
-  // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
-  const int total = p.tiles_m * p.tiles_n;
+  // ---- persistent walk over the work units blockIdx, blockIdx + gridDim, ...  A unit is an
+  // output tile, or with split-K (p.splits > 1) one of a tile's p.splits contiguous K ranges,
+  // whose raw partial sums go to the workspace for splitk_reduce_kernel.
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int total = tiles * p.splits;
   const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-  int tile = blockIdx.x;
-  int tm, tn;
-  tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
-  int m0 = tm * BM, n0 = tn * BN;
-  int par = 0;  // stage that holds K block 0 of the current tile
+  auto unit_origin = [&](int u, int& um0, int& un0, int& ukb0) {
+    const int split = u / tiles;
+    int tm, tn;
+    tile_of_block(u - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
+    um0 = tm * BM;
+    un0 = tn * BN;
+    ukb0 = split * nkb;
+  };
+  int unit = blockIdx.x;
+  int m0, n0, kb0;
+  unit_origin(unit, m0, n0, kb0);
+  int par = 0;  // stage that holds the unit's first K block
 
   off_a = off_a2 = a_offset(m0);
   off_b = off_b2 = b_offset(n0);
   if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
+  for (int j = 0; j < 4; ++j) copy_a(j, 0, kb0 * 128, off_a);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_b(j, 0, 0, off_b);
-  if constexpr (BLOCK) copy_scales(0, 0, sc_voff);
+  for (int j = 0; j < 4; ++j) copy_b(j, 0, kb0 * 128, off_b);
+  if constexpr (BLOCK) copy_scales(0, kb0, sc_voff);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -968,27 +979,30 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
-    // The block's next tile; past its last tile the prefetches are pointed at rows beyond M
+    // The block's next unit; past its last one the prefetches are pointed at rows beyond M
     // and N, which the buffer bounds turn into zero fill without memory traffic.
-    const int next_tile = tile + (int)gridDim.x;
-    const bool has_next = next_tile < total;
-    tile_of_block(has_next ? next_tile : 0, p.tiles_m, p.tiles_n, tm, tn);
-    const int nm0 = has_next ? tm * BM : p.tiles_m * BM;
-    const int nn0 = has_next ? tn * BN : p.tiles_n * BN;
+    const int next_unit = unit + (int)gridDim.x;
+    const bool has_next = next_unit < total;
+    int nm0, nn0, nkb0;
+    unit_origin(has_next ? next_unit : 0, nm0, nn0, nkb0);
+    if (!has_next) {
+      nm0 = p.tiles_m * BM;
+      nn0 = p.tiles_n * BN;
+    }
 
-    // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
+    // (a unit has at least three K blocks, so its first, last-but-one and last step are distinct)
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
     uint32_t sc_voff_next = OOB;
     if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
-    k_step(par, 1, 2, std::true_type{}, std::false_type{});
+    k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{});
     for (int kb = 1; kb + 1 < nkb; ++kb) {
-      const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
+      const bool pen = kb + 2 == nkb;  // the block two ahead is the next unit's first
       off_a2 = pen ? off_a_next : off_a2;
       off_b2 = pen ? off_b_next : off_b2;
       sc_voff2 = pen ? sc_voff_next : sc_voff2;
-      k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
+      k_step((kb + par) & 1, kb0 + kb + 1, pen ? nkb0 : kb0 + kb + 2, std::false_type{}, std::false_type{});
     }
-    // last K block: its copies (the next tile's second block) wait for the next tile's first step
+    // last K block: its copies (the next unit's second block) wait for the next unit's first step
     const int last_stage = (nkb - 1 + par) & 1;
     k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
     off_a = off_a2;
@@ -997,7 +1011,9 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
-    if constexpr (KIND == KIND_I8_RAW) {
+    if (p.splits > 1) {
+      store_partials<MI, NI>(p, acc, unit / tiles, m0 + wm * TM, n0 + wn * TN, r16, g);
+    } else if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
@@ -1008,9 +1024,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     }
     if (!has_next) break;
-    tile = next_tile;
+    unit = next_unit;
     m0 = nm0;
     n0 = nn0;
+    kb0 = nkb0;
     par = last_stage ^ 1;
   }
 }
@@ -1727,18 +1744,40 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 static int g_force_tile = 0;
 
 template <int KIND, int OUT_DT>
-static void launch_big(GemmArgs& p, hipStream_t st) {
+static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 255) / 256;
   p.splits = 1;
   // persistent: one block per CU walks the tiles blockIdx, blockIdx + gridDim, ...
   const int tiles = p.tiles_m * p.tiles_n;
-  const int blocks = tiles < num_cus() ? tiles : num_cus();
   // the pipelined kernel needs three K blocks; 256 forces the plain one (test hook)
   if (g_force_tile != 256 && p.K >= 384) {
-    g_last_kernel = "gemm_pipe_kernel";
+    // Too few tiles for the chip: split K into equal contiguous ranges of at least four K
+    // blocks, as many as fill the CUs and the workspace holds; the partial sums cost
+    // 8 M N splits bytes of traffic, which must stay well under the operands'.
+    const int nkb = p.K >> 7;
+    int splits = 1;
+    if (2 * tiles <= num_cus() || g_force_splits > 0) {
+      int want = g_force_splits > 0 ? g_force_splits : num_cus() / tiles;
+      const int64_t per_split = (int64_t)p.M * p.N * 4;
+      if (!p.ws || ws_bytes < 2 * per_split) want = 1;
+      else if (want * per_split > ws_bytes) want = (int)(ws_bytes / per_split);
+      const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
+      if (g_force_splits == 0 && want > by_traffic) want = (int)(by_traffic > 0 ? by_traffic : 1);
+      for (int s = want; s >= 2; --s)
+        if (nkb % s == 0 && nkb / s >= (g_force_splits > 0 ? 3 : 4)) {
+          splits = s;
+          break;
+        }
+    }
+    p.splits = splits;
+    const int units = tiles * splits;
+    const int blocks = units < num_cus() ? units : num_cus();
+    g_last_kernel = splits > 1 ? "gemm_pipe_kernel+splitk_reduce_kernel" : "gemm_pipe_kernel";
     gemm_pipe_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+    if (splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
   } else {
+    const int blocks = tiles < num_cus() ? tiles : num_cus();
     g_last_kernel = "gemm_big_kernel";
     gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
   }
@@ -1854,14 +1893,18 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // the 256 CUs (e.g. 144 tiles at M = 4096, N = 2112; 192 at M = 512, N = 24576); with
   // fewer tiles the 128 x 128 kernel with split-K keeps more CUs busy.
   const int big_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
+  // ... unless the problem is large and deep enough for the pipelined kernel with K split over
+  // (tile, K range) units: 512 x 7168 x 16384 90.6 -> 75.6 us, 1024 x 7168 x 16384 164.5 -> 122.6 us,
+  // but 1024 x 4096 x 7168 49 -> 56 us (measured).
+  const bool deep = p.M > 256 && (p.K >> 7) >= 64 && 2.0 * p.M * p.N * p.K >= 1e11;
   const bool forced_256 = g_force_tile == 256 || g_force_tile == 258 || g_force_tile == 192 || g_force_tile == 224 || g_force_tile == 257;
-  if ((p.K & 127) == 0 && (forced_256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && big_tiles >= 140))) {
-    int width = g_force_tile == 0 ? pick_tile_width(p) : g_force_tile;
+  if ((p.K & 127) == 0 && (forced_256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && (big_tiles >= 140 || deep)))) {
+    int width = g_force_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p) : 256) : g_force_tile;
     if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
     else if (width == 257) launch_wide<KIND, OUT_DT, 8>(p, st);
-    else launch_big<KIND, OUT_DT>(p, st);
+    else launch_big<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
   if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, ws_bytes, st);

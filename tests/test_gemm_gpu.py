@@ -361,6 +361,47 @@ def test_mid_m_split_k(gpu, splits, mnk):
     assert torch.equal(int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()[rows], O.int8_mm_i32(a8[rows], w8.t()))
 
 
+@pytest.mark.parametrize("mnk", [(100, 384, 1536), (512, 640, 7168), (300, 2112, 3072), (1000, 256, 1536)])
+def test_pipelined_kernel_split_k(gpu, splits, mnk):
+    """The pipelined 256 x 256 kernel takes (tile, K range) work units when the tiles do not fill
+    the chip (forced here): every kind, block-scaled INT8 included, and any split factor that
+    leaves three K blocks per unit."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32
+
+    say("pipelined kernel split-K", mnk, "splits", splits)
+    lib = _lib.load()
+    lib.sglq_debug_force_tile(258)
+    try:
+        m, n, k = mnk
+        _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+        rows = sample_rows(m)
+        ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+        xs_cm = xs.t().contiguous().to(gpu).t()
+        out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.bfloat16)
+        kernel = lib.sglq_debug_last_gemm_kernel().decode()
+        assert kernel.startswith("gemm_pipe_kernel")
+        if splits in (2, 3, 4) and (k // 128) % splits == 0 and (k // 128) // splits >= 3:
+            assert kernel.endswith("splitk_reduce_kernel")
+        torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+        g = torch.Generator().manual_seed(m)
+        sa = torch.rand((m, 1), generator=g) * 0.05 + 0.01
+        sb = torch.rand((n, 1), generator=g) * 0.001 + 0.0005
+        bias = (torch.randn(n, generator=g) * 0.1).to(torch.float16)
+        ref = O.fp8_scaled_mm(xq[rows], wq.t(), sa[rows], sb, torch.float32, bias, acc_dtype=torch.float64)
+        out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.float16, bias.to(gpu))
+        torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+        a8, w8 = rand_i8((m, k), 5), rand_i8((n, k), 6)
+        assert torch.equal(int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()[rows], O.int8_mm_i32(a8[rows], w8.t()))
+        x8, s8, wq8, ws8 = make_block_int8_case(m, n, k, seed=n + k)
+        ref = O.w8a8_block_int8_matmul(x8[rows], wq8, s8[rows], ws8, torch.float32, acc_dtype=torch.float64)
+        out = w8a8_block_int8_matmul(x8.to(gpu), wq8.to(gpu), s8.to(gpu), ws8.to(gpu), [128, 128], torch.bfloat16)
+        torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+    finally:
+        lib.sglq_debug_force_tile(0)
+
+
 def test_gemm_empty_m(gpu):
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, int8_scaled_mm
 
