@@ -1,0 +1,77 @@
+"""Seeded random shapes through every GEMM kernel selection: ragged M, N that is a multiple
+of 8 only, K any multiple of 128 (16 for the kernels that take it), against the CPU oracle.
+INT32 accumulators bit-exact; 16-bit outputs within rtol 1e-2 / atol 1e-2."""
+import random
+
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+RTOL, ATOL = 1e-2, 1e-2
+
+# (force_tile code, M range, needs K % 128 == 0)
+SELECTIONS = [
+    (0, (1, 700), False), (128, (1, 300), False), (256, (65, 600), True), (258, (65, 600), True),
+    (192, (65, 600), True), (224, (65, 600), True), (257, (65, 600), True), (64, (1, 64), True),
+    (16, (1, 32), True), (32, (1, 32), True),
+]
+
+
+def shapes_for(code, m_range, k128, count, seed):
+    rng = random.Random(seed * 1000 + code)
+    out = []
+    for _ in range(count):
+        m = rng.randint(*m_range)
+        n = 8 * rng.randint(1, 150)
+        k = 128 * rng.randint(1, 18) if k128 else 16 * rng.randint(1, 140)
+        if code in (16, 32):
+            k = 128 * rng.randint(4, 40)
+        out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("code,m_range,k128", SELECTIONS, ids=[f"tile{c[0]}" for c in SELECTIONS])
+def test_random_shapes_all_kinds(gpu, code, m_range, k128):
+    from sglang_amd import _lib
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32, int8_scaled_mm
+
+    lib = _lib.load()
+    lib.sglq_debug_force_tile(code)
+    try:
+        for (m, n, k) in shapes_for(code, m_range, k128, 12, seed=7):
+            print("random shape", code, (m, n, k), flush=True)
+            g = torch.Generator().manual_seed(m * 31 + n * 7 + k)
+            kb, nb = (k + 127) // 128, (n + 127) // 128
+            a8 = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+            w8 = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int8)
+            af = (torch.randn((m, k), generator=g) * 2).to(FP8)
+            wf = (torch.randn((n, k), generator=g) * 0.5).to(FP8)
+            sa = torch.rand((m, 1), generator=g) * 0.05 + 0.01
+            sb = torch.rand((n, 1), generator=g) * 0.01 + 0.001
+            bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16)
+            # INT32 accumulators: exact
+            acc = int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()
+            assert torch.equal(acc, O.int8_mm_i32(a8, w8.t())), (code, m, n, k)
+            # per-row / per-column kinds
+            ref = O.int8_scaled_mm(a8, w8.t(), sa * 0.01, sb, torch.bfloat16, bias)
+            out = int8_scaled_mm(a8.to(gpu), w8.to(gpu).t(), (sa * 0.01).to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+            torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
+            ref = O.fp8_scaled_mm(af, wf.t(), sa, sb, torch.float32, None, acc_dtype=torch.float64)
+            out = fp8_scaled_mm(af.to(gpu), wf.to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.float16, None)
+            torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+            # block-scaled kinds
+            sfa = torch.rand((m, kb), generator=g) * 0.05 + 0.01
+            sfb = torch.rand((nb, kb), generator=g) * 0.01 + 0.001
+            ref = O.fp8_blockwise_scaled_mm(af, wf.t(), sfa, sfb.t(), torch.float32, acc_dtype=torch.float64)
+            sfa_cm = sfa.t().contiguous().to(gpu).t()
+            out = fp8_blockwise_scaled_mm(af.to(gpu), wf.to(gpu).t(), sfa_cm, sfb.to(gpu).t(), torch.bfloat16)
+            torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+            ref = O.w8a8_block_int8_matmul(a8, w8, sfa * 0.01, sfb, torch.float32, acc_dtype=torch.float64)
+            out = w8a8_block_int8_matmul(a8.to(gpu), w8.to(gpu), (sfa * 0.01).to(gpu), sfb.to(gpu), [128, 128], torch.float16)
+            torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    finally:
+        lib.sglq_debug_force_tile(0)
