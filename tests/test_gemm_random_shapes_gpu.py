@@ -75,3 +75,35 @@ def test_random_shapes_all_kinds(gpu, code, m_range, k128):
             torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
     finally:
         lib.sglq_debug_force_tile(0)
+
+
+@pytest.mark.parametrize("code,m", [(0, 300), (128, 300), (256, 300), (258, 300), (224, 300), (192, 300), (64, 48), (16, 9), (32, 20)],
+                         ids=lambda v: str(v))
+def test_strided_operands(gpu, code, m):
+    """mat_a a column slice of a wider tensor (row stride 2 K + 64), mat_b a slice of a wider
+    [N, 3 K] weight (column stride 3 K): the kernels take the strides, nothing is copied."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, int8_mm_i32
+
+    lib = _lib.load()
+    lib.sglq_debug_force_tile(code)
+    try:
+        n, k = 520, 2048
+        g = torch.Generator().manual_seed(code * 100 + m)
+        a_big = torch.randint(-128, 128, (m, 2 * k + 64), generator=g, dtype=torch.int8)
+        w_big = torch.randint(-128, 128, (n, 3 * k), generator=g, dtype=torch.int8)
+        a, w = a_big[:, 64 : 64 + k], w_big[:, k : 2 * k]
+        ag, wg = a_big.to(gpu)[:, 64 : 64 + k], w_big.to(gpu)[:, k : 2 * k]
+        assert ag.stride(0) == 2 * k + 64 and wg.t().stride(1) == 3 * k
+        assert torch.equal(int8_mm_i32(ag, wg.t()).cpu(), O.int8_mm_i32(a.contiguous(), w.contiguous().t()))
+        af_big = (torch.randn((m, 2 * k + 64), generator=g) * 2).to(FP8)
+        wf_big = (torch.randn((n, 3 * k), generator=g) * 0.5).to(FP8)
+        sfa = torch.rand((m, k // 128), generator=g) * 0.05 + 0.01
+        sfb = torch.rand(((n + 127) // 128, k // 128), generator=g) * 0.01 + 0.001
+        ref = O.fp8_blockwise_scaled_mm(af_big[:, 64 : 64 + k].contiguous(), wf_big[:, k : 2 * k].contiguous().t(), sfa, sfb.t(),
+                                        torch.float32, acc_dtype=torch.float64)
+        out = fp8_blockwise_scaled_mm(af_big.to(gpu)[:, 64 : 64 + k], wf_big.to(gpu)[:, k : 2 * k].t(),
+                                      sfa.t().contiguous().to(gpu).t(), sfb.to(gpu).t(), torch.bfloat16)
+        torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    finally:
+        lib.sglq_debug_force_tile(0)
