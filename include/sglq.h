@@ -104,6 +104,16 @@ int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int6
                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                  int64_t workspace_bytes, void* stream);
 
+/* sglq_fp8_blockwise_scaled_mm fused with the bias add that its caller performs on the
+ * result (python/sglang/srt/layers/quantization/fp8_utils.py:207-211: the GEMM, then
+ * `output += bias` on the rounded output): out = round(round(gemm) + bias), bias [N] in
+ * out_dtype or NULL.  Saves one read-modify-write pass over [M, N]. */
+int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                      int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                      int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out,
+                                      int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                      int64_t workspace_bytes, void* stream);
+
 /* Replaces w8a8_block_int8_matmul, a Triton kernel in the reference
  * (python/sglang/srt/layers/quantization/int8_kernel.py:212-425; there is no
  * sgl_kernel C++ op): out[m,n] = sum_kb float(sum_{k in block kb} a[m,k] b[k,n])

@@ -122,6 +122,13 @@ SGLQ_DEV void store4(void* out, int64_t idx, float v0, float v1, float v2, float
   }
 }
 
+// fp32 -> output type -> fp32
+template <int OUT_DT>
+SGLQ_DEV float round_out(float v) {
+  if constexpr (OUT_DT == SGLQ_BF16) return (float)(__bf16)v;
+  else return (float)(_Float16)v;
+}
+
 template <int OUT_DT>
 SGLQ_DEV void load_bias4(const void* bias, int n, float (&b)[4]) {
   if constexpr (OUT_DT == SGLQ_BF16) {
@@ -155,13 +162,25 @@ SGLQ_DEV void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn)
 }
 
 // Scale, add bias and store four consecutive outputs C[m][n..n+3] from their accumulators.
-template <int KIND, int OUT_DT, typename acc_t>
+// BLOCK_BIAS (block-scaled kinds only): 1 / 0 = the caller knows at compile time that there
+// is / is not a bias, -1 = look at p.bias.
+template <int KIND, int OUT_DT, int BLOCK_BIAS = -1, typename acc_t>
 SGLQ_DEV void finish4(const GemmArgs& p, int m, int n, const acc_t& a, float sam) {
   const int64_t idx = (int64_t)m * p.ldo + n;
   if constexpr (KIND == KIND_I8_RAW) {
     *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(p.out) + idx) = a;
   } else if constexpr (is_block(KIND)) {
-    store4<OUT_DT>(p.out, idx, a[0], a[1], a[2], a[3]);
+    if (BLOCK_BIAS == 1 || (BLOCK_BIAS == -1 && p.bias)) {
+      // the caller's `output += bias` on the rounded GEMM result (fp8_utils.py:210-211), fused:
+      // round to the output type, add the bias in fp32, round again
+      float bv[4], o[4];
+      load_bias4<OUT_DT>(p.bias, n, bv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = round_out<OUT_DT>(a[e]) + bv[e];
+      store4<OUT_DT>(p.out, idx, o[0], o[1], o[2], o[3]);
+    } else {
+      store4<OUT_DT>(p.out, idx, a[0], a[1], a[2], a[3]);
+    }
   } else {
     float o[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
     const v4f sbn = *reinterpret_cast<const v4f*>(p.sb + n);
@@ -179,6 +198,7 @@ SGLQ_DEV void finish4(const GemmArgs& p, int m, int n, const acc_t& a, float sam
 // workspace, laid out [split][M][N] (fp32 or int32); splitk_reduce_kernel finishes them.
 template <int MI, int NI, typename acc_t>
 SGLQ_DEV void store_partials(const GemmArgs& p, acc_t (&acc)[MI][NI], int split, int m_base, int n_base, int r16, int g) {
+  asm volatile("" : "+v"(r16), "+v"(g));  // keep the address arithmetic here (see epilogue_via_lds)
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + i * 16 + r16;
@@ -193,10 +213,31 @@ SGLQ_DEV void store_partials(const GemmArgs& p, acc_t (&acc)[MI][NI], int split,
   }
 }
 
+// The same for the 256-row kernels, as buffer stores that need neither branches nor 64-bit
+// addresses: a row beyond M lies beyond the split's extent and is dropped by the bounds
+// check, a column beyond N gets an offset that is.  The host keeps (M + 256) N 4 below 2 GiB.
+template <int MI, int NI, typename acc_t>
+SGLQ_DEV void store_partials_bounded(const GemmArgs& p, acc_t (&acc)[MI][NI], int split, int m_base, int n_base, int r16, int g) {
+  asm volatile("" : "+v"(r16), "+v"(g));  // keep the address arithmetic here (see epilogue_via_lds)
+  const uint32_t row_bytes = (uint32_t)p.N * 4u, split_bytes = (uint32_t)p.M * row_bytes;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(reinterpret_cast<char*>(p.ws) + (int64_t)split * split_bytes, split_bytes);
+  const int n_lane = n_base + g * 4;
+  const uint32_t off = (uint32_t)(m_base + r16) * row_bytes + (uint32_t)n_lane * 4u;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const uint32_t voff = (n_lane + j * 16 < p.N) ? off + (uint32_t)(i * 16) * row_bytes + (uint32_t)(j * 64) : OOB;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[i][j]), rw, voff, 0, 0);
+    }
+  }
+}
+
 // Scale, add bias and store a wave's accumulators.  acc[i][j][e] belongs to
 // C[m_base + 16 i + r16][n_base + 16 j + 4 g + e].
-template <int KIND, int OUT_DT, int MI, int NI, typename acc_t>
+template <int KIND, int OUT_DT, int MI, int NI, int BLOCK_BIAS = -1, typename acc_t>
 SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int n_base, int r16, int g) {
+  asm volatile("" : "+v"(r16), "+v"(g));  // keep the address arithmetic here (see epilogue_via_lds)
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + i * 16 + r16;
@@ -207,7 +248,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + j * 16 + g * 4;
       if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
-      finish4<KIND, OUT_DT>(p, m, n, acc[i][j], sam);
+      finish4<KIND, OUT_DT, BLOCK_BIAS>(p, m, n, acc[i][j], sam);
     }
   }
 }
@@ -220,10 +261,16 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 // chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
-template <int KIND, int OUT_DT, int MI, int NI, int BN, typename acc_t>
-SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, int m0, int n0, int wm, int wn,
-                               int r16, int g, int lane, int wave) {
+template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, typename acc_t>
+SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, float* bias_lds, int m0, int n0,
+                               int wm, int wn, int r16, int g, int lane, int wave) {
   constexpr int TN = NI * 16;
+  // The addresses below depend on the lane only, not on the tile: left alone, the compiler
+  // computes them once before the caller's tile loop and keeps dozens of registers alive
+  // through every K step (and spills them inside the pipelined steps, where a scratch access
+  // waits for all copies in flight).  Hide the lane-derived values' origin so that the
+  // arithmetic stays here.
+  asm volatile("" : "+v"(r16), "+v"(g), "+v"(lane));
   float bv[NI][4], sbv[NI][4];
   if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
 #pragma unroll
@@ -245,6 +292,22 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   const int c = lane & 31;
   const int n = n0 + c * 8;
   char* out = reinterpret_cast<char*>(p.out);
+  // Block-scaled kinds: the optional bias is the caller's `output += bias` on the rounded
+  // result (fp8_utils.py:210-211), added to the image's values on their way out.  The tile's
+  // 256 bias values wait in LDS behind the image (`bias_lds`, 1 KiB, written here and made
+  // visible by the first barrier below), so that no register holds them across the epilogue.
+  // (BIAS: a kernel variant of its own, launched only with a bias, so that the plain variant's
+  // register allocation is not disturbed)
+  constexpr bool add_bias = BIAS && is_block(KIND);
+  if (add_bias && threadIdx.x < 256) {
+    const int nb = n0 + (int)threadIdx.x;
+    float b = 0.f;
+    if (nb < p.N) {
+      if constexpr (OUT_DT == SGLQ_BF16) b = u2f((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[nb] << 16);
+      else b = (float)reinterpret_cast<const _Float16*>(p.bias)[nb];
+    }
+    bias_lds[threadIdx.x] = b;
+  }
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     if (((wm * MI * 16) >> 7) == half) {  // wave-uniform: a wave's rows lie in one half
@@ -284,7 +347,28 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
     for (int it = 0; it < 8; ++it) {
       const int ml = wave * 16 + it * 2 + (lane >> 5);
       const int m = m0 + half * 128 + ml;
-      const v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
+      v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
+      if constexpr (add_bias) {
+        const v4f blo = *reinterpret_cast<const v4f*>(bias_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(bias_lds + c * 8 + 4);
+        const float bias8[8] = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w = (uint32_t)v[q];
+          float lo, hi;
+          if constexpr (OUT_DT == SGLQ_BF16) {
+            lo = u2f(w << 16) + bias8[2 * q];
+            hi = u2f(w & 0xffff0000u) + bias8[2 * q + 1];
+            typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+            v[q] = __builtin_bit_cast(int, bf2{(__bf16)lo, (__bf16)hi});
+          } else {
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+            const h2 h = __builtin_bit_cast(h2, w);
+            lo = (float)h[0] + bias8[2 * q];
+            hi = (float)h[1] + bias8[2 * q + 1];
+            v[q] = __builtin_bit_cast(int, h2{(_Float16)lo, (_Float16)hi});
+          }
+        }
+      }
       if (m < p.M && c * 8 < BN) {
         char* row = out + ((int64_t)m * p.ldo + n) * 2;
         if (n + 8 <= p.N) {
@@ -465,7 +549,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
 // byte is read once per wave and the 128 accumulator registers leave room for
 // two waves per SIMD.
 // ---------------------------------------------------------------------------
-template <int KIND, int OUT_DT>
+template <int KIND, int OUT_DT, bool BIAS>
 __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
   constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
@@ -475,6 +559,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   constexpr bool BLOCK = is_block(KIND);
 
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
+  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -693,10 +778,10 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, cm0, cn0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, cm0, cn0, wm, wn, r16, g, lane,
                                                wave);
       else
-        epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+        epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
     }
     if (!has_next) break;
     tile = next_tile;
@@ -729,7 +814,11 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 // the current one); only the copies behind a tile's last step are deferred to the next
 // tile's first step, because the freed stage stages the C tile.
 // ---------------------------------------------------------------------------
-template <int KIND, int OUT_DT>
+// MODE selects one of three variants, each launched only where it is needed so that the
+// plain one keeps its register allocation: 0 = whole tiles, 1 = split-K work units (raw
+// partial sums to the workspace), 2 = whole tiles of a block-scaled kind with a bias.
+constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2;
+template <int KIND, int OUT_DT, int MODE>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
   constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
@@ -740,6 +829,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
+  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -798,7 +888,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // (all lanes out of range; kept so that the instruction stream has no branch).
   // sc_voff / sc_voff2: per-lane source offsets for the tile of block u + 1 / u + 2.
   const int nkb_all = p.K >> 7;
-  const int nkb = nkb_all / p.splits;  // K blocks of one work unit (the host makes it divide)
+  const int splits = MODE == PIPE_SPLITK ? p.splits : 1;
+  const int nkb = nkb_all / splits;  // K blocks of one work unit (the host makes it divide)
   float sfa_cur[MI];
   float sfb_cur = 0.f;
   __amdgpu_buffer_rsrc_t rsc = ra;
@@ -939,10 +1030,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // output tile, or with split-K (p.splits > 1) one of a tile's p.splits contiguous K ranges,
   // whose raw partial sums go to the workspace for splitk_reduce_kernel.
   const int tiles = p.tiles_m * p.tiles_n;
-  const int total = tiles * p.splits;
+  const int total = tiles * splits;
   const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   auto unit_origin = [&](int u, int& um0, int& un0, int& ukb0) {
-    const int split = u / tiles;
+    const int split = MODE == PIPE_SPLITK ? u / tiles : 0;
     int tm, tn;
     tile_of_block(u - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
     um0 = tm * BM;
@@ -1011,17 +1102,17 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
-    if (p.splits > 1) {
-      store_partials<MI, NI>(p, acc, unit / tiles, m0 + wm * TM, n0 + wn * TN, r16, g);
+    if constexpr (MODE == PIPE_SPLITK) {
+      store_partials_bounded<MI, NI>(p, acc, unit / tiles, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, m0, n0, wm, wn, r16, g, lane,
-                                                   wave);
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, m0, n0, wm, wn,
+                                                                     r16, g, lane, wave);
       else
-        epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+        epilogue<KIND, OUT_DT, MI, NI, (MODE == PIPE_BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     }
     if (!has_next) break;
     unit = next_unit;
@@ -1045,7 +1136,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 // four activation fragments are in registers) and is refilled two K blocks ahead; the
 // weight copies of block u + 2 follow behind the last weight fragment's MFMAs.
 // ---------------------------------------------------------------------------
-template <int KIND, int OUT_DT, int NI>
+template <int KIND, int OUT_DT, int NI, bool BIAS>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   constexpr int BM = 256, NW = 8, WAVES_N = 2, MI = 4;
   constexpr int TM = MI * 16, TN = NI * 16, BN = WAVES_N * TN;
@@ -1058,6 +1149,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
   __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
+  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1345,10 +1437,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN>(p, acc, smem + last_stage * STAGE_BYTES, m0, n0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, m0, n0, wm, wn, r16, g, lane,
                                                    wave);
       else
-        epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+        epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     }
     if (!has_next) break;
     tile = next_tile;
@@ -1760,7 +1852,8 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     if (2 * tiles <= num_cus() || g_force_splits > 0) {
       int want = g_force_splits > 0 ? g_force_splits : num_cus() / tiles;
       const int64_t per_split = (int64_t)p.M * p.N * 4;
-      if (!p.ws || ws_bytes < 2 * per_split) want = 1;
+      // (the kernel addresses a split's partial sums, tile padding included, with 31 bits)
+      if (!p.ws || ws_bytes < 2 * per_split || (int64_t)(p.M + 256) * p.N * 4 >= (int64_t)1 << 31) want = 1;
       else if (want * per_split > ws_bytes) want = (int)(ws_bytes / per_split);
       const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
       if (g_force_splits == 0 && want > by_traffic) want = (int)(by_traffic > 0 ? by_traffic : 1);
@@ -1774,12 +1867,23 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     const int units = tiles * splits;
     const int blocks = units < num_cus() ? units : num_cus();
     g_last_kernel = splits > 1 ? "gemm_pipe_kernel+splitk_reduce_kernel" : "gemm_pipe_kernel";
-    gemm_pipe_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
-    if (splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
+    const dim3 grid((uint32_t)blocks), block(512);
+    if (splits > 1) {
+      gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK><<<grid, block, 0, st>>>(p);
+      launch_reduce<KIND, OUT_DT>(p, st);  // (adds the bias)
+    } else if (is_block(KIND) && p.bias) {
+      if constexpr (is_block(KIND)) gemm_pipe_kernel<KIND, OUT_DT, PIPE_BIAS><<<grid, block, 0, st>>>(p);
+    } else {
+      gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
+    }
   } else {
     const int blocks = tiles < num_cus() ? tiles : num_cus();
     g_last_kernel = "gemm_big_kernel";
-    gemm_big_kernel<KIND, OUT_DT><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+    if (is_block(KIND) && p.bias) {
+      if constexpr (is_block(KIND)) gemm_big_kernel<KIND, OUT_DT, true><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+    } else {
+      gemm_big_kernel<KIND, OUT_DT, false><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+    }
   }
 }
 
@@ -1791,7 +1895,11 @@ static void launch_wide(GemmArgs& p, hipStream_t st) {
   const int tiles = p.tiles_m * p.tiles_n;
   const int blocks = tiles < num_cus() ? tiles : num_cus();
   g_last_kernel = NI == 6 ? "gemm_wide_kernel<6>" : NI == 7 ? "gemm_wide_kernel<7>" : "gemm_wide_kernel<8>";
-  gemm_wide_kernel<KIND, OUT_DT, NI><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  if (is_block(KIND) && p.bias) {
+    if constexpr (is_block(KIND)) gemm_wide_kernel<KIND, OUT_DT, NI, true><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  } else {
+    gemm_wide_kernel<KIND, OUT_DT, NI, false><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  }
 }
 
 // Tile width of the 256-row kernels.  Every CU works through ceil(tiles / CUs) tiles, each
@@ -1986,8 +2094,8 @@ extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel;
 template <int KIND>
 static int blockwise_entry(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb, int64_t sfb_stride_k,
-                           int64_t sfb_stride_n, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
-                           void* workspace, int64_t workspace_bytes, void* stream) {
+                           int64_t sfb_stride_n, const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M,
+                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
@@ -2003,6 +2111,7 @@ static int blockwise_entry(const char* name, const void* a, int64_t lda, const v
   fill_common(p, a, lda, b, ldb, out, ldo, M, N, K);
   p.sa = sfa;
   p.sb = sfb;
+  p.bias = bias;
   p.sa_stride_m = sfa_stride_m;
   p.sa_stride_k = sfa_stride_k;
   p.sb_stride_k = sfb_stride_k;
@@ -2020,7 +2129,17 @@ extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const vo
                                             int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                             int64_t workspace_bytes, void* stream) {
   return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
-                                         sfb_stride_k, sfb_stride_n, out, ldo, out_dtype, M, N, K, workspace,
+                                         sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N, K, workspace,
+                                         workspace_bytes, stream);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                                 int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                                 int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out,
+                                                 int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm_bias", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k,
+                                         sfb, sfb_stride_k, sfb_stride_n, bias, out, ldo, out_dtype, M, N, K, workspace,
                                          workspace_bytes, stream);
 }
 
@@ -2030,7 +2149,7 @@ extern "C" int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const v
                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                              int64_t workspace_bytes, void* stream) {
   return blockwise_entry<KIND_I8_BLOCK>("w8a8_block_int8_matmul", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
-                                        sfb_stride_k, sfb_stride_n, out, ldo, out_dtype, M, N, K, workspace,
+                                        sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N, K, workspace,
                                         workspace_bytes, stream);
 }
 

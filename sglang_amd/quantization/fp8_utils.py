@@ -8,6 +8,7 @@ from typing import List, Optional
 import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
+from ..sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
 from .fp8_kernel import per_token_group_quant_fp8, scaled_fp8_quant, sglang_per_token_quant_fp8
 
 
@@ -30,9 +31,13 @@ def w8a8_block_fp8_linear(
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[0]]
     q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
-    output = fp8_blockwise_scaled_mm(q_input, weight.T, x_scale, weight_scale.T, out_dtype=input_2d.dtype)
-    if bias is not None:
-        output += bias
+    if bias is not None and bias.dtype == input_2d.dtype and bias.is_contiguous() and bias.numel() == weight.shape[0]:
+        # the GEMM and `output += bias` (fp8_utils.py:207-211) in one kernel, same two roundings
+        output = fp8_blockwise_scaled_mm_bias(q_input, weight.T, x_scale, weight_scale.T, input_2d.dtype, bias)
+    else:
+        output = fp8_blockwise_scaled_mm(q_input, weight.T, x_scale, weight_scale.T, out_dtype=input_2d.dtype)
+        if bias is not None:
+            output += bias
     return output.to(dtype=input_2d.dtype).view(*output_shape)
 
 

@@ -186,6 +186,28 @@ def _fp8_blockwise_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype):
     return out
 
 
+def fp8_blockwise_scaled_mm_bias(mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
+    """fp8_blockwise_scaled_mm followed by the caller's `output += bias`
+    (fp8_utils.py:207-211) in one kernel; no counterpart among the reference's ops."""
+    check_mm_common(mat_a, mat_b, out_dtype, FP8, "Float8_e4m3fn")
+    check_blockwise_scales(mat_a, mat_b, scales_a, scales_b)
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    _check(bias.is_cuda and bias.is_contiguous() and bias.numel() == n and bias.dtype == out_dtype,
+           "bias must be a contiguous CUDA tensor of N elements in out_dtype")
+    out = torch.empty((m, n), dtype=out_dtype, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_fp8_blockwise_scaled_mm_bias(
+        mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
+        scales_b.data_ptr(), scales_b.stride(0), scales_b.stride(1), bias.data_ptr(),
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, *_lib.workspace(mat_a.device),
+        _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "fp8_blockwise_scaled_mm_bias")
+    return out
+
+
 def _group_quant_impl(fn_name, q_dtype, input, output_q, output_s, group_size, eps, qmin, qmax):
     check_group_quant(input, output_q, output_s, group_size, q_dtype)
     if input.numel() == 0:

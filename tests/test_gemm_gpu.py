@@ -119,6 +119,40 @@ def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
     torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (5, 2112, 1536), (17, 7168, 2048), (127, 512, 7168), (128, 4096, 256),
+                                 (300, 2048, 1024), (512, 1544, 1024), (1024, 640, 2048)])
+def test_fp8_blockwise_scaled_mm_fused_bias(gpu, tile, mnk, out_dtype):
+    """The fused variant performs the caller's two steps (fp8_utils.py:207-211: the GEMM rounded
+    to the output type, then `output += bias`) in one kernel: bit-identical to doing them apart,
+    on every kernel selection, with and without split-K."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
+
+    say("fp8_blockwise fused bias", mnk, out_dtype, "tile", tile)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(out_dtype).to(gpu)
+    a, b = xq.to(gpu), wq.to(gpu).t()
+    sa, sb = xs.t().contiguous().to(gpu).t(), ws.to(gpu).t()
+    lib = _lib.load()
+    for splits in (0, 2):
+        lib.sglq_debug_force_splits(splits)
+        try:
+            plain = fp8_blockwise_scaled_mm(a, b, sa, sb, out_dtype)
+            kernel_plain = lib.sglq_debug_last_gemm_kernel().decode()
+            fused = fp8_blockwise_scaled_mm_bias(a, b, sa, sb, out_dtype, bias)
+            assert lib.sglq_debug_last_gemm_kernel().decode() == kernel_plain
+        finally:
+            lib.sglq_debug_force_splits(0)
+        plain += bias
+        assert torch.equal(fused.view(torch.int16), plain.view(torch.int16)), (kernel_plain, splits)
+    rows = sample_rows(m)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64) + bias.cpu().float()
+    torch.testing.assert_close(fused.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
 def make_block_int8_case(m, n, k, seed):
     x = O.gen_activation(m, k, seed=seed, outliers=True)
     wq, ws = O.block_quant_weight_int8(O.gen_weight(n, k, seed=seed))

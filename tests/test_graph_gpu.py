@@ -39,7 +39,8 @@ def test_graph_replay_matches_eager(gpu, m):
         xq, xs = per_token_group_quant_int8(x, 128)
         y3 = w8a8_block_int8_matmul(xq, w8, xs, ws8, [128, 128], torch.bfloat16)
         xq, _ = scaled_fp8_quant(x, static_scale)
-        return y0, y1, y2, y3, xq
+        xq_dyn, s_dyn = scaled_fp8_quant(x)  # zero-fills its scale with a fill kernel, then an atomic max
+        return y0, y1, y2, y3, xq, xq_dyn, s_dyn
 
     run(x)  # warm-up outside the capture
     torch.cuda.synchronize()
