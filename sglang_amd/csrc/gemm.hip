@@ -262,7 +262,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
 template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, typename acc_t>
-SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, float* bias_lds, int m0, int n0,
+SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, float* col_lds, int m0, int n0,
                                int wm, int wn, int r16, int g, int lane, int wave) {
   constexpr int TN = NI * 16;
   // The addresses below depend on the lane only, not on the tile: left alone, the compiler
@@ -271,30 +271,30 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   // waits for all copies in flight).  Hide the lane-derived values' origin so that the
   // arithmetic stays here.
   asm volatile("" : "+v"(r16), "+v"(g), "+v"(lane));
-  float bv[NI][4], sbv[NI][4];
-  if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      const int n = n0 + wn * TN + j * 16 + g * 4;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        bv[j][e] = 0.f;
-        sbv[j][e] = 0.f;
-      }
-      if (n < p.N) {
-        const v4f t = *reinterpret_cast<const v4f*>(p.sb + n);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sbv[j][e] = t[e];
-        if (p.bias) load_bias4<OUT_DT>(p.bias, n, bv[j]);
+  constexpr bool ROWCOL = KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL;
+  // Per-row / per-column kinds: the tile's 256 column scales and bias values go through LDS
+  // (`col_lds`: bias in floats 0..255, scales in 256..511) and are read per column group while
+  // converting, so that they do not occupy 8 NI registers next to the accumulators.
+  if constexpr (ROWCOL) {
+    const int t = (int)threadIdx.x & 255, nb = n0 + t;
+    float v = 0.f;
+    if (nb < p.N) {
+      if (threadIdx.x >= 256) v = p.sb[nb];
+      else if (p.bias) {
+        if constexpr (OUT_DT == SGLQ_BF16) v = u2f((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[nb] << 16);
+        else v = (float)reinterpret_cast<const _Float16*>(p.bias)[nb];
       }
     }
+    col_lds[threadIdx.x] = v;
+    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
+    __builtin_amdgcn_s_barrier();
   }
   const int c = lane & 31;
   const int n = n0 + c * 8;
   char* out = reinterpret_cast<char*>(p.out);
   // Block-scaled kinds: the optional bias is the caller's `output += bias` on the rounded
   // result (fp8_utils.py:210-211), added to the image's values on their way out.  The tile's
-  // 256 bias values wait in LDS behind the image (`bias_lds`, 1 KiB, written here and made
+  // 256 bias values wait in LDS behind the image (`col_lds`, written here and made
   // visible by the first barrier below), so that no register holds them across the epilogue.
   // (BIAS: a kernel variant of its own, launched only with a bias, so that the plain variant's
   // register allocation is not disturbed)
@@ -306,29 +306,38 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
       if constexpr (OUT_DT == SGLQ_BF16) b = u2f((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[nb] << 16);
       else b = (float)reinterpret_cast<const _Float16*>(p.bias)[nb];
     }
-    bias_lds[threadIdx.x] = b;
+    col_lds[threadIdx.x] = b;
   }
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     if (((wm * MI * 16) >> 7) == half) {  // wave-uniform: a wave's rows lie in one half
+      float sam[MI];
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        const int ml = ((wm * MI * 16) & 127) + i * 16 + r16;  // row inside the half
-        float sam = 1.f;
-        if constexpr (KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL) {
-          const int m = m0 + half * 128 + ml;
-          sam = (m < p.M) ? p.sa[m] : 0.f;
+        sam[i] = 1.f;
+        if constexpr (ROWCOL) {
+          const int m = m0 + wm * MI * 16 + i * 16 + r16;
+          sam[i] = (m < p.M) ? p.sa[m] : 0.f;
         }
+      }
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
+      for (int j = 0; j < NI; ++j) {
+        v4f bv = {0.f, 0.f, 0.f, 0.f}, sbv = bv;
+        if constexpr (ROWCOL) {
+          bv = *reinterpret_cast<const v4f*>(col_lds + wn * TN + j * 16 + g * 4);
+          sbv = *reinterpret_cast<const v4f*>(col_lds + 256 + wn * TN + j * 16 + g * 4);
+        }
+        const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+          const int ml = ((wm * MI * 16) & 127) + i * 16 + r16;  // row inside the half
           float o[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[j][e] * sam, bv[j][e]);
-            else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam, sbv[j][e] * acc[i][j][e], bv[j][e]);
+            if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[e] * sam[i], bv[e]);
+            else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam[i], sbv[e] * acc[i][j][e], bv[e]);
             else o[e] = acc[i][j][e];
           }
-          const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
           char* dst = img + ml * 512 + ((chunk ^ (ml & 31)) * 16) + (g & 1) * 8;
           if constexpr (OUT_DT == SGLQ_BF16) {
             typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
@@ -349,7 +358,7 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
       const int m = m0 + half * 128 + ml;
       v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
       if constexpr (add_bias) {
-        const v4f blo = *reinterpret_cast<const v4f*>(bias_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(bias_lds + c * 8 + 4);
+        const v4f blo = *reinterpret_cast<const v4f*>(col_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(col_lds + c * 8 + 4);
         const float bias8[8] = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -558,8 +567,12 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
   constexpr bool IS_FP8 = fp8_operands(KIND);
   constexpr bool BLOCK = is_block(KIND);
 
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES];
-  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
+  // One LDS object per kernel: with a second __shared__ array the compiler tells the arrays
+  // apart by alias scopes and then orders every LDS read behind the direct-to-LDS copies in
+  // flight (s_waitcnt vmcnt(0) throughout the K loop).  The epilogue's 512 floats (bias values
+  // and column scales of the tile's columns) therefore live at the end of `smem`.
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2048];
+  float* const col_lds = reinterpret_cast<float*>(smem + 2 * STAGE_BYTES);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -778,7 +791,7 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, cm0, cn0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, cm0, cn0, wm, wn, r16, g, lane,
                                                wave);
       else
         epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
@@ -828,8 +841,9 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   static_assert(NI == 4 && MI == 8, "the copy schedule below is written for 4 x 8 fragments");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
-  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
+  // (one LDS object per kernel, see gemm_big_kernel: the epilogue's 512 floats sit at the end)
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES + 2048];
+  float* const col_lds = reinterpret_cast<float*>(smem + 2 * STAGE_BYTES + 2 * SCALE_BYTES);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1109,7 +1123,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, m0, n0, wm, wn,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn,
                                                                      r16, g, lane, wave);
       else
         epilogue<KIND, OUT_DT, MI, NI, (MODE == PIPE_BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
@@ -1148,8 +1162,9 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES];
-  __shared__ float bias_lds[256];  // the epilogue's bias values of the tile's columns
+  // (one LDS object per kernel, see gemm_big_kernel: the epilogue's 512 floats sit at the end)
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES + 2048];
+  float* const col_lds = reinterpret_cast<float*>(smem + 2 * STAGE_BYTES + 2 * SCALE_BYTES);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1437,7 +1452,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, bias_lds, m0, n0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
                                                    wave);
       else
         epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
