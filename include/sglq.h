@@ -67,6 +67,15 @@ int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* outpu
 int sglq_per_tensor_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
                               int64_t num_elements, int is_static, void* stream);
 
+/* Replaces static_quant_fp8, a Triton kernel in the reference
+ * (python/sglang/srt/layers/quantization/fp8_kernel.py:395-490; caller
+ * apply_fp8_linear, fp8_utils.py:684-689): codes are
+ * clamp(x * (1 / *scale), -448, 448) rounded to e4m3fn for the contiguous
+ * [num_tokens, hidden] input; scale_repeat, if not NULL, receives *scale once per
+ * token ([num_tokens] floats, the reference's repeat_scale=True output [M, 1]). */
+int sglq_static_quant_fp8(const void* input, int in_dtype, void* output_q, const float* scale,
+                          float* scale_repeat, int64_t num_tokens, int64_t hidden, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
  * (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:166-227; schema
  * common_extension.cc:129-130), zero rows giving zero codes as in the

@@ -207,6 +207,24 @@ def per_tensor_quant_fp8(x: torch.Tensor, scale: Optional[torch.Tensor] = None) 
     return v.to(FP8), scale
 
 
+def static_quant_fp8(x: torch.Tensor, x_s: torch.Tensor, repeat_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """python/sglang/srt/layers/quantization/fp8_kernel.py:395-490.
+
+    Per row (:424-430): y widened to fp32, y_s widened to fp32, y_s_inv = 1 / y_s,
+    q = clamp(y * y_s_inv, -448, 448) -> e4m3fn RNE.  With repeat_scale the scale is
+    returned once per row, shape [M, 1] fp32 (:431-432,458-465), otherwise x_s itself (:488).
+    NaN inputs are not pinned: the reference leaves tl.clamp's NaN behaviour open."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    assert x_s.numel() == 1, "only supports per-tensor scale"
+    s = x_s.to(torch.float32).reshape(())
+    inv = torch.tensor(1.0, dtype=torch.float32) / s
+    q = torch.clamp(x.to(torch.float32) * inv, -FP8_E4M3_MAX, FP8_E4M3_MAX).to(FP8)
+    if repeat_scale:
+        m = x.numel() // x.shape[-1]
+        return q, s.reshape(1, 1).repeat(m, 1)
+    return q, x_s
+
+
 # ---------------------------------------------------------------------------
 # a4  block-scaled FP8 GEMM
 # ---------------------------------------------------------------------------

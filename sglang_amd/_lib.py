@@ -28,6 +28,7 @@ SIGNATURES = {
     "sglq_per_token_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_token_quant_int8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_tensor_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p],
+    "sglq_static_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                      c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_bias": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,

@@ -417,12 +417,18 @@ SGLQ_DEV float clamp_like_fminf_fmaxf(float v) {
   return __builtin_fmaxf(__builtin_fminf(v, 448.0f), -448.0f);
 }
 
+// `repeat` (optional): the scale broadcast to `repeat_n` floats, one per token, which is what
+// static_quant_fp8 hands to a GEMM that takes per-token scales (fp8_kernel.py:431-432,458-465).
 template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void tensor_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
-                                                           const float* __restrict__ s, int64_t n) {
-  const float inv = 1.0f / *s;  // per_tensor_quant_fp8.cu:56
+                                                           const float* __restrict__ s, int64_t n,
+                                                           float* __restrict__ repeat, int64_t repeat_n) {
+  const float scale = *s;
+  const float inv = 1.0f / scale;  // per_tensor_quant_fp8.cu:56, fp8_kernel.py:428
   const int64_t nchunks = VEC ? (n >> 3) : 0;
   const int64_t stride = (int64_t)gridDim.x * 256;
+  if (repeat)
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < repeat_n; t += stride) repeat[t] = scale;
   for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += stride) {
     Chunk8<DT> ch;
     ch.load(x + c * Chunk8<DT>::kBytes);
@@ -589,7 +595,8 @@ static int token_quant_entry(const char* name, const void* input, int in_dtype, 
 }
 
 template <int DT>
-static void launch_tensor_quant(const void* x, void* q, float* s, int64_t n, bool is_static, hipStream_t st) {
+static void launch_tensor_quant(const void* x, void* q, float* s, int64_t n, bool is_static, hipStream_t st,
+                                float* repeat = nullptr, int64_t repeat_n = 0) {
   const bool vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
   const int64_t work = vec ? (n + 7) / 8 : n;
   int64_t blocks = (work + 255) / 256;
@@ -603,10 +610,10 @@ static void launch_tensor_quant(const void* x, void* q, float* s, int64_t n, boo
   char* qc = static_cast<char*>(q);
   if (vec) {
     if (!is_static) tensor_absmax_kernel<DT, true><<<grid_max, block, 0, st>>>(xc, s, n);
-    tensor_quant_kernel<DT, true><<<grid, block, 0, st>>>(xc, qc, s, n);
+    tensor_quant_kernel<DT, true><<<grid, block, 0, st>>>(xc, qc, s, n, repeat, repeat_n);
   } else {
     if (!is_static) tensor_absmax_kernel<DT, false><<<grid_max, block, 0, st>>>(xc, s, n);
-    tensor_quant_kernel<DT, false><<<grid, block, 0, st>>>(xc, qc, s, n);
+    tensor_quant_kernel<DT, false><<<grid, block, 0, st>>>(xc, qc, s, n, repeat, repeat_n);
   }
 }
 
@@ -638,7 +645,42 @@ static int tensor_quant_entry(const void* input, int in_dtype, void* output_q, f
   return check_launch(name);
 }
 
+static int static_quant_entry(const void* input, int in_dtype, void* output_q, const float* scale, float* scale_repeat,
+                              int64_t num_tokens, int64_t hidden, void* stream) {
+  const char* name = "static_quant_fp8";
+  if (num_tokens < 0 || hidden < 0) {
+    set_error("%s: negative shape", name);
+    return SGLQ_EINVAL;
+  }
+  if (!scale) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t n = num_tokens * hidden;
+  if (n > 0 && (!input || !output_q)) {
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (n == 0 && !(scale_repeat && num_tokens > 0)) return SGLQ_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* s = const_cast<float*>(scale);  // static mode only reads it
+  switch (in_dtype) {
+    case SGLQ_BF16: launch_tensor_quant<SGLQ_BF16>(input, output_q, s, n, true, st, scale_repeat, num_tokens); break;
+    case SGLQ_FP16: launch_tensor_quant<SGLQ_FP16>(input, output_q, s, n, true, st, scale_repeat, num_tokens); break;
+    case SGLQ_FP32: launch_tensor_quant<SGLQ_FP32>(input, output_q, s, n, true, st, scale_repeat, num_tokens); break;
+    default:
+      set_error("%s: input dtype must be bf16, fp16 or fp32", name);
+      return SGLQ_EUNSUPPORTED;
+  }
+  return check_launch(name);
+}
+
 }  // namespace sglq
+
+extern "C" int sglq_static_quant_fp8(const void* input, int in_dtype, void* output_q, const float* scale,
+                                     float* scale_repeat, int64_t num_tokens, int64_t hidden, void* stream) {
+  return sglq::static_quant_entry(input, in_dtype, output_q, scale, scale_repeat, num_tokens, hidden, stream);
+}
 
 extern "C" int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
                                               int64_t num_tokens, int64_t hidden, int group_size,

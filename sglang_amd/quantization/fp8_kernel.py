@@ -6,8 +6,10 @@ from __future__ import annotations
 
 import torch
 
-from typing import Optional
+from typing import Optional, Tuple
 
+from .. import _lib
+from .._lib import DTYPE_CODE
 from ..sgl_kernel import sgl_per_tensor_quant_fp8, sgl_per_token_group_quant_fp8, sgl_per_token_quant_fp8
 
 # gfx950 implements the OCP formats: e4m3fn with maximum 448 (fp8_kernel.py:71-85
@@ -77,6 +79,31 @@ def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
     x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
     sgl_per_token_quant_fp8(x, x_q, x_s)
     return x_q, x_s
+
+
+def static_quant_fp8(
+    x: torch.Tensor,
+    x_s: torch.Tensor,
+    repeat_scale: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp8_kernel.py:437-490: quantize `x` (ndim >= 2, contiguous) with the given per-tensor
+    scale; with repeat_scale the returned scale is that value once per token, shape [M, 1]."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    assert x_s.numel() == 1, "only supports per-tensor scale"
+    if not x.is_cuda:
+        raise RuntimeError("static_quant_fp8: input must be a CUDA tensor")
+    if x.dtype not in DTYPE_CODE:
+        raise NotImplementedError(f"static_quant_fp8: unsupported input dtype {x.dtype}")
+    x_q = torch.empty_like(x, device=x.device, dtype=fp8_dtype)
+    n = x.shape[-1]
+    m = x.numel() // n if n > 0 else 0
+    scale = x_s if x_s.dtype == torch.float32 and x_s.device == x.device else x_s.to(device=x.device, dtype=torch.float32)
+    x_s_repeat = torch.empty((m, 1), device=x.device, dtype=torch.float32) if repeat_scale else None
+    rc = _lib.load().sglq_static_quant_fp8(
+        x.data_ptr(), DTYPE_CODE[x.dtype], x_q.data_ptr(), scale.data_ptr(),
+        x_s_repeat.data_ptr() if repeat_scale else None, m, n, _lib.stream_ptr(x.device))
+    _lib.check(rc, "static_quant_fp8")
+    return x_q, (x_s_repeat if repeat_scale else x_s)
 
 
 def scaled_fp8_quant(

@@ -9,7 +9,7 @@ import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from ..sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
-from .fp8_kernel import per_token_group_quant_fp8, scaled_fp8_quant, sglang_per_token_quant_fp8
+from .fp8_kernel import per_token_group_quant_fp8, sglang_per_token_quant_fp8, static_quant_fp8
 
 
 def w8a8_block_fp8_linear(
@@ -55,10 +55,10 @@ def apply_fp8_linear(
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[1]]
     if input_scale is not None:
-        # static per-tensor activation scale (scaled_fp8_quant, fp8_utils.py:569-573); the GEMM
-        # takes one scale per row, so the scalar is repeated
-        qinput, x_scale = scaled_fp8_quant(input_2d, input_scale)
-        x_scale = x_scale.reshape(1, 1).expand(input_2d.shape[0], 1).contiguous()
+        # static per-tensor activation scale, broadcast to one scale per token because the GEMM
+        # takes per-token scales (fp8_utils.py:684-689)
+        assert input_scale.numel() == 1
+        qinput, x_scale = static_quant_fp8(input_2d.contiguous(), input_scale, repeat_scale=True)
     else:
         qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
     assert weight_scale.numel() == weight.shape[1], "cutlass w8a8 fp8 sgl-kernel only supports per-channel scale"

@@ -54,8 +54,8 @@ def test_fp8_per_channel_linear(gpu):
 
 
 def test_fp8_static_activation_scale_linear(gpu):
-    """apply_fp8_linear with a static per-tensor activation scale: scaled_fp8_quant
-    (fp8_utils.py:569-573) then the per-channel GEMM."""
+    """apply_fp8_linear with a static per-tensor activation scale: static_quant_fp8 with the
+    scale repeated per token (fp8_utils.py:684-689), then the per-channel GEMM."""
     from sglang_amd.quantization.fp8_utils import apply_fp8_linear
 
     print("fp8 linear, static activation scale", flush=True)
@@ -63,7 +63,7 @@ def test_fp8_static_activation_scale_linear(gpu):
     wq, ws = O.per_tensor_quant_weight(O.gen_weight(4096, 4096, seed=3003))
     in_scale = torch.tensor([0.02], dtype=torch.float32)
     bias = (torch.randn(4096, generator=torch.Generator().manual_seed(2)) * 0.1).to(torch.bfloat16)
-    xq, _ = O.per_tensor_quant_fp8(x, in_scale)
-    ref = O.fp8_scaled_mm(xq, wq.t(), in_scale.expand(48, 1), ws, torch.bfloat16, bias)
+    xq, xs = O.static_quant_fp8(x, in_scale, repeat_scale=True)
+    ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16, bias)
     out = apply_fp8_linear(x.to(gpu), wq.to(gpu).t(), ws.to(gpu), input_scale=in_scale.to(gpu), bias=bias.to(gpu))
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)

@@ -237,6 +237,39 @@ def test_tensor_fp8_closed_form_and_zero_tensor(c_oracle):
     assert fp8_bits(q).unique().tolist() == [0x7E] and qc.unique().tolist() == [0x7E]
 
 
+# ------------------------------------------------------------------ f2 static per-tensor quant
+@pytest.mark.parametrize("dtype", [torch.half, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("num_tokens,d", [(7, 512), (83, 4096), (33, 5120)])
+def test_static_quant_fp8_vs_reference_test_formula(c_oracle, dtype, num_tokens, d):
+    """The reference's own check (python/sglang/test/test_block_fp8.py:98-159): uniform inputs,
+    scale = max / 448 in the input's dtype, native torch formula, allclose at rtol 0.5.  In fp32
+    the native formula is the kernel's arithmetic, so the codes must be identical; the C
+    restatement's static per-tensor path must agree bit for bit for every dtype."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand((num_tokens, d), generator=g).to(dtype)
+    x_s = x.max() / 448.0
+    native = (x * (1.0 / x_s)).clamp(min=-448.0, max=448.0).to(FP8)
+    q, s = O.static_quant_fp8(x, x_s, repeat_scale=True)
+    assert torch.allclose(q.float(), native.float(), rtol=0.50)
+    if dtype == torch.float32:
+        assert_bits_equal(q, native, "codes vs the reference test's native formula")
+    assert tuple(s.shape) == (num_tokens, 1) and s.dtype == torch.float32
+    assert torch.all(s == x_s.float())
+    qc, _ = c_tensor_quant_fp8(c_oracle, x, x_s.float().reshape(1))
+    assert_bits_equal(fp8_bits(q), qc, "codes vs C restatement")
+    q2, s2 = O.static_quant_fp8(x, x_s)
+    assert s2 is x_s and torch.equal(fp8_bits(q2), fp8_bits(q))
+
+
+def test_static_quant_fp8_closed_form():
+    # power-of-two scale: x / s is exact, representable values come back, the rest saturates or rounds to even
+    x = torch.tensor([[0.5, -1.0, 100.0, 0.0, 0.0634765625, -1e9, 3.25 * 0.125, 17.0 * 0.125]])
+    q, s = O.static_quant_fp8(x, torch.tensor(0.125))
+    assert q.float().tolist() == [[4.0, -8.0, 448.0, 0.0, 0.5, -448.0, 3.25, 16.0]]
+    q, s = O.static_quant_fp8(x.reshape(2, 2, 2), torch.tensor([0.125], dtype=torch.bfloat16), repeat_scale=True)
+    assert tuple(q.shape) == (2, 2, 2) and s.tolist() == [[0.125]] * 4
+
+
 # ------------------------------------------------------------------ GEMMs
 def rand_fp8(shape, seed, scale=1.0):
     g = torch.Generator().manual_seed(seed)

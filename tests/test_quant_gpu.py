@@ -227,6 +227,50 @@ def test_tensor_quant_fp8_unaligned_zero_and_padding(gpu):
     assert_bits_equal(s, s_ref, "per-token scales")
 
 
+@pytest.mark.parametrize("dtype", [torch.half, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("num_tokens", [7, 83, 2048])
+@pytest.mark.parametrize("d", [512, 4096, 5120, 13824])
+def test_static_quant_fp8_bit_exact(gpu, dtype, num_tokens, d):
+    """static_quant_fp8 on the grid of the reference's test (python/sglang/test/test_block_fp8.py:119-159:
+    uniform inputs, scale = max / 448 in the input's dtype), bit for bit against the oracle, with
+    and without the repeated scale."""
+    from sglang_amd.quantization.fp8_kernel import static_quant_fp8
+
+    say("static_quant", dtype, num_tokens, d)
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand((num_tokens, d), generator=g).to(dtype)
+    x_s = x.max() / 448.0
+    q_ref, s_ref = O.static_quant_fp8(x, x_s, repeat_scale=True)
+    xg, sg = x.to(gpu), x_s.to(gpu)
+    q, s = static_quant_fp8(xg, sg, repeat_scale=True)
+    assert q.dtype == FP8 and q.shape == x.shape and tuple(s.shape) == (num_tokens, 1) and s.dtype == torch.float32
+    assert_bits_equal(q, q_ref, "codes")
+    assert_bits_equal(s, s_ref, "repeated scale")
+    q, s = static_quant_fp8(xg, sg)
+    assert s is sg
+    assert_bits_equal(q, q_ref, "codes, scale not repeated")
+
+
+def test_static_quant_fp8_shapes_and_errors(gpu):
+    from sglang_amd.quantization.fp8_kernel import static_quant_fp8
+
+    # ndim 3, a length that is not a multiple of 8, values beyond the range
+    x = (O.gen_activation(6, 203, seed=4, outliers=True).float() * 40).reshape(2, 3, 203).contiguous()
+    scale = torch.tensor([0.25])
+    q_ref, s_ref = O.static_quant_fp8(x, scale, repeat_scale=True)
+    q, s = static_quant_fp8(x.to(gpu), scale.to(gpu), repeat_scale=True)
+    assert q.shape == x.shape and tuple(s.shape) == (6, 1)
+    assert_bits_equal(q, q_ref, "codes, 3-D input")
+    assert_bits_equal(s, s_ref, "repeated scale, 3-D input")
+    assert float(q.float().abs().max()) == 448.0
+    with pytest.raises(AssertionError, match="not contiguous"):
+        static_quant_fp8(x.to(gpu).transpose(0, 1), scale.to(gpu))
+    with pytest.raises(AssertionError, match="per-tensor"):
+        static_quant_fp8(x.to(gpu), torch.ones(2, device=gpu))
+    q, s = static_quant_fp8(torch.empty((0, 64), device=gpu, dtype=torch.bfloat16), scale.to(gpu), repeat_scale=True)
+    assert q.shape == (0, 64) and s.shape == (0, 1)
+
+
 def test_tensor_quant_full_size_properties(gpu):
     """8192 x 16384 (the largest activation of the configurations): quantizing the dequantized
     tensor with the same static scale reproduces the codes; the maximum code is 448."""
