@@ -253,12 +253,14 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
   }
 }
 
-// Epilogue of the 256-row kernels for 16-bit outputs, in two halves of 128 rows: the
-// waves that own the half convert their accumulators (scales and bias applied) and drop
-// them into a 128 x 512-byte image in one stage buffer, then all eight waves write the
-// image out in rows, 16 bytes per lane, so that a wavefront store covers two full 512-byte
-// row segments instead of sixteen 32-byte pieces.  Chunk c (16 bytes) of row r sits at
-// chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
+// Epilogue of the 256-row kernels for 16-bit outputs, in two halves of 128 rows: every
+// wave converts one half of its accumulators (fragment rows i < MI / 2, then the rest; scales
+// and bias applied) and drops them into a 128 x 512-byte image in one stage buffer, then all
+// eight waves write the image out in rows, 16 bytes per lane, so that a wavefront store
+// covers two full 512-byte row segments instead of sixteen 32-byte pieces.  A half is
+// therefore the upper (lower) 8 MI rows of every wave row's 16 MI; splitting the tile into
+// its upper and lower 128 rows instead leaves half of the waves idle while the others
+// convert.  Chunk c (16 bytes) of image row r sits at chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
 template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, typename acc_t>
@@ -308,16 +310,26 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
     }
     col_lds[threadIdx.x] = b;
   }
+  constexpr int HR = MI * 8;  // rows of a wave row in one half
+  // The tile's part of the output as a buffer: rows m0 .. min(M, m0 + 256) - 1 from column n0
+  // on.  Used when every 16-byte chunk of the tile's columns lies inside N and the extent fits
+  // the 31-bit offsets (wave-uniform conditions).
+  const uint32_t row_bytes = (uint32_t)p.ldo * 2u;
+  const int rows_left = p.M - m0 < 256 ? p.M - m0 : 256;
+  const bool whole_chunks = n0 + BN <= p.N && p.ldo < (1 << 21);
+  const __amdgpu_buffer_rsrc_t r_out =
+      make_rsrc(out + ((int64_t)m0 * p.ldo + n0) * 2, whole_chunks ? (uint32_t)rows_left * row_bytes - (uint32_t)n0 * 2u : 0u);
+  static_assert(MI % 2 == 0 && (HR & (HR - 1)) == 0 && 128 % HR == 0, "the halves are split by fragment row");
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    if (((wm * MI * 16) >> 7) == half) {  // wave-uniform: a wave's rows lie in one half
-      float sam[MI];
+    {
+      float sam[MI / 2];
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        sam[i] = 1.f;
+      for (int ii = 0; ii < MI / 2; ++ii) {
+        sam[ii] = 1.f;
         if constexpr (ROWCOL) {
-          const int m = m0 + wm * MI * 16 + i * 16 + r16;
-          sam[i] = (m < p.M) ? p.sa[m] : 0.f;
+          const int m = m0 + wm * MI * 16 + half * HR + ii * 16 + r16;
+          sam[ii] = (m < p.M) ? p.sa[m] : 0.f;
         }
       }
 #pragma unroll
@@ -329,13 +341,14 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
         }
         const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-          const int ml = ((wm * MI * 16) & 127) + i * 16 + r16;  // row inside the half
+        for (int ii = 0; ii < MI / 2; ++ii) {
+          const int i = half * (MI / 2) + ii;
+          const int ml = wm * HR + ii * 16 + r16;  // row inside the image
           float o[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[e] * sam[i], bv[e]);
-            else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam[i], sbv[e] * acc[i][j][e], bv[e]);
+            if constexpr (KIND == KIND_I8_ROWCOL) o[e] = __builtin_fmaf((float)acc[i][j][e], sbv[e] * sam[ii], bv[e]);
+            else if constexpr (KIND == KIND_FP8_ROWCOL) o[e] = __builtin_fmaf(sam[ii], sbv[e] * acc[i][j][e], bv[e]);
             else o[e] = acc[i][j][e];
           }
           char* dst = img + ml * 512 + ((chunk ^ (ml & 31)) * 16) + (g & 1) * 8;
@@ -351,39 +364,61 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
     __builtin_amdgcn_s_barrier();
-    // 128 rows, 8 waves: wave w writes rows 16 w .. 16 w + 15, two rows per store instruction
-#pragma unroll 4
+    // 128 image rows, 8 waves: wave w writes rows 16 w .. 16 w + 15, two rows per store
+    // instruction; image row ml is row ml % HR of wave row ml / HR's half.  All eight reads are
+    // issued before the first store (one LDS latency instead of eight).
+    v4i v[8];
+#pragma unroll
     for (int it = 0; it < 8; ++it) {
       const int ml = wave * 16 + it * 2 + (lane >> 5);
-      const int m = m0 + half * 128 + ml;
-      v4i v = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
-      if constexpr (add_bias) {
-        const v4f blo = *reinterpret_cast<const v4f*>(col_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(col_lds + c * 8 + 4);
-        const float bias8[8] = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
+      v[it] = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
+    }
+    if constexpr (add_bias) {
+      const v4f blo = *reinterpret_cast<const v4f*>(col_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(col_lds + c * 8 + 4);
+      const float bias8[8] = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t w = (uint32_t)v[q];
+          const uint32_t w = (uint32_t)v[it][q];
           float lo, hi;
           if constexpr (OUT_DT == SGLQ_BF16) {
             lo = u2f(w << 16) + bias8[2 * q];
             hi = u2f(w & 0xffff0000u) + bias8[2 * q + 1];
             typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-            v[q] = __builtin_bit_cast(int, bf2{(__bf16)lo, (__bf16)hi});
+            v[it][q] = __builtin_bit_cast(int, bf2{(__bf16)lo, (__bf16)hi});
           } else {
             typedef _Float16 h2 __attribute__((ext_vector_type(2)));
             const h2 h = __builtin_bit_cast(h2, w);
             lo = (float)h[0] + bias8[2 * q];
             hi = (float)h[1] + bias8[2 * q + 1];
-            v[q] = __builtin_bit_cast(int, h2{(_Float16)lo, (_Float16)hi});
+            v[it][q] = __builtin_bit_cast(int, h2{(_Float16)lo, (_Float16)hi});
           }
         }
       }
-      if (m < p.M && c * 8 < BN) {
-        char* row = out + ((int64_t)m * p.ldo + n) * 2;
-        if (n + 8 <= p.N) {
-          *reinterpret_cast<v4i*>(row) = v;
-        } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
-          *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[0], (uint32_t)v[1]};
+    }
+    if (whole_chunks) {
+      // bounds-checked buffer stores: rows past M and lanes past the tile's width get an offset
+      // beyond the extent and are dropped; no branches, no 64-bit address arithmetic
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int ml = wave * 16 + it * 2 + (lane >> 5);
+        const uint32_t m_rel = (uint32_t)((ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1)));
+        const uint32_t voff = (c * 8 < BN) ? m_rel * row_bytes + (uint32_t)c * 16u : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int ml = wave * 16 + it * 2 + (lane >> 5);
+        const int m = m0 + (ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1));
+        if (m < p.M && c * 8 < BN) {
+          char* row = out + ((int64_t)m * p.ldo + n) * 2;
+          if (n + 8 <= p.N) {
+            *reinterpret_cast<v4i*>(row) = v[it];
+          } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
+            *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[it][0], (uint32_t)v[it][1]};
+          }
         }
       }
     }
