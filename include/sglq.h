@@ -123,6 +123,29 @@ int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b,
                                       int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                       int64_t workspace_bytes, void* stream);
 
+/* Replaces torch.ops.sgl_kernel.fp8_blockwise_scaled_grouped_mm
+ * (sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:587-754; schema
+ * common_extension.cc:192-197; callers python/sglang/srt/layers/moe/cutlass_moe.py:170-213):
+ * num_experts block-scaled FP8 GEMMs that share N and K in one launch sequence.  Expert e
+ * multiplies rows expert_offsets[e] .. expert_offsets[e] + problem_sizes[e][0] - 1 of
+ * a [total_m, K] (e4m3fn, row stride lda) with its weight b + e * b_expert_stride
+ * ([N, K] rows of ldb bytes, i.e. the reference's column-major [K, N] slice) into the same
+ * rows of out [total_m, N].  sfa [total_m, K/128] (element strides given; the reference's
+ * K-major SM100 convention is strides (K/128, 1)), sfb element (e, kb, nb) at
+ * sfb + e * sfb_expert_stride + kb * sfb_stride_k + nb * sfb_stride_n.  problem_sizes
+ * ([num_experts, 3] int32, only column 0 is read: N and K are arguments) and
+ * expert_offsets ([num_experts] int32) are DEVICE pointers: nothing is copied to the host.
+ * The reference's pointer, stride and layout scratch tensors have no counterpart; the
+ * workspace holds the tile plan, 16 * (total_m / 32 + num_experts + 1) bytes always suffice.
+ * Rows outside every expert's range are left untouched. */
+int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                         int64_t b_expert_stride, const float* sfa, int64_t sfa_stride_m,
+                                         int64_t sfa_stride_k, const float* sfb, int64_t sfb_expert_stride,
+                                         int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                         int out_dtype, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                                         int64_t num_experts, int64_t total_m, int64_t N, int64_t K, void* workspace,
+                                         int64_t workspace_bytes, void* stream);
+
 /* Replaces w8a8_block_int8_matmul, a Triton kernel in the reference
  * (python/sglang/srt/layers/quantization/int8_kernel.py:212-425; there is no
  * sgl_kernel C++ op): out[m,n] = sum_kb float(sum_{k in block kb} a[m,k] b[k,n])

@@ -260,6 +260,33 @@ def fp8_blockwise_scaled_mm(
     return out.to(out_dtype)
 
 
+def fp8_blockwise_scaled_grouped_mm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scales_a: torch.Tensor,
+    scales_b: torch.Tensor,
+    problem_sizes: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    out_dtype: torch.dtype,
+    acc_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:587-754 (semantics; callers
+    python/sglang/srt/layers/moe/cutlass_moe.py:170-213): expert e computes the block-scaled
+    product of rows expert_offsets[e] .. + problem_sizes[e][0] of a [total_m, K] with b[e]
+    ([K, N]), activation scales scales_a [total_m, K/128] (K-major), weight scales
+    scales_b[e] [K/128, N/128], into the same rows of the output.  Rows that belong to no
+    expert are returned as zeros (the operator leaves them untouched)."""
+    total_m, n = a.shape[0], b.shape[2]
+    out = torch.zeros((total_m, n), dtype=out_dtype)
+    for e in range(b.shape[0]):
+        rows, first = int(problem_sizes[e][0]), int(expert_offsets[e])
+        if rows == 0:
+            continue
+        sl = slice(first, first + rows)
+        out[sl] = fp8_blockwise_scaled_mm(a[sl], b[e], scales_a[sl], scales_b[e], out_dtype, acc_dtype=acc_dtype)
+    return out
+
+
 # ---------------------------------------------------------------------------
 # a5  INT8 scaled GEMM
 # ---------------------------------------------------------------------------

@@ -51,9 +51,14 @@ struct GemmArgs {
   uint32_t a_bytes, b_bytes;
   int M, N, K;
   int tiles_m, tiles_n;
-  void* ws;        // split-K partial sums [splits][M][N], fp32 or int32
+  void* ws;        // split-K partial sums [splits][M][N], fp32 or int32; grouped GEMM: the tile plan
   int splits;
+  int64_t b_expert_stride, sb_expert_stride;  // grouped GEMM: bytes / floats between experts' weights / weight scales
 };
+
+// Grouped GEMM tile plan in the workspace (int32): [0] = number of row tiles, then from [4] on
+// one entry of four per row tile: expert, first row, end row (both absolute rows of A and C).
+constexpr int PLAN_HEADER = 4, PLAN_ENTRY = 4;
 
 // s_waitcnt immediate: wait until at most `vm` vector-memory loads are outstanding
 // and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
@@ -427,8 +432,13 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   }
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT, bool DMA>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const GemmArgs p) {
+// GROUPED: one launch for a group of problems that share N and K (the experts of an MoE
+// layer).  Row tile t of the grid belongs to expert plan[t].expert and covers rows
+// plan[t].row0 .. of A and C up to the expert's last row; B and its scales are the
+// expert's.  Rows of the tile beyond the expert's are other experts' rows: they are
+// computed and dropped by the epilogue's row bound.
+template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT, bool DMA, bool GROUPED = false>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const GemmArgs p_in) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;  // per-wave tile
   constexpr int MI = TM / 16, NI = TN / 16;
@@ -446,11 +456,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_kernel(const Ge
   const int r16 = lane & 15, g = lane >> 4;
 
   // blockIdx = split * tiles + tile; split s works on K blocks [kb_lo, kb_hi)
+  GemmArgs p = p_in;
   const int tiles = p.tiles_m * p.tiles_n;
-  const int split = blockIdx.x / tiles;
+  const int split = GROUPED ? 0 : blockIdx.x / tiles;
   int tm, tn;
   tile_of_block(blockIdx.x - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
+  int m0 = tm * BM;
+  const int n0 = tn * BN;
+  if constexpr (GROUPED) {
+    const int* plan = static_cast<const int*>(p.ws);
+    if (tm >= plan[0]) return;  // the grid covers the largest possible number of row tiles
+    const int* entry = plan + PLAN_HEADER + PLAN_ENTRY * tm;
+    const int expert = entry[0];
+    m0 = entry[1];
+    p.M = entry[2];
+    p.b += (int64_t)expert * p.b_expert_stride;
+    p.sb += (int64_t)expert * p.sb_expert_stride;
+  }
 
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, p.a_bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, p.b_bytes);
@@ -1850,6 +1872,64 @@ static thread_local const char* g_last_kernel = "";  // which GEMM kernel the ca
 template <int KIND, int OUT_DT>
 static void launch_reduce(GemmArgs& p, hipStream_t st);
 
+// Tile plan of a grouped GEMM, from the experts' row counts and first rows in device memory
+// (problem_sizes[e][0], expert_offsets[e]); one block.  Inconsistent inputs cannot make the
+// GEMM leave its buffers: rows are clamped to [0, total_m] and tiles to the grid's count.
+__global__ __launch_bounds__(256) void grouped_plan_kernel(const int* __restrict__ problem_sizes,
+                                                          const int* __restrict__ expert_offsets, int num_experts,
+                                                          int total_m, int bm, int max_tiles, int* __restrict__ plan) {
+  __shared__ int scan[256];
+  __shared__ int base_s;
+  const int tid = threadIdx.x;
+  if (tid == 0) base_s = 0;
+  __syncthreads();
+  for (int e0 = 0; e0 < num_experts; e0 += 256) {
+    const int e = e0 + tid;
+    int rows = 0, first = 0;
+    if (e < num_experts) {
+      first = expert_offsets[e];
+      rows = problem_sizes[3 * e];
+      if (first < 0) first = 0;
+      if (first > total_m) first = total_m;
+      if (rows < 0) rows = 0;
+      if (rows > total_m - first) rows = total_m - first;
+    }
+    const int t = (rows + bm - 1) / bm;
+    scan[tid] = t;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int v = tid >= d ? scan[tid - d] : 0;
+      __syncthreads();
+      scan[tid] += v;
+      __syncthreads();
+    }
+    const int begin = base_s + scan[tid] - t;
+    for (int i = 0; i < t; ++i) {
+      const int slot = begin + i;
+      if (slot < max_tiles) {
+        int* entry = plan + PLAN_HEADER + PLAN_ENTRY * slot;
+        entry[0] = e;
+        entry[1] = first + i * bm;
+        entry[2] = first + rows;
+        entry[3] = 0;
+      }
+    }
+    __syncthreads();
+    if (tid == 255) base_s += scan[255];
+    __syncthreads();
+  }
+  if (tid == 0) plan[0] = base_s < max_tiles ? base_s : max_tiles;
+}
+
+template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT>
+static void launch_grouped_cfg(GemmArgs& p, int max_tiles, hipStream_t st) {
+  p.tiles_m = max_tiles;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  p.splits = 1;
+  const dim3 grid((uint32_t)(p.tiles_m * p.tiles_n)), block(WAVES_M * WAVES_N * 64);
+  gemm_kernel<KIND, BM, BN, WAVES_M, WAVES_N, OUT_DT, true, true><<<grid, block, 0, st>>>(p);
+}
+
 // 128 x 128 (and narrower) tiles.  When the tiles do not fill the chip (two blocks per
 // CU), K is split across blocks as far as the workspace and the partial sums' traffic allow.
 template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT>
@@ -2191,6 +2271,80 @@ extern "C" int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, con
   return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm_bias", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k,
                                          sfb, sfb_stride_k, sfb_stride_n, bias, out, ldo, out_dtype, M, N, K, workspace,
                                          workspace_bytes, stream);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                                    int64_t b_expert_stride, const float* sfa, int64_t sfa_stride_m,
+                                                    int64_t sfa_stride_k, const float* sfb, int64_t sfb_expert_stride,
+                                                    int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                                    int out_dtype, const int32_t* problem_sizes,
+                                                    const int32_t* expert_offsets, int64_t num_experts, int64_t total_m,
+                                                    int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                                    void* stream) {
+  using namespace sglq;
+  const char* name = "fp8_blockwise_scaled_grouped_mm";
+  if (num_experts < 0) {
+    set_error("%s: negative number of experts", name);
+    return SGLQ_EINVAL;
+  }
+  int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, total_m, N, K, 2);
+  if (rc < 0 || num_experts == 0) return SGLQ_OK;
+  if (rc) return rc;
+  if (!sfa || !sfb || !problem_sizes || !expert_offsets) {
+    set_error("%s: null scale, problem_sizes or expert_offsets pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (out_dtype != SGLQ_BF16 && out_dtype != SGLQ_FP16) {
+    set_error("%s: output must be bfloat16 or half", name);
+    return SGLQ_EINVAL;
+  }
+  if (K % 128 != 0) {
+    set_error("%s: K (%lld) must be a multiple of 128", name, (long long)K);
+    return SGLQ_EINVAL;
+  }
+  if (b_expert_stride % 16 != 0 || num_experts >= (1 << 20)) {
+    set_error("%s: the experts' weights must be 16-byte aligned, fewer than 2^20 experts", name);
+    return SGLQ_EINVAL;
+  }
+  // row tile height from the average group: the experts' row counts are device data
+  const int64_t avg = total_m / num_experts;
+  const int bm = avg <= 32 ? 32 : avg <= 64 ? 64 : 128;
+  const int64_t max_tiles = total_m / bm + num_experts;
+  const int64_t need = (int64_t)(PLAN_HEADER + PLAN_ENTRY * max_tiles) * 4;
+  if (!workspace || workspace_bytes < need) {
+    set_error("%s: workspace of %lld bytes needed for the tile plan (%lld given)", name, (long long)need,
+              (long long)workspace_bytes);
+    return SGLQ_EINVAL;
+  }
+  if (max_tiles * ((N + 127) / 128) >= (1ll << 31)) {
+    set_error("%s: too many tiles", name);
+    return SGLQ_EUNSUPPORTED;
+  }
+  GemmArgs p;
+  fill_common(p, a, lda, b, ldb, out, ldo, total_m, N, K);
+  p.sa = sfa;
+  p.sb = sfb;
+  p.sa_stride_m = sfa_stride_m;
+  p.sa_stride_k = sfa_stride_k;
+  p.sb_stride_k = sfb_stride_k;
+  p.sb_stride_n = sfb_stride_n;
+  p.b_expert_stride = b_expert_stride;
+  p.sb_expert_stride = sfb_expert_stride;
+  p.ws = workspace;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  grouped_plan_kernel<<<dim3(1), dim3(256), 0, st>>>(problem_sizes, expert_offsets, (int)num_experts, (int)total_m, bm,
+                                                     (int)max_tiles, static_cast<int*>(workspace));
+  g_last_kernel = "grouped_plan_kernel+gemm_kernel<grouped>";
+  if (out_dtype == SGLQ_BF16) {
+    if (bm == 32) launch_grouped_cfg<KIND_FP8_BLOCK, 32, 128, 1, 4, SGLQ_BF16>(p, (int)max_tiles, st);
+    else if (bm == 64) launch_grouped_cfg<KIND_FP8_BLOCK, 64, 128, 1, 4, SGLQ_BF16>(p, (int)max_tiles, st);
+    else launch_grouped_cfg<KIND_FP8_BLOCK, 128, 128, 2, 2, SGLQ_BF16>(p, (int)max_tiles, st);
+  } else {
+    if (bm == 32) launch_grouped_cfg<KIND_FP8_BLOCK, 32, 128, 1, 4, SGLQ_FP16>(p, (int)max_tiles, st);
+    else if (bm == 64) launch_grouped_cfg<KIND_FP8_BLOCK, 64, 128, 1, 4, SGLQ_FP16>(p, (int)max_tiles, st);
+    else launch_grouped_cfg<KIND_FP8_BLOCK, 128, 128, 2, 2, SGLQ_FP16>(p, (int)max_tiles, st);
+  }
+  return finish(name);
 }
 
 extern "C" int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,

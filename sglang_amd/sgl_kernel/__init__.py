@@ -1,5 +1,5 @@
 """Stand-in for the part of the reference's ``sgl_kernel`` package that serves the
-W8A8 quantized-linear path (sgl-kernel/python/sgl_kernel/__init__.py)."""
+W8A8 quantized-linear path and its grouped (MoE) GEMM (sgl-kernel/python/sgl_kernel/__init__.py)."""
 
 from .gemm import (
     fp8_blockwise_scaled_mm,
@@ -11,8 +11,10 @@ from .gemm import (
     sgl_per_tensor_quant_fp8,
     sgl_per_token_quant_fp8,
 )
+from .moe import fp8_blockwise_scaled_grouped_mm
 
 __all__ = [
+    "fp8_blockwise_scaled_grouped_mm",
     "fp8_blockwise_scaled_mm",
     "fp8_scaled_mm",
     "int8_mm_i32",

@@ -69,3 +69,41 @@ def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
         idx = bad.nonzero()[:5].tolist()
         raise AssertionError(f"{what}: {nbad} of {got.numel()} elements differ, first at {idx}: "
                              f"got {[got[tuple(i)].item() for i in idx]} want {[want[tuple(i)].item() for i in idx]}")
+
+
+FP8 = torch.float8_e4m3fn
+
+
+def moe_case(num_experts, rows_per_expert, n, k, seed, dtype=torch.bfloat16):
+    """Inputs built the way the reference's grouped-GEMM test builds them
+    (sgl-kernel/tests/test_fp8_blockwise_moe.py:39-63,119-190): N(0,1) activations quantized per
+    token and 128 columns with amax clamped at 1e-4, N(0,1) weights quantized per 128 x 128 block,
+    experts' rows stacked, K-major activation scales, [E, K/128, N/128] weight scales."""
+    g = torch.Generator().manual_seed(seed)
+    offsets, sizes, a_orig, b_orig, aq, asc, bq, bsc = [0], [], [], [], [], [], [], []
+    for m_g in rows_per_expert:
+        offsets.append(offsets[-1] + m_g)
+        sizes.append([m_g, n, k])
+        a = torch.randn((m_g, k), generator=g).to(dtype)
+        b = torch.randn((n, k), generator=g).to(dtype)
+        av = a.float().view(m_g, k // 128, 128)
+        amax = av.abs().amax(dim=2).clamp(1e-4)
+        aq.append((av * (448.0 / amax.unsqueeze(2))).to(FP8).view(m_g, k))
+        asc.append(amax / 448.0)
+        bv = b.float().view(n // 128, 128, k // 128, 128)
+        bmax = bv.abs().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+        bq.append((bv * (448.0 / bmax)).to(FP8).view(n, k))
+        bsc.append((bmax / 448.0).view(n // 128, k // 128).t().contiguous())  # [K/128, N/128]
+        a_orig.append(a)
+        b_orig.append(b)
+    return dict(
+        a=torch.cat(aq) if aq else torch.empty((0, k), dtype=FP8), b=torch.stack(bq).transpose(1, 2),
+        scales_a=torch.cat(asc), scales_b=torch.stack(bsc),
+        problem_sizes=torch.tensor(sizes, dtype=torch.int32), expert_offsets=torch.tensor(offsets[:-1], dtype=torch.int32),
+        a_orig=a_orig, b_orig=b_orig)
+
+
+def calc_diff(x, y):
+    # the reference test's criterion (sgl-kernel/tests/test_fp8_blockwise_moe.py:29-33)
+    x, y = x.double(), y.double()
+    return float(1 - 2 * (x * y).sum() / (x * x + y * y).sum())

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from helpers import (assert_bits_equal, c_group_quant_fp8, c_tensor_quant_fp8, c_token_quant_fp8, c_token_quant_int8,
-                     fp8_bits)
+                     calc_diff, fp8_bits, moe_case)
 from oracle import w8a8_oracle as O
 
 FP8 = torch.float8_e4m3fn
@@ -316,6 +316,40 @@ def test_blockwise_mm_vs_c_double_brute_force(c_oracle):
     deq_a = a.double() * sa.double().repeat_interleave(128, dim=1)
     deq_w = w.double() * sbw.double().repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)
     torch.testing.assert_close(out.double(), deq_a @ deq_w.t(), rtol=1e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.half, torch.bfloat16])
+def test_grouped_mm_oracle_vs_reference_test_baseline(out_dtype):
+    """The reference accepts its grouped GEMM when, per expert, 1 - cosine-like similarity with
+    torch.mm of the unquantized operands is below 0.001 (test_fp8_blockwise_moe.py:247-251)."""
+    rows = [16, 64, 0, 48, 112, 16, 32, 80]
+    c = moe_case(len(rows), rows, n=256, k=512, seed=21, dtype=out_dtype)
+    out = O.fp8_blockwise_scaled_grouped_mm(c["a"], c["b"], c["scales_a"], c["scales_b"], c["problem_sizes"],
+                                            c["expert_offsets"], out_dtype)
+    first = 0
+    for e, m_g in enumerate(rows):
+        if m_g:
+            baseline = torch.mm(c["a_orig"][e].float(), c["b_orig"][e].float().t())
+            assert calc_diff(out[first:first + m_g], baseline) < 0.001
+        first += m_g
+
+
+def test_grouped_mm_oracle_reduces_to_dense_and_leaves_gaps():
+    # one expert: the dense operator; experts in any order, with rows between them that belong to nobody
+    c = moe_case(1, [40], n=128, k=256, seed=3)
+    dense = O.fp8_blockwise_scaled_mm(c["a"], c["b"][0], c["scales_a"], c["scales_b"][0], torch.bfloat16)
+    out = O.fp8_blockwise_scaled_grouped_mm(c["a"], c["b"], c["scales_a"], c["scales_b"], c["problem_sizes"],
+                                            c["expert_offsets"], torch.bfloat16)
+    assert torch.equal(out, dense)
+    c = moe_case(3, [16, 16, 16], n=128, k=128, seed=4)
+    sizes = torch.tensor([[8, 128, 128], [16, 128, 128], [5, 128, 128]], dtype=torch.int32)
+    offsets = torch.tensor([32, 0, 20], dtype=torch.int32)  # expert 0 -> rows 32..39, 1 -> 0..15, 2 -> 20..24
+    out = O.fp8_blockwise_scaled_grouped_mm(c["a"], c["b"], c["scales_a"], c["scales_b"], sizes, offsets, torch.bfloat16)
+    for e, (first, m_g) in enumerate([(32, 8), (0, 16), (20, 5)]):
+        sl = slice(first, first + m_g)
+        want = O.fp8_blockwise_scaled_mm(c["a"][sl], c["b"][e], c["scales_a"][sl], c["scales_b"][e], torch.bfloat16)
+        assert torch.equal(out[sl], want)
+    assert float(out[16:20].abs().max()) == 0.0 and float(out[25:32].abs().max()) == 0.0 and float(out[40:].abs().max()) == 0.0
 
 
 def test_block_int8_mm_pins(c_oracle):
