@@ -400,6 +400,35 @@ def run_sweep(args):
             fl_tot += 2.0 * m * n * k
             torch.cuda.empty_cache()
         emit(cfg=4, op="total", M=m, total_us=round(tot * 1e3, 1), TFLOPs=round(fl_tot / tot / 1e9, 2))
+    # grouped (MoE) block-FP8 GEMM, DeepSeek-V3 expert shapes: 256 experts (one GPU holding all of them) and
+    # 32 (an 8-way expert-parallel share), equal groups of `rows` routed rows; every expert's weight is read once
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_grouped_mm
+
+    for e in (32, 256):
+        for (n, k) in ((4096, 7168), (7168, 2048)):
+            g = torch.Generator(device=dev).manual_seed(5000 + e)
+            b = (torch.randn((e, n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
+            sb = torch.rand((e, k // 128, n // 128), generator=g, device=dev) * 1e-3 + 1e-4
+            for rows in (2, 32, 128, 256):
+                total = e * rows
+                a = torch.randn((total, k), generator=g, device=dev).to(torch.float8_e4m3fn)
+                sa = torch.rand((total, k // 128), generator=g, device=dev) * 1e-2 + 1e-3
+                ps = torch.tensor([[rows, n, k]] * e, dtype=torch.int32, device=dev)
+                eo = torch.arange(e, dtype=torch.int32, device=dev) * rows
+                out = torch.empty((total, n), dtype=torch.bfloat16, device=dev)
+                i64 = torch.empty((e,), dtype=torch.int64, device=dev)
+                lay = torch.zeros((e, 5), dtype=torch.int32, device=dev)
+                ws = torch.empty((1 << 20,), dtype=torch.uint8, device=dev)
+                tg = time_kernel(lambda j: fp8_blockwise_scaled_grouped_mm(out, i64, i64, i64, i64, i64, a, b.transpose(1, 2), sa, sb,
+                                                                           i64, i64, i64, lay, lay, ps, eo, ws), max(2, args.iters // 4))
+                fl = 2.0 * total * n * k
+                nbytes = e * n * k + total * k + 2 * total * n + 4 * total * (k // 128) + 4 * e * (k // 128) * (n // 128)
+                emit(cfg="moe", op="fp8_blockwise_scaled_grouped_mm", experts=e, rows_per_expert=rows, N=n, K=k,
+                     kernel=_lib.load().sglq_debug_last_gemm_kernel().decode(), gemm_us=round(tg * 1e3, 1),
+                     gemm_TFLOPs=round(fl / tg / 1e9, 2), gemm_frac_mfma=round(fl / tg / 1e9 / PEAK_FP8_TFLOPS, 4),
+                     gemm_GBs=round(nbytes / tg / 1e6, 1), gemm_frac_hbm=round(nbytes / tg / 1e6 / PEAK_HBM_GBS, 4))
+            del b
+            torch.cuda.empty_cache()
     f.close()
 
 

@@ -71,6 +71,8 @@ def load() -> ctypes.CDLL:
     lib.sglq_debug_force_tile.restype = None
     lib.sglq_debug_force_splits.argtypes = [c_int]
     lib.sglq_debug_force_splits.restype = None
+    lib.sglq_debug_grouped_tile.argtypes = [c_int]
+    lib.sglq_debug_grouped_tile.restype = None
     lib.sglq_debug_last_gemm_kernel.argtypes = []
     lib.sglq_debug_last_gemm_kernel.restype = ctypes.c_char_p
     _lib = lib

@@ -54,6 +54,7 @@ struct GemmArgs {
   void* ws;        // split-K partial sums [splits][M][N], fp32 or int32; grouped GEMM: the tile plan
   int splits;
   int64_t b_expert_stride, sb_expert_stride;  // grouped GEMM: bytes / floats between experts' weights / weight scales
+  int num_experts;
 };
 
 // Grouped GEMM tile plan in the workspace (int32): [0] = number of row tiles, then from [4] on
@@ -886,8 +887,9 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------
 // MODE selects one of three variants, each launched only where it is needed so that the
 // plain one keeps its register allocation: 0 = whole tiles, 1 = split-K work units (raw
-// partial sums to the workspace), 2 = whole tiles of a block-scaled kind with a bias.
-constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2;
+// partial sums to the workspace), 2 = whole tiles of a block-scaled kind with a bias,
+// 3 = grouped GEMM (row tiles and their experts from the plan in the workspace).
+constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2, PIPE_GROUPED = 3;
 template <int KIND, int OUT_DT, int MODE>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
@@ -928,10 +930,20 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
                                              off + (uint32_t)j * step_a, k0, 0, 0);
   };
-  auto copy_b = [&](int j, int stage, int k0, uint32_t off) {
+  // Grouped mode: every tile has its expert's weight; b_cur / b_two are the weights of the
+  // tiles of the block after the current one and of the block two after it (like off_b / off_b2).
+  const char* b_cur = p.b;
+  const char* b_two = p.b;
+  auto copy_b = [&](int j, int stage, int k0, uint32_t off, bool two_ahead) {
     char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16,
-                                             off + (uint32_t)j * step_b, k0, 0, 0);
+    if constexpr (MODE == PIPE_GROUPED) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(two_ahead ? b_two : b_cur, p.b_bytes),
+                                               (__attribute__((address_space(3))) void*)dst, 16, off + (uint32_t)j * step_b, k0,
+                                               0, 0);
+    } else {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16,
+                                               off + (uint32_t)j * step_b, k0, 0, 0);
+    }
   };
   auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
   auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
@@ -972,11 +984,12 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   if constexpr (BLOCK) {
     const int nblocks = (p.N + 127) >> 7;
     const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb_all - 1) * p.sa_stride_k + 1;
-    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb_all - 1) * p.sb_stride_k + 1;
+    int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb_all - 1) * p.sb_stride_k + 1;
+    if constexpr (MODE == PIPE_GROUPED) sfb_elems += (int64_t)(p.num_experts - 1) * p.sb_expert_stride;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
   }
-  auto scale_offset = [&](int m0, int n0) -> uint32_t {
+  auto scale_offset = [&](int m0, int n0, int expert) -> uint32_t {
     if (wave < 4) {
       const int row = m0 + wave * 64 + lane;
       return row < p.M ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
@@ -984,7 +997,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     const int nblocks = (p.N + 127) >> 7;
     int nb = (n0 >> 7) + lane;
     if (nb >= nblocks) nb = nblocks - 1;
-    return (wave == 4 && lane < 2) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
+    return (wave == 4 && lane < 2) ? (uint32_t)((nb * p.sb_stride_n + expert * p.sb_expert_stride) * 4) : OOB;
   };
   auto copy_scales = [&](int buf, int kb, uint32_t voff) {
     char* dst = smem + buf * SCALE_BYTES + sc_dst;
@@ -1067,12 +1080,12 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           }
         }
         if constexpr (first) {
-          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b);
+          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b, false);
           if (idx >= 8 && idx < 12) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
           if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
-          if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2);
+          if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2, true);
         } else if constexpr (!last) {
-          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2);
+          if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2, true);
         }
         if constexpr (BLOCK) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
@@ -1100,29 +1113,43 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // ---- persistent walk over the work units blockIdx, blockIdx + gridDim, ...  A unit is an
   // output tile, or with split-K (p.splits > 1) one of a tile's p.splits contiguous K ranges,
   // whose raw partial sums go to the workspace for splitk_reduce_kernel.
-  const int tiles = p.tiles_m * p.tiles_n;
+  // Grouped mode: the row tiles come from the plan in the workspace (their number is device
+  // data); a tile's rows end where its expert's rows end.
+  const int* plan = static_cast<const int*>(p.ws);
+  const int tiles_m = MODE == PIPE_GROUPED ? plan[0] : p.tiles_m;
+  const int tiles = tiles_m * p.tiles_n;
   const int total = tiles * splits;
   const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-  auto unit_origin = [&](int u, int& um0, int& un0, int& ukb0) {
+  auto unit_origin = [&](int u, int& um0, int& un0, int& ukb0, int& uexpert, int& um_end) {
     const int split = MODE == PIPE_SPLITK ? u / tiles : 0;
     int tm, tn;
-    tile_of_block(u - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
+    tile_of_block(u - split * tiles, tiles_m, p.tiles_n, tm, tn);
     um0 = tm * BM;
     un0 = tn * BN;
     ukb0 = split * nkb;
+    uexpert = 0;
+    um_end = p.M;
+    if constexpr (MODE == PIPE_GROUPED) {
+      const int* entry = plan + PLAN_HEADER + PLAN_ENTRY * tm;
+      uexpert = entry[0];
+      um0 = entry[1];
+      um_end = entry[2];
+    }
   };
   int unit = blockIdx.x;
-  int m0, n0, kb0;
-  unit_origin(unit, m0, n0, kb0);
+  if (MODE == PIPE_GROUPED && unit >= total) return;  // the grid is sized for the largest possible plan
+  int m0, n0, kb0, expert, m_end;
+  unit_origin(unit, m0, n0, kb0, expert, m_end);
   int par = 0;  // stage that holds the unit's first K block
 
   off_a = off_a2 = a_offset(m0);
   off_b = off_b2 = b_offset(n0);
-  if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0);
+  if constexpr (MODE == PIPE_GROUPED) b_cur = b_two = p.b + (int64_t)expert * p.b_expert_stride;
+  if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0, expert);
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_a(j, 0, kb0 * 128, off_a);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_b(j, 0, kb0 * 128, off_b);
+  for (int j = 0; j < 4; ++j) copy_b(j, 0, kb0 * 128, off_b, false);
   if constexpr (BLOCK) copy_scales(0, kb0, sc_voff);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
@@ -1145,23 +1172,26 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     // and N, which the buffer bounds turn into zero fill without memory traffic.
     const int next_unit = unit + (int)gridDim.x;
     const bool has_next = next_unit < total;
-    int nm0, nn0, nkb0;
-    unit_origin(has_next ? next_unit : 0, nm0, nn0, nkb0);
+    int nm0, nn0, nkb0, nexpert, nm_end;
+    unit_origin(has_next ? next_unit : 0, nm0, nn0, nkb0, nexpert, nm_end);
     if (!has_next) {
-      nm0 = p.tiles_m * BM;
+      nm0 = MODE == PIPE_GROUPED ? p.M : p.tiles_m * BM;
       nn0 = p.tiles_n * BN;
     }
+    const char* b_next = p.b;
+    if constexpr (MODE == PIPE_GROUPED) b_next = p.b + (int64_t)nexpert * p.b_expert_stride;
 
     // (a unit has at least three K blocks, so its first, last-but-one and last step are distinct)
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
     uint32_t sc_voff_next = OOB;
-    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
+    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0, nexpert);
     k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{});
     for (int kb = 1; kb + 1 < nkb; ++kb) {
       const bool pen = kb + 2 == nkb;  // the block two ahead is the next unit's first
       off_a2 = pen ? off_a_next : off_a2;
       off_b2 = pen ? off_b_next : off_b2;
       sc_voff2 = pen ? sc_voff_next : sc_voff2;
+      if constexpr (MODE == PIPE_GROUPED) b_two = pen ? b_next : b_two;
       k_step((kb + par) & 1, kb0 + kb + 1, pen ? nkb0 : kb0 + kb + 2, std::false_type{}, std::false_type{});
     }
     // last K block: its copies (the next unit's second block) wait for the next unit's first step
@@ -1170,6 +1200,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     off_a = off_a2;
     off_b = off_b2;
     sc_voff = sc_voff2;
+    if constexpr (MODE == PIPE_GROUPED) b_cur = b_two;
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
@@ -1177,6 +1208,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       store_partials_bounded<MI, NI>(p, acc, unit / tiles, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+    } else if constexpr (MODE == PIPE_GROUPED) {
+      GemmArgs q = p;
+      q.M = m_end;  // rows past the expert's last one belong to other experts
+      if (aligned_out)
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, false>(q, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
+                                                          wave);
+      else
+        epilogue<KIND, OUT_DT, MI, NI, 0>(q, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
@@ -1190,6 +1229,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     m0 = nm0;
     n0 = nn0;
     kb0 = nkb0;
+    expert = nexpert;
+    m_end = nm_end;
     par = last_stage ^ 1;
   }
 }
@@ -1867,6 +1908,7 @@ static int num_cus() {
 }
 
 static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
+static int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile (0 = from the average group)
 static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
 
 template <int KIND, int OUT_DT>
@@ -2219,6 +2261,7 @@ using namespace sglq;
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
+extern "C" void sglq_debug_grouped_tile(int rows) { g_grouped_tile = (rows == 32 || rows == 64 || rows == 128 || rows == 256) ? rows : 0; }
 extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel; }
 
 template <int KIND>
@@ -2306,9 +2349,19 @@ extern "C" int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, 
     set_error("%s: the experts' weights must be 16-byte aligned, fewer than 2^20 experts", name);
     return SGLQ_EINVAL;
   }
-  // row tile height from the average group: the experts' row counts are device data
+  // Row tile height from the average group: the experts' row counts are device data.
+  // Measured with 256 experts of 4096 x 7168 (one launch streams every expert's weight once,
+  // 7.5 GB): 64-row tiles are fastest below about 12 rows per expert (1.27-1.31 ms, 5.7-5.9
+  // TB/s), 128-row tiles up to about 64 (1.47-2.19 ms), and from there the pipelined 256-row
+  // kernel even with its tiles partly empty (2.2-2.3 ms whatever the fill, against 3.0 ms for
+  // 128-row tiles at 96 rows per expert).
   const int64_t avg = total_m / num_experts;
-  const int bm = avg <= 32 ? 32 : avg <= 64 ? 64 : 128;
+  const bool pipelined = g_grouped_tile == 256 || (g_grouped_tile == 0 && avg >= 64 && K >= 384);
+  const int bm = g_grouped_tile ? g_grouped_tile : pipelined ? 256 : avg < 12 ? 64 : 128;
+  if (g_grouped_tile == 256 && K < 384) {
+    set_error("%s: the 256-row kernel needs K >= 384", name);
+    return SGLQ_EINVAL;
+  }
   const int64_t max_tiles = total_m / bm + num_experts;
   const int64_t need = (int64_t)(PLAN_HEADER + PLAN_ENTRY * max_tiles) * 4;
   if (!workspace || workspace_bytes < need) {
@@ -2330,10 +2383,22 @@ extern "C" int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, 
   p.sb_stride_n = sfb_stride_n;
   p.b_expert_stride = b_expert_stride;
   p.sb_expert_stride = sfb_expert_stride;
+  p.num_experts = (int)num_experts;
   p.ws = workspace;
   hipStream_t st = static_cast<hipStream_t>(stream);
   grouped_plan_kernel<<<dim3(1), dim3(256), 0, st>>>(problem_sizes, expert_offsets, (int)num_experts, (int)total_m, bm,
                                                      (int)max_tiles, static_cast<int*>(workspace));
+  if (bm == 256) {
+    g_last_kernel = "grouped_plan_kernel+gemm_pipe_kernel<grouped>";
+    p.tiles_m = (int)max_tiles;
+    p.tiles_n = (int)((N + 255) / 256);
+    p.splits = 1;
+    const int64_t units = max_tiles * p.tiles_n;
+    const dim3 grid((uint32_t)(units < num_cus() ? units : num_cus())), block(512);
+    if (out_dtype == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_BF16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
+    else gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_FP16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
+    return finish(name);
+  }
   g_last_kernel = "grouped_plan_kernel+gemm_kernel<grouped>";
   if (out_dtype == SGLQ_BF16) {
     if (bm == 32) launch_grouped_cfg<KIND_FP8_BLOCK, 32, 128, 1, 4, SGLQ_BF16>(p, (int)max_tiles, st);

@@ -17,6 +17,16 @@ def say(*a):
     print(*a, flush=True)
 
 
+# the row tile: chosen from the average group, the 128-row kernel's tiles, the pipelined 256-row kernel
+@pytest.fixture(params=[0, 32, 64, 128, 256], ids=["rows_auto", "rows32", "rows64", "rows128", "rows256"])
+def gtile(request):
+    from sglang_amd import _lib
+
+    _lib.load().sglq_debug_grouped_tile(request.param)
+    yield request.param
+    _lib.load().sglq_debug_grouped_tile(0)
+
+
 def run_grouped(gpu, c, out_dtype, problem_sizes=None, expert_offsets=None, scales_b=None):
     """Calls the operator with the reference's argument list (scratch tensors included); the
     output starts filled with a sentinel so that untouched rows can be told apart."""
@@ -54,7 +64,7 @@ def check_against_oracle(c, out, rows_per_expert, out_dtype, cap=24):
 
 @pytest.mark.parametrize("out_dtype", [torch.half, torch.bfloat16])
 @pytest.mark.parametrize("num_experts", [8, 16])
-def test_grouped_mm_reference_test_grid(gpu, num_experts, out_dtype):
+def test_grouped_mm_reference_test_grid(gpu, gtile, num_experts, out_dtype):
     """The reference's test (sgl-kernel/tests/test_fp8_blockwise_moe.py:109-251): 8 or 16 experts
     with 16 .. 1024 rows each in steps of 16, N and K multiples of 2048; its acceptance
     criterion per expert, and the oracle on sampled rows."""
@@ -63,7 +73,7 @@ def test_grouped_mm_reference_test_grid(gpu, num_experts, out_dtype):
     rnd = random.Random(num_experts)
     rows = [16 * rnd.randint(1, 64) for _ in range(num_experts)]
     n, k = 2048 * rnd.randint(1, 2), 2048 * rnd.randint(1, 2)
-    say("grouped mm, reference grid", num_experts, out_dtype, rows, n, k)
+    say("grouped mm, reference grid", num_experts, out_dtype, rows, n, k, "row tile", gtile)
     c = moe_case(num_experts, rows, n, k, seed=num_experts, dtype=out_dtype)
     out = run_grouped(gpu, c, out_dtype).cpu()
     assert out.dtype == out_dtype
@@ -79,17 +89,17 @@ def test_grouped_mm_reference_test_grid(gpu, num_experts, out_dtype):
                                   [1, 2, 0, 17, 31, 5, 32, 33],              # average 15: 32-row tiles
                                   [300, 0, 1, 257, 128, 127]],               # average 135: 128-row tiles
                          ids=["tiles64", "tiles32", "tiles128"])
-def test_grouped_mm_ragged_groups(gpu, rows):
+def test_grouped_mm_ragged_groups(gpu, gtile, rows):
     """Groups of any size, empty ones included: a tile that straddles two experts must not
     write the other expert's rows; N not a multiple of 128."""
-    say("grouped mm, ragged", rows)
+    say("grouped mm, ragged", rows, "row tile", gtile)
     c = moe_case(len(rows), rows, n=384, k=640, seed=len(rows))
     out = run_grouped(gpu, c, torch.bfloat16).cpu()
     check_against_oracle(c, out, rows, torch.bfloat16, cap=1 << 30)
     assert not bool((out == SENTINEL).any())
 
 
-def test_grouped_mm_gaps_order_and_scale_strides(gpu):
+def test_grouped_mm_gaps_order_and_scale_strides(gpu, gtile):
     """Experts in any order with unowned rows between them (left untouched); weight scales
     passed as a transposed view (the reference's [E, N/128, K/128] storage)."""
     c = moe_case(3, [64, 64, 64], n=256, k=384, seed=5)
@@ -107,10 +117,11 @@ def test_grouped_mm_gaps_order_and_scale_strides(gpu):
     assert bool((out[~owned] == SENTINEL).all())
 
 
-def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu):
+@pytest.mark.parametrize("rows_per_tile", [128, 256])
+def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu, rows_per_tile):
     """DeepSeek-V3-shaped expert GEMM (N = 4096, K = 7168, 32 experts, 8192 routed rows): every
-    expert's rows equal the dense operator's result on that expert with the same 128 x 128
-    tiles and no split-K, bit for bit (same kernel, same summation order)."""
+    expert's rows equal the dense operator's result on that expert with the same kernel (the
+    128 x 128 one, the pipelined 256 x 256 one) and no split-K, bit for bit (same summation order)."""
     from sglang_amd import _lib
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
@@ -128,10 +139,15 @@ def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu):
     c = dict(a=a, b=b.transpose(1, 2), scales_a=sa, scales_b=sb,
              problem_sizes=torch.tensor([[r, n, k] for r in rows], dtype=torch.int32),
              expert_offsets=cuts[:-1].to(torch.int32))
-    out = run_grouped(gpu, c, torch.bfloat16)
     lib = _lib.load()
-    assert lib.sglq_debug_last_gemm_kernel().decode() == "grouped_plan_kernel+gemm_kernel<grouped>"
-    lib.sglq_debug_force_tile(128)
+    lib.sglq_debug_grouped_tile(rows_per_tile)
+    try:
+        out = run_grouped(gpu, c, torch.bfloat16)
+    finally:
+        lib.sglq_debug_grouped_tile(0)
+    want_kernel = "grouped_plan_kernel+gemm_kernel<grouped>" if rows_per_tile == 128 else "grouped_plan_kernel+gemm_pipe_kernel<grouped>"
+    assert lib.sglq_debug_last_gemm_kernel().decode() == want_kernel
+    lib.sglq_debug_force_tile(128 if rows_per_tile == 128 else 258)
     lib.sglq_debug_force_splits(1)
     try:
         for x in (0, 5, 17, 31):
@@ -140,6 +156,7 @@ def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu):
             sl = slice(int(cuts[x]), int(cuts[x + 1]))
             sa_cm = sa[sl].t().contiguous().t()  # the dense operator takes M-major activation scales
             dense = fp8_blockwise_scaled_mm(a[sl], b[x].t(), sa_cm, sb[x].t().contiguous().t(), torch.bfloat16)  # K-major weight scales
+            assert lib.sglq_debug_last_gemm_kernel().decode() == ("gemm_kernel" if rows_per_tile == 128 else "gemm_pipe_kernel")
             assert torch.equal(out[sl].view(torch.int16), dense.view(torch.int16)), x
     finally:
         lib.sglq_debug_force_tile(0)
