@@ -344,8 +344,14 @@ def run_sweep(args):
              gemm_frac_hbm=round(block_gemm_bytes(m, n, k) / tg / 1e6 / PEAK_HBM_GBS, 4))
         return tq, tg
 
+    only = None if not args.sweep_only else set(args.sweep_only.split(","))
+
+    def want(cfg):
+        return only is None or str(cfg) in only
+
     # cfg 0
-    block_case(0, "cfg0", 256, 2048, 7168, 0)
+    if want(0):
+        block_case(0, "cfg0", 256, 2048, 7168, 0)
     # cfg 1
     g = torch.Generator(device=dev).manual_seed(1000)
     n, k = 14336, 4096
@@ -353,7 +359,7 @@ def run_sweep(args):
     s_b = torch.rand((n,), generator=g, device=dev) * 9e-3 + 1e-3
     bias = (torch.randn((n,), generator=g, device=dev) * 0.1).to(torch.bfloat16)
     w8s = [w8] + [w8.clone() for _ in range(7)]
-    for m in (1, 16, 128, 1024):
+    for m in (1, 16, 128, 1024) if want(1) else ():
         x = make_activation(m, k, 1000 + m, dev)
         tq = time_kernel(lambda j: per_token_quant_int8(x), args.iters)
         xq, xs = per_token_quant_int8(x)
@@ -366,11 +372,11 @@ def run_sweep(args):
              gemm_frac_hbm=round(rowcol_gemm_bytes(m, n, k, True) / tg / 1e6 / PEAK_HBM_GBS, 4))
     del w8s
     # cfg 2
-    for i, (n, k) in enumerate(DSV3_NK):
+    for i, (n, k) in enumerate(DSV3_NK if want(2) else ()):
         for m in (1, 8, 64, 512, 4096, 8192):
             block_case(2, "dsv3", m, n, k, 2000 + i)
     # cfg 3
-    for i, (n, k) in enumerate(LLAMA8B_NK):
+    for i, (n, k) in enumerate(LLAMA8B_NK if want(3) else ()):
         g = torch.Generator(device=dev).manual_seed(3000 + i)
         w = torch.randn((n, k), generator=g, device=dev) * 0.02
         sc = w.abs().amax() / 448.0
@@ -391,7 +397,7 @@ def run_sweep(args):
                  gemm_frac_hbm=round(rowcol_gemm_bytes(m, n, k) / tg / 1e6 / PEAK_HBM_GBS, 4))
         del wqs
     # cfg 4
-    for m in (4096, 64):
+    for m in (4096, 64) if want(4) else ():
         tot = 0.0
         fl_tot = 0.0
         for i, (name, n, k) in enumerate(LLAMA70B_NK):
@@ -404,7 +410,7 @@ def run_sweep(args):
     # 32 (an 8-way expert-parallel share), equal groups of `rows` routed rows; every expert's weight is read once
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_grouped_mm
 
-    for e in (32, 256):
+    for e in (32, 256) if want("moe") else ():
         for (n, k) in ((4096, 7168), (7168, 2048)):
             g = torch.Generator(device=dev).manual_seed(5000 + e)
             b = (torch.randn((e, n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
@@ -443,6 +449,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--sweep-only", type=str, default=None,
+                    help="with --sweep: comma-separated configurations to run (0, 1, 2, 3, 4, moe); default all")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is measured on one GPU only (it needs no exchange between GPUs; "
