@@ -57,3 +57,54 @@ def test_graph_replay_matches_eager(gpu, m):
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"replay {rep}, output {i} differs from eager"
+
+
+@pytest.mark.parametrize("rows_per_expert", [3, 40, 200])
+def test_graph_replay_grouped_mm(gpu, rows_per_expert):
+    """The grouped GEMM reads the experts' row counts on the device: a captured launch follows
+    new routing (other problem_sizes / expert_offsets contents) on every replay."""
+    from helpers import moe_case
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_grouped_mm
+
+    print("graph replay, grouped", rows_per_expert, flush=True)
+    e, n, k = 6, 512, 1024
+    total = e * rows_per_expert
+    c = moe_case(e, [rows_per_expert] * e, n, k, seed=rows_per_expert)
+    a, b = c["a"].to(gpu), c["b"].transpose(1, 2).contiguous().to(gpu).transpose(1, 2)
+    sa, sb = c["scales_a"].to(gpu), c["scales_b"].to(gpu)
+    ps, eo = c["problem_sizes"].to(gpu), c["expert_offsets"].to(gpu)
+    out = torch.zeros((total, n), dtype=torch.bfloat16, device=gpu)
+    i64 = torch.empty((e,), dtype=torch.int64, device=gpu)
+    lay = torch.zeros((e, 5), dtype=torch.int32, device=gpu)
+    ws = torch.empty((1 << 16,), dtype=torch.uint8, device=gpu)
+
+    def run(dst):
+        fp8_blockwise_scaled_grouped_mm(dst, i64, i64, i64, i64, i64, a, b, sa, sb, i64, i64, i64, lay, lay, ps, eo, ws)
+
+    run(out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(out)
+    g = torch.Generator().manual_seed(1)
+    for rep in range(3):
+        # new routing with the same total: random cuts of the rows
+        cuts = torch.cat([torch.zeros(1, dtype=torch.long), torch.sort(torch.randint(0, total + 1, (e - 1,), generator=g)).values,
+                          torch.tensor([total])])
+        ps.copy_(torch.stack([cuts[1:] - cuts[:-1], torch.full((e,), n), torch.full((e,), k)], dim=1).to(torch.int32))
+        eo.copy_(cuts[:-1].to(torch.int32))
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = torch.zeros_like(out)
+        run(want)  # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"replay {rep} differs from eager"
+        first = int(cuts[2])
+        rows = int(cuts[3] - cuts[2])
+        if rows:
+            ref = O.fp8_blockwise_scaled_mm(c["a"][first:first + rows], c["b"][2], c["scales_a"][first:first + rows], c["scales_b"][2],
+                                            torch.float32, acc_dtype=torch.float64)
+            torch.testing.assert_close(got[first:first + rows].cpu().float(), ref, rtol=1e-2, atol=1e-2)
