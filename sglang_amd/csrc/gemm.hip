@@ -1573,7 +1573,9 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 // flight per CU).  All copies of a stage are vector-memory loads that retire in
 // order, so "stage t has landed" is a vmcnt wait that leaves the younger stages'
 // loads outstanding.  With splits > 1 the partial sums go to a workspace and
-// splitk_reduce_kernel applies the epilogue.
+// splitk_reduce_kernel applies the epilogue.  For 64 < M <= 512 the grid has a second
+// dimension of 64-row tiles (blockIdx.y): the tiles of one weight tile run side by side, so
+// the weights still come from HBM once and from the caches after that.
 // ---------------------------------------------------------------------------
 template <int KIND, int MI, int OUT_DT>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
@@ -1597,6 +1599,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 
   const int tile_n = blockIdx.x % p.tiles_n, split = blockIdx.x / p.tiles_n;
   const int n0 = tile_n * BN;
+  const int m_base = (int)blockIdx.y * 64;
   const int nkb = p.K >> 7;
   // Split s takes the K blocks s, s + splits, s + 2 splits, ...: the blocks that share a
   // weight tile then read neighbouring 128-byte pieces of the same rows at about the same
@@ -1612,14 +1615,14 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   // group, chunk (l % 8) ^ swz(row); copies of one wave differ by 32 rows.
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
   const uint32_t off_w = (uint32_t)(n0 + wave * 8 + l8) * p.ldb + c16;
-  const uint32_t off_a = (uint32_t)(wave * 8 + l8) * p.lda + c16;
+  const uint32_t off_a = (uint32_t)(m_base + wave * 8 + l8) * p.lda + c16;
   const uint32_t step_w = 32u * p.ldb, step_a = 32u * p.lda;
   uint32_t off_s = 0;
   int sfa_step = 0;
   if constexpr (BLOCK) {
     const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
     rs = make_rsrc_sgpr(p.sa, (uint32_t)(sfa_elems * 4));
-    off_s = lane < p.M ? (uint32_t)(lane * p.sa_stride_m * 4) : OOB;  // lane = activation row
+    off_s = m_base + lane < p.M ? (uint32_t)((m_base + lane) * p.sa_stride_m * 4) : OOB;  // lane = activation row of the tile
     sfa_step = (int)(p.sa_stride_k * 4);
     const int nblocks = (p.N + 127) >> 7;
     const int nb = tile_n < nblocks ? tile_n : nblocks - 1;
@@ -1703,8 +1706,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
     }
   }
 
-  if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, 0, n0 + wave * 32, r16, g);
-  else store_partials<MI, NI>(p, acc, split, 0, n0 + wave * 32, r16, g);
+  if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, m_base, n0 + wave * 32, r16, g);
+  else store_partials<MI, NI>(p, acc, split, m_base, n0 + wave * 32, r16, g);
 }
 
 // ---------------------------------------------------------------------------
@@ -2101,19 +2104,19 @@ static void launch_reduce(GemmArgs& p, hipStream_t st) {
 template <int KIND, int MI, int OUT_DT>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
   g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
-  gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits)), dim3(256), 0, st>>>(p);
+  gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits), (uint32_t)p.tiles_m), dim3(256), 0, st>>>(p);
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
 // Decode path: choose the split-K factor so that every CU streams weights.
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
-  p.tiles_m = 1;
+  p.tiles_m = (p.M + 63) / 64;
   p.tiles_n = (p.N + 127) / 128;
   const int nkb = p.K >> 7;
   // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
   // more blocks only add partial-sum traffic.
-  int splits = 256 / p.tiles_n;
+  int splits = 256 / (p.tiles_n * p.tiles_m);
   const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
   if (splits > by_steps) splits = by_steps;
   if (splits < 1) splits = 1;
@@ -2125,7 +2128,7 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.splits = splits;
   if (p.M <= 16) launch_skinny_mi<KIND, 1, OUT_DT>(p, st);
   else if (p.M <= 32) launch_skinny_mi<KIND, 2, OUT_DT>(p, st);
-  else launch_skinny_mi<KIND, 4, OUT_DT>(p, st);
+  else launch_skinny_mi<KIND, 4, OUT_DT>(p, st);  // (64-row tiles for any M > 32)
 }
 
 // Decode path without split-K: blocks of 16 or 32 weight rows over the whole of K.
@@ -2165,7 +2168,11 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (g_force_tile == 0 || g_force_tile == 16 || g_force_tile == 32) &&
       launch_stream<KIND, OUT_DT>(p, st))
     return;
-  if ((p.K & 127) == 0 && p.M <= 64 && p.K <= 1024 * 128 && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
+  // ... and up to 128 rows (two 64-row tiles side by side) with K <= 8192 it still beats the
+  // 128 x 128 kernel (measured, e.g. 128 x 24576 x 1536: 28.3 -> 16.3 us, 128 x 4096 x 7168:
+  // 21.2 -> 17.9 us; at K = 16384 the 128 x 128 kernel wins, 35 against 49 us).
+  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192) || (g_force_tile == 64 && p.M <= 512);
+  if ((p.K & 127) == 0 && skinny_rows && p.K <= 1024 * 128 && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }

@@ -290,15 +290,11 @@ def splits(request):
     _lib.load().sglq_debug_force_splits(0)
 
 
-@pytest.mark.parametrize("mnk", [(1, 128, 128), (7, 2112, 7168), (16, 7168, 2048), (17, 264, 1024), (33, 4096, 512),
-                                 (64, 1536, 4096), (48, 136, 16384)])
-def test_decode_kernel_split_k(gpu, splits, mnk):
-    """M <= 64 runs on the weight-streaming kernel; its split-K partial sums and the
-    reduction must reproduce the oracle for every kind and any split factor."""
+def check_every_kind(gpu, m, n, k):
+    """Block-scaled FP8 (both output types), per-row / per-column FP8 and INT8 with bias, raw
+    INT32 accumulators: against the oracle on all rows."""
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32, int8_scaled_mm
 
-    say("decode kernel", mnk, "splits", splits)
-    m, n, k = mnk
     # block-scaled FP8
     _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m * n + k, outliers=True)
     ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
@@ -324,6 +320,33 @@ def test_decode_kernel_split_k(gpu, splits, mnk):
     ref = O.int8_scaled_mm(a8, w8.t(), sa8, sb, torch.bfloat16, bias)
     out = int8_scaled_mm(a8.to(gpu), w8.to(gpu).t(), sa8.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (7, 2112, 7168), (16, 7168, 2048), (17, 264, 1024), (33, 4096, 512),
+                                 (64, 1536, 4096), (48, 136, 16384)])
+def test_decode_kernel_split_k(gpu, splits, mnk):
+    """M <= 64 runs on the weight-streaming kernel; its split-K partial sums and the
+    reduction must reproduce the oracle for every kind and any split factor."""
+    say("decode kernel", mnk, "splits", splits)
+    check_every_kind(gpu, *mnk)
+
+
+@pytest.mark.parametrize("mnk", [(65, 264, 1024), (100, 2112, 1536), (128, 4096, 512), (129, 640, 2048), (300, 384, 1024),
+                                 (512, 256, 4096)])
+def test_decode_kernel_row_tiles(gpu, splits, mnk):
+    """The weight-streaming kernel with a second grid dimension of 64-row tiles (up to M = 512
+    when forced; the heuristic takes it up to M = 128): every kind, any split factor, ragged
+    last tile."""
+    from sglang_amd import _lib
+
+    say("decode kernel, row tiles", mnk, "splits", splits)
+    lib = _lib.load()
+    lib.sglq_debug_force_tile(64)
+    try:
+        check_every_kind(gpu, *mnk)
+        assert lib.sglq_debug_last_gemm_kernel().decode().startswith("gemm_skinny_kernel")
+    finally:
+        lib.sglq_debug_force_tile(0)
 
 
 @pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
