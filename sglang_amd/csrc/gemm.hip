@@ -1583,15 +1583,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int AR = MI * 16 < 32 ? 32 : MI * 16;  // activation rows staged (at least one copy per wave)
   constexpr int ACW = AR / 32;                     // activation copies per wave per stage
   constexpr bool BLOCK = is_block(KIND);
-  constexpr int CPW = 4 + ACW + (BLOCK ? 1 : 0);   // vector-memory loads per wave per stage
-  constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 1024 : 0;
+  constexpr int CPW = 4 + ACW + (BLOCK ? 2 : 0);   // vector-memory loads per wave per stage
+  constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 2048 : 0;  // 4 x 256 B of activation scales, then the weight scale
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
-  constexpr int NSTAGE = 3;  // 64-77 KiB of LDS: two blocks (eight waves) per CU
-  constexpr int MAX_STEPS = 1024;                  // K blocks per split that the weight-scale table holds
+  // 60-78 KiB of LDS: two blocks (eight waves) per CU.  A ring of six stages (one block per CU,
+  // five stages in flight) was measured and is no faster: a launch of 256 blocks asks for its
+  // first stages all at once, and what the memory system delivers to that burst sets the time.
+  constexpr int NSTAGE = 3;
   constexpr bool IS_FP8 = fp8_operands(KIND);
 
   __shared__ __attribute__((aligned(1024))) char smem[NSTAGE * STAGE_BYTES];
-  __shared__ float sfb_tab[BLOCK ? MAX_STEPS : 1];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1609,7 +1610,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 
   const v4u ra = make_rsrc_sgpr(p.a, p.a_bytes);
   const v4u rb = make_rsrc_sgpr(p.b, p.b_bytes);
-  v4u rs = ra;
+  v4u rs = ra, rsb = ra;
 
   // Same copy plan as the prefill kernel: lane l brings row l / 8 of an 8-row
   // group, chunk (l % 8) ^ swz(row); copies of one wave differ by 32 rows.
@@ -1617,17 +1618,22 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   const uint32_t off_w = (uint32_t)(n0 + wave * 8 + l8) * p.ldb + c16;
   const uint32_t off_a = (uint32_t)(m_base + wave * 8 + l8) * p.lda + c16;
   const uint32_t step_w = 32u * p.ldb, step_a = 32u * p.lda;
-  uint32_t off_s = 0;
-  int sfa_step = 0;
+  uint32_t off_s = 0, off_sb = OOB;
+  int sfa_step = 0, sfb_step = 0;
   if constexpr (BLOCK) {
     const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
     rs = make_rsrc_sgpr(p.sa, (uint32_t)(sfa_elems * 4));
     off_s = m_base + lane < p.M ? (uint32_t)((m_base + lane) * p.sa_stride_m * 4) : OOB;  // lane = activation row of the tile
     sfa_step = (int)(p.sa_stride_k * 4);
+    // the weight scale of the block's 128 weight rows travels with every stage as well: one
+    // dword, brought by lane 0 of wave 0 (the other lanes and waves are out of range; the
+    // instruction stays so that every wave counts the same number of copies per stage)
     const int nblocks = (p.N + 127) >> 7;
     const int nb = tile_n < nblocks ? tile_n : nblocks - 1;
-    for (int t = threadIdx.x; t < nsteps; t += 256)
-      sfb_tab[t] = p.sb[(int64_t)(kb0 + t * kstride) * p.sb_stride_k + nb * p.sb_stride_n];
+    const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
+    rsb = make_rsrc_sgpr(p.sb, (uint32_t)(sfb_elems * 4));
+    off_sb = (wave == 0 && lane == 0) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
+    sfb_step = (int)(p.sb_stride_k * 4);
   }
 
   const uint32_t smem_base = lds_addr(smem);
@@ -1639,7 +1645,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < ACW; ++j) lds_copy16(ra, st + W_BYTES + (wave + 4 * j) * 1024, off_a + j * step_a, k0);
     // one dword per lane: its row's activation scale for this K block
-    if constexpr (BLOCK) lds_copy4(rs, st + W_BYTES + A_BYTES + wave * 256, off_s, (uint32_t)((kb0 + t * kstride) * sfa_step));
+    if constexpr (BLOCK) {
+      lds_copy4(rs, st + W_BYTES + A_BYTES + wave * 256, off_s, (uint32_t)((kb0 + t * kstride) * sfa_step));
+      lds_copy4(rsb, st + W_BYTES + A_BYTES + 1024 + wave * 256, off_sb, (uint32_t)((kb0 + t * kstride) * sfb_step));
+    }
   };
 
   const int sw = (r16 & 7) ^ (r16 >> 3);
@@ -1657,10 +1666,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
-
-  // the sfb table was filled with ordinary loads and LDS stores: make it visible before the ring starts
-  __builtin_amdgcn_s_waitcnt(0);
-  __builtin_amdgcn_s_barrier();
 
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
@@ -1681,7 +1686,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
     for (int i = 0; i < MI; ++i) af[i] = read_frag(st + W_BYTES + i * 16 * 128);
     float sc[MI];
     if constexpr (BLOCK) {
-      const float sfb = sfb_tab[t];
+      const float sfb = *reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + 1024);
       const float* sfa = reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + wave * 256);
 #pragma unroll
       for (int i = 0; i < MI; ++i) sc[i] = sfa[i * 16 + r16] * sfb;
@@ -2104,7 +2109,8 @@ static void launch_reduce(GemmArgs& p, hipStream_t st) {
 template <int KIND, int MI, int OUT_DT>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
   g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
-  gemm_skinny_kernel<KIND, MI, OUT_DT><<<dim3((uint32_t)(p.tiles_n * p.splits), (uint32_t)p.tiles_m), dim3(256), 0, st>>>(p);
+  const dim3 grid((uint32_t)(p.tiles_n * p.splits), (uint32_t)p.tiles_m), block(256);
+  gemm_skinny_kernel<KIND, MI, OUT_DT><<<grid, block, 0, st>>>(p);
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
@@ -2164,7 +2170,6 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
 
 template <int KIND, int OUT_DT>
 static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
-  // the decode kernel keeps one weight scale per K block of its split in a 1024-entry table
   if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (g_force_tile == 0 || g_force_tile == 16 || g_force_tile == 32) &&
       launch_stream<KIND, OUT_DT>(p, st))
     return;
@@ -2172,7 +2177,7 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // 128 x 128 kernel (measured, e.g. 128 x 24576 x 1536: 28.3 -> 16.3 us, 128 x 4096 x 7168:
   // 21.2 -> 17.9 us; at K = 16384 the 128 x 128 kernel wins, 35 against 49 us).
   const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192) || (g_force_tile == 64 && p.M <= 512);
-  if ((p.K & 127) == 0 && skinny_rows && p.K <= 1024 * 128 && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
+  if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
