@@ -189,7 +189,8 @@ void sglq_debug_set_direct_lds(int on);
 /* Test hook: 0 = choose the GEMM kernel and tile by shape (default); 16 / 32 = the M <= 32
  * kernel whose blocks own 16 / 32 weight rows and all of K; 64 = the M <= 64 split-K kernel;
  * 128 = the 128x128 kernel; 256 = the plain 256x256 kernel; 258 = the pipelined 256x256
- * kernel; 192 / 224 / 257 = the pipelined 4x2-wave kernel with tiles 192 / 224 / 256 wide.
+ * kernel; 130 = the same kernel with 128-row tiles; 192 / 224 / 257 = the pipelined 4x2-wave
+ * kernel with tiles 192 / 224 / 256 wide.
  * A kernel that does not apply to the shape falls through to the next one that does. */
 void sglq_debug_force_tile(int tile);
 /* Test hook: > 0 fixes the split-K factor of the M <= 64 kernels (0 = by shape);

@@ -269,7 +269,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 // convert.  Chunk c (16 bytes) of image row r sits at chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
-template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, typename acc_t>
+template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, int HALF_ROWS = 128, typename acc_t>
 SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, float* col_lds, int m0, int n0,
                                int wm, int wn, int r16, int g, int lane, int wave) {
   constexpr int TN = NI * 16;
@@ -321,11 +321,12 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   // on.  Used when every 16-byte chunk of the tile's columns lies inside N and the extent fits
   // the 31-bit offsets (wave-uniform conditions).
   const uint32_t row_bytes = (uint32_t)p.ldo * 2u;
-  const int rows_left = p.M - m0 < 256 ? p.M - m0 : 256;
+  const int rows_left = p.M - m0 < 2 * HALF_ROWS ? p.M - m0 : 2 * HALF_ROWS;
   const bool whole_chunks = n0 + BN <= p.N && p.ldo < (1 << 21);
   const __amdgpu_buffer_rsrc_t r_out =
       make_rsrc(out + ((int64_t)m0 * p.ldo + n0) * 2, whole_chunks ? (uint32_t)rows_left * row_bytes - (uint32_t)n0 * 2u : 0u);
-  static_assert(MI % 2 == 0 && (HR & (HR - 1)) == 0 && 128 % HR == 0, "the halves are split by fragment row");
+  static_assert(MI % 2 == 0 && (HR & (HR - 1)) == 0 && HALF_ROWS % HR == 0 && HALF_ROWS % 16 == 0, "the halves are split by fragment row");
+  constexpr int RPW = HALF_ROWS / 8;  // image rows per wave in the store phase
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     {
@@ -373,17 +374,17 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
     // 128 image rows, 8 waves: wave w writes rows 16 w .. 16 w + 15, two rows per store
     // instruction; image row ml is row ml % HR of wave row ml / HR's half.  All eight reads are
     // issued before the first store (one LDS latency instead of eight).
-    v4i v[8];
+    v4i v[RPW / 2];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int ml = wave * 16 + it * 2 + (lane >> 5);
+    for (int it = 0; it < RPW / 2; ++it) {
+      const int ml = wave * RPW + it * 2 + (lane >> 5);
       v[it] = *reinterpret_cast<const v4i*>(img + ml * 512 + ((c ^ (ml & 31)) * 16));
     }
     if constexpr (add_bias) {
       const v4f blo = *reinterpret_cast<const v4f*>(col_lds + c * 8), bhi = *reinterpret_cast<const v4f*>(col_lds + c * 8 + 4);
       const float bias8[8] = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
+      for (int it = 0; it < RPW / 2; ++it) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint32_t w = (uint32_t)v[it][q];
@@ -407,16 +408,16 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
       // bounds-checked buffer stores: rows past M and lanes past the tile's width get an offset
       // beyond the extent and are dropped; no branches, no 64-bit address arithmetic
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int ml = wave * 16 + it * 2 + (lane >> 5);
+      for (int it = 0; it < RPW / 2; ++it) {
+        const int ml = wave * RPW + it * 2 + (lane >> 5);
         const uint32_t m_rel = (uint32_t)((ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1)));
         const uint32_t voff = (c * 8 < BN) ? m_rel * row_bytes + (uint32_t)c * 16u : OOB;
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 0);
       }
     } else {
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int ml = wave * 16 + it * 2 + (lane >> 5);
+      for (int it = 0; it < RPW / 2; ++it) {
+        const int ml = wave * RPW + it * 2 + (lane >> 5);
         const int m = m0 + (ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1));
         if (m < p.M && c * 8 < BN) {
           char* row = out + ((int64_t)m * p.ldo + n) * 2;
@@ -890,14 +891,17 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 // partial sums to the workspace), 2 = whole tiles of a block-scaled kind with a bias,
 // 3 = grouped GEMM (row tiles and their experts from the plan in the workspace).
 constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2, PIPE_GROUPED = 3;
-template <int KIND, int OUT_DT, int MODE>
+// BM = 128: tiles of 128 rows (a wave owns 64 x 64, 16 MFMAs per step) for problems whose
+// 256-row tiles would leave most of the chip idle; same schedule, half the activation copies.
+template <int KIND, int OUT_DT, int MODE, int BM = 256>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
-  constexpr int BM = 256, BN = 256, NW = 8, WAVES_N = 4;
-  constexpr int TM = 128, TN = 64, MI = TM / 16, NI = TN / 16;
+  constexpr int BN = 256, NW = 8, WAVES_N = 4;
+  constexpr int TM = BM / 2, TN = 64, MI = TM / 16, NI = TN / 16;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
+  constexpr int NCOPY_A = BM / 64;  // activation copies per wave per stage
   constexpr bool IS_FP8 = fp8_operands(KIND);
   constexpr bool BLOCK = is_block(KIND);
-  static_assert(NI == 4 && MI == 8, "the copy schedule below is written for 4 x 8 fragments");
+  static_assert(NI == 4 && (MI == 8 || MI == 4), "the copy schedule below is written for 4 x 8 or 4 x 4 fragments");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
   // (one LDS object per kernel, see gemm_big_kernel: the epilogue's 512 floats sit at the end)
@@ -992,7 +996,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   auto scale_offset = [&](int m0, int n0, int expert) -> uint32_t {
     if (wave < 4) {
       const int row = m0 + wave * 64 + lane;
-      return row < p.M ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
+      return (wave * 64 < BM && row < p.M) ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
     }
     const int nblocks = (p.N + 127) >> 7;
     int nb = (n0 >> 7) + lane;
@@ -1038,7 +1042,9 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         // tile's first step).  Younger than it are only the four weight copies of block u + 2,
         // which stay in flight.  lgkmcnt(0): this wave's LDS reads of block u's activations
         // and scales are complete.  A bare s_barrier: these waits are all the ordering needed.
-        constexpr int YOUNGER = last ? 0 : 4;
+        // (with 16 MFMAs per step the first step's weight copies of block u + 2 come behind
+        // this barrier, and what is in flight here are the deferred copies of block u + 1)
+        constexpr int YOUNGER = (last || (first && MI == 4)) ? 0 : 4;
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(YOUNGER));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -1069,19 +1075,19 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           // weight fragment j has had its last use in this step: refill it from block u + 1
           bf[j] = read_frag(sn + b_base + j * 16 * 128);
           if (j == 0) a_nxt = read_frag(sn + a_base);
-          if (!last) copy_a(j, cur, kn2 * 128, off_a2);
+          if (!last && j < NCOPY_A) copy_a(j, cur, kn2 * 128, off_a2);
           if constexpr (BLOCK) {
-            // scales i < 7 had their last use when fragment 7's scale was formed; sfa_cur[7] and
-            // sfb_cur are dead as well: `sc` holds their product
-            sfa_cur[2 * j] = read_sfa(cur ^ 1, 2 * j);
-            sfa_cur[2 * j + 1] = read_sfa(cur ^ 1, 2 * j + 1);
+            // scales i < MI - 1 had their last use when the last fragment's scale was formed; its own
+            // scale and sfb_cur are dead as well: `sc` holds their product
+#pragma unroll
+            for (int q = 0; q < MI / NI; ++q) sfa_cur[(MI / NI) * j + q] = read_sfa(cur ^ 1, (MI / NI) * j + q);
             if (j == 0) sfb_cur = read_sfb(cur ^ 1);
             if (j == 0 && !last) copy_scales(cur, kn2, sc_voff2);
           }
         }
         if constexpr (first) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b, false);
-          if (idx >= 8 && idx < 12) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
+          if (idx >= 8 && idx < 8 + NCOPY_A) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
           if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
           if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2, true);
         } else if constexpr (!last) {
@@ -1147,7 +1153,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   if constexpr (MODE == PIPE_GROUPED) b_cur = b_two = p.b + (int64_t)expert * p.b_expert_stride;
   if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0, expert);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_a(j, 0, kb0 * 128, off_a);
+  for (int j = 0; j < NCOPY_A; ++j) copy_a(j, 0, kb0 * 128, off_a);
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_b(j, 0, kb0 * 128, off_b, false);
   if constexpr (BLOCK) copy_scales(0, kb0, sc_voff);
@@ -1212,14 +1218,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       GemmArgs q = p;
       q.M = m_end;  // rows past the expert's last one belong to other experts
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, false>(q, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, false, BM / 2>(q, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
                                                           wave);
       else
         epilogue<KIND, OUT_DT, MI, NI, 0>(q, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
       if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn,
+        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS, BM / 2>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn,
                                                                      r16, g, lane, wave);
       else
         epilogue<KIND, OUT_DT, MI, NI, (MODE == PIPE_BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
@@ -2012,7 +2018,8 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 
 // test hook: 0 = heuristic, 64 = the M <= 64 kernel where it applies, 128 = the 128 x 128 kernel,
 // 256 = the plain 256 x 256 kernel, 258 = the pipelined one (K >= 384, else the plain one),
-// 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258)
+// 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258),
+// 130 = the pipelined kernel with 128-row tiles (K >= 384, else the 128 x 128 kernel)
 static int g_force_tile = 0;
 
 template <int KIND, int OUT_DT>
@@ -2064,6 +2071,41 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     } else {
       gemm_big_kernel<KIND, OUT_DT, false><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
     }
+  }
+}
+
+// The pipelined kernel with 128-row tiles: (tile, K range) work units, about one per CU.
+template <int KIND, int OUT_DT>
+static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  p.tiles_m = (p.M + 127) / 128;
+  p.tiles_n = (p.N + 255) / 256;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int nkb = p.K >> 7;
+  int splits = 1;
+  if (tiles < num_cus() || g_force_splits > 0) {
+    int want = g_force_splits > 0 ? g_force_splits : (num_cus() + tiles / 2) / tiles;
+    const int64_t per_split = (int64_t)p.M * p.N * 4;
+    if (!p.ws || ws_bytes < 2 * per_split || (int64_t)(p.M + 256) * p.N * 4 >= (int64_t)1 << 31) want = 1;
+    else if (want * per_split > ws_bytes) want = (int)(ws_bytes / per_split);
+    const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
+    if (g_force_splits == 0 && want > by_traffic) want = (int)(by_traffic > 0 ? by_traffic : 1);
+    for (int s = want; s >= 2; --s)
+      if (nkb % s == 0 && nkb / s >= (g_force_splits > 0 ? 3 : 4)) {
+        splits = s;
+        break;
+      }
+  }
+  p.splits = splits;
+  const int units = tiles * splits;
+  const dim3 grid((uint32_t)(units < num_cus() ? units : num_cus())), block(512);
+  g_last_kernel = splits > 1 ? "gemm_pipe_kernel<128 rows>+splitk_reduce_kernel" : "gemm_pipe_kernel<128 rows>";
+  if (splits > 1) {
+    gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK, 128><<<grid, block, 0, st>>>(p);
+    launch_reduce<KIND, OUT_DT>(p, st);  // (adds the bias)
+  } else if (is_block(KIND) && p.bias) {
+    if constexpr (is_block(KIND)) gemm_pipe_kernel<KIND, OUT_DT, PIPE_BIAS, 128><<<grid, block, 0, st>>>(p);
+  } else {
+    gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN, 128><<<grid, block, 0, st>>>(p);
   }
 }
 
@@ -2197,6 +2239,15 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
     else if (width == 257) launch_wide<KIND, OUT_DT, 8>(p, st);
     else launch_big<KIND, OUT_DT>(p, ws_bytes, st);
+    return;
+  }
+  // Between the two: the pipelined kernel with 128-row tiles and K split over work units.
+  // Measured against the 128 x 128 kernel: 256 x 7168 x 16384 64 -> 44 us, 1024 x 7168 x 2048
+  // 26 -> 20 us, 2048 x 4096 x 7168 74 -> 58 us, 2048 x 2112 x 7168 64 -> 48 us; below 256 rows
+  // it only wins on large weights (256 x 24576 x 1536 22 -> 17 us, but 256 x 2112 x 7168 19 -> 21 us).
+  const bool mid = p.M > 256 || (p.M > 128 && (int64_t)p.N * p.K >= (24 << 20));
+  if ((p.K & 127) == 0 && p.K >= 384 && (g_force_tile == 130 || (g_force_tile == 0 && g_use_dma && mid))) {
+    launch_pipe128<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
   if (p.M <= 32) launch_cfg<KIND, 32, 128, 1, 4, OUT_DT>(p, ws_bytes, st);

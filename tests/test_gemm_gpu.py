@@ -37,10 +37,10 @@ def load_path(request):
     _lib.load().sglq_debug_set_direct_lds(1)
 
 
-# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel,
+# tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel, 130 the same kernel with 128-row tiles,
 # 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 16, 32],
-                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "stream16", "stream32"])
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32],
+                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -418,8 +418,9 @@ def test_mid_m_split_k(gpu, splits, mnk):
     assert torch.equal(int8_mm_i32(a8.to(gpu), w8.to(gpu).t()).cpu()[rows], O.int8_mm_i32(a8[rows], w8.t()))
 
 
+@pytest.mark.parametrize("rows", [256, 128], ids=["pipe256", "pipe128"])
 @pytest.mark.parametrize("mnk", [(100, 384, 1536), (512, 640, 7168), (300, 2112, 3072), (1000, 256, 1536)])
-def test_pipelined_kernel_split_k(gpu, splits, mnk):
+def test_pipelined_kernel_split_k(gpu, splits, mnk, rows):
     """The pipelined 256 x 256 kernel takes (tile, K range) work units when the tiles do not fill
     the chip (forced here): every kind, block-scaled INT8 included, and any split factor that
     leaves three K blocks per unit."""
@@ -427,9 +428,9 @@ def test_pipelined_kernel_split_k(gpu, splits, mnk):
     from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_mm_i32
 
-    say("pipelined kernel split-K", mnk, "splits", splits)
+    say("pipelined kernel split-K", mnk, "splits", splits, "rows per tile", rows)
     lib = _lib.load()
-    lib.sglq_debug_force_tile(258)
+    lib.sglq_debug_force_tile(258 if rows == 256 else 130)
     try:
         m, n, k = mnk
         _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)

@@ -14,7 +14,7 @@ RTOL, ATOL = 1e-2, 1e-2
 
 # (force_tile code, M range, needs K % 128 == 0)
 SELECTIONS = [
-    (0, (1, 700), False), (128, (1, 300), False), (256, (65, 600), True), (258, (65, 600), True),
+    (0, (1, 700), False), (128, (1, 300), False), (256, (65, 600), True), (258, (65, 600), True), (130, (65, 600), True),
     (192, (65, 600), True), (224, (65, 600), True), (257, (65, 600), True), (64, (1, 64), True),
     (16, (1, 32), True), (32, (1, 32), True),
 ]
@@ -77,7 +77,7 @@ def test_random_shapes_all_kinds(gpu, code, m_range, k128):
         lib.sglq_debug_force_tile(0)
 
 
-@pytest.mark.parametrize("code,m", [(0, 300), (128, 300), (256, 300), (258, 300), (224, 300), (192, 300), (64, 48), (16, 9), (32, 20)],
+@pytest.mark.parametrize("code,m", [(0, 300), (128, 300), (256, 300), (258, 300), (130, 300), (224, 300), (192, 300), (64, 48), (16, 9), (32, 20)],
                          ids=lambda v: str(v))
 def test_strided_operands(gpu, code, m):
     """mat_a a column slice of a wider tensor (row stride 2 K + 64), mat_b a slice of a wider
