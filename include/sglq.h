@@ -35,7 +35,7 @@ int sglq_abi_version(void);
 /* Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_fp8
  * (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217,230-240; schema
  * sgl-kernel/csrc/common_extension.cc:116-119).  The UE8M0 packed-scale mode
- * (scale_ue8m0=true) is not built.
+ * (scale_ue8m0=true) is sglq_per_token_group_quant_fp8_ue8m0.
  *
  * input  [num_tokens, hidden] contiguous, in_dtype in {BF16, FP16, FP32}
  * output_q  same shape, one e4m3fn byte per element
@@ -47,6 +47,19 @@ int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output
                                    int64_t num_tokens, int64_t hidden, int group_size,
                                    int64_t s_stride_row, int64_t s_stride_col, float eps, float fp8_min,
                                    float fp8_max, void* stream);
+
+/* sgl_per_token_group_quant_fp8 with scale_ue8m0 = true
+ * (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:50-65,86-105,193-204; the
+ * output tensor of python/sglang/srt/layers/quantization/fp8_kernel.py:308-320):
+ * groups of 128; the scale of a group is the smallest power of two >=
+ * max(max(|x|, eps) / fp8_max, 1e-10) and codes are clamp(x / scale) rounded to
+ * e4m3fn.  output_s is the reference's packed int32 tensor [num_tokens, ceil4(K/128)/4]
+ * with column stride s_stride_col (in 32-bit words, >= num_tokens) and row stride 1: byte
+ * g % 4 of word (row, g / 4) receives the biased exponent (scale = 2^(byte - 127)) of
+ * group g.  Bytes of groups beyond K/128 are left as they are (the caller zero-fills). */
+int sglq_per_token_group_quant_fp8_ue8m0(const void* input, int in_dtype, void* output_q, void* output_s,
+                                         int64_t num_tokens, int64_t hidden, int64_t s_stride_col, float eps,
+                                         float fp8_min, float fp8_max, void* stream);
 
 /* Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_int8
  * (per_token_group_quant_8bit.cu:219-228; schema common_extension.cc:121-124):

@@ -187,6 +187,41 @@ def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q.to(FP8), scale
 
 
+def per_token_group_quant_fp8_ue8m0(x: torch.Tensor, eps: float = 1e-10) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """sgl_per_token_group_quant_fp8 with scale_ue8m0 = true, groups of 128
+    (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:45,72-113).
+
+    amax = max(eps, max|x|) per group (:45,72-84); y_s = amax / 448 (:86);
+    y_s = exp2(ceil(log2(max(y_s, 1e-10)))) (:87-89), taken here as the smallest power of two
+    that is >= its argument, read off the float's exponent and mantissa bits; the stored byte
+    is log2(y_s) + 127 (:94-99); q = clamp(x / y_s, -448, 448) -> e4m3fn RNE (:108-111).
+    Where log2f's own rounding could cross an integer (a quotient within a few units in the
+    last place above a power of two, fp32 inputs only) the reference's result depends on its
+    log2f and is not pinned.
+
+    Returns (q, exponent bytes [M, K/128] uint8, packed int32 [M, ceil4(K/128)/4] laid out as
+    python/sglang/srt/layers/quantization/fp8_kernel.py:308-320: zero-filled words of four
+    bytes, column-major with the column stride rounded up to 4 rows)."""
+    m, k = x.shape
+    assert k % 128 == 0
+    xf = x.to(torch.float32).reshape(m, k // 128, 128)
+    amax = torch.clamp(xf.abs().amax(dim=2), min=eps)
+    y = torch.clamp(amax / torch.tensor(FP8_E4M3_MAX, dtype=torch.float32), min=1e-10)
+    bits = y.view(torch.int32)
+    biased = (bits >> 23) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+    scale = ((biased << 23).to(torch.int32)).view(torch.float32)
+    q = torch.clamp(xf / scale.unsqueeze(2), -FP8_E4M3_MAX, FP8_E4M3_MAX).to(FP8).reshape(m, k)
+    groups = k // 128
+    words = (groups + 3) // 4
+    padded = torch.zeros((m, words * 4), dtype=torch.int32)
+    padded[:, :groups] = biased
+    packed_vals = padded[:, 0::4] | (padded[:, 1::4] << 8) | (padded[:, 2::4] << 16) | (padded[:, 3::4] << 24)
+    aligned_m = (m + 3) // 4 * 4
+    packed = torch.zeros((words, aligned_m), dtype=torch.int32).transpose(0, 1)[:m, :]
+    packed.copy_(packed_vals)
+    return q, biased.to(torch.uint8), packed
+
+
 def per_tensor_quant_fp8(x: torch.Tensor, scale: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-123.
 

@@ -27,6 +27,7 @@ SIGNATURES = {
     "sglq_per_token_group_quant_int8": _GROUP_QUANT,
     "sglq_per_token_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_token_quant_int8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    "sglq_per_token_group_quant_fp8_ue8m0": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_void_p],
     "sglq_per_tensor_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p],
     "sglq_static_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,

@@ -200,6 +200,45 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict
 }
 
 // ---------------------------------------------------------------------------
+// Per-token-group FP8 quantization with power-of-two scales packed as exponent bytes
+// (scale_ue8m0, per_token_group_quant_8bit.cu:86-105 and :50-65; groups of 128).  The scale
+// is the smallest power of two >= max(amax / 448, 1e-10), which is what
+// exp2f(ceilf(log2f(.))) (:87-89) yields wherever log2f's own rounding cannot cross an
+// integer: always for bf16 / fp16 inputs (amax / 448 is then an exact power of two or at
+// least 2^-9 away from one in relative terms), and for fp32 inputs except a quotient a few
+// units in the last place above a power of two.  Byte g % 4 of 32-bit word
+// [g / 4][row] of the output (word column stride s_stride_col) is the biased exponent of
+// group g's scale (:57-64, :94).  16 lanes per group, 8 elements per lane.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void group_quant_ue8m0_kernel(const char* __restrict__ x, char* __restrict__ q,
+                                                                unsigned char* __restrict__ s, uint32_t num_groups,
+                                                                FastDiv groups_per_row, int64_t s_stride_col, float eps,
+                                                                float qmin, float qmax, float rqmax) {
+  constexpr int EB = elem_bytes<DT>();
+  const uint32_t sub = threadIdx.x & 15;
+  const uint32_t gid = blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (gid >= num_groups) return;
+  Chunk8<DT> ch;
+  ch.load(x + ((int64_t)gid * 128 + sub * 8) * EB);
+  const uint32_t mb = group_umax<16>(ch.amax_bits());
+  const float amax = u2f(umax(mb, f2u(eps)));
+  const float y = __builtin_fmaxf(div_by(amax, qmax, rqmax), 1e-10f);
+  const uint32_t bits = f2u(y);  // positive and normal (>= 1e-10)
+  const uint32_t biased = (bits >> 23) + ((bits & 0x7fffffu) != 0 ? 1u : 0u);  // exponent of the power of two >= y
+  const float inv = u2f((254u - biased) << 23);                                // 2^-(biased - 127), exact
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = __builtin_fminf(__builtin_fmaxf(ch.get(i) * inv, qmin), qmax);
+  *reinterpret_cast<v2u*>(q + (int64_t)gid * 128 + sub * 8) = Fp8Pack::pack(v);
+  if (sub == 0) {
+    const uint32_t row = groups_per_row.div(gid);
+    const uint32_t col = gid - row * groups_per_row.d;
+    s[((int64_t)(col >> 2) * s_stride_col + row) * 4 + (col & 3)] = (unsigned char)biased;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Per-token (whole-row) quantization.  TEAM lanes share one row (64 = one
 // wavefront, 256 = the block); each lane keeps V 16-byte chunks in registers.
 // ---------------------------------------------------------------------------
@@ -540,6 +579,52 @@ static int group_quant_entry(const char* name, const void* input, int in_dtype, 
   return SGLQ_EUNSUPPORTED;
 }
 
+static int group_quant_ue8m0_entry(const void* input, int in_dtype, void* output_q, void* output_s, int64_t num_tokens,
+                                   int64_t hidden, int64_t s_stride_col, float eps, float qmin, float qmax, void* stream) {
+  const char* name = "sgl_per_token_group_quant_fp8 (scale_ue8m0)";
+  if (!input || !output_q || !output_s) {
+    if (num_tokens == 0) return SGLQ_OK;
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_tokens < 0 || hidden <= 0 || hidden % 128 != 0) {
+    set_error("%s: hidden (%lld) must be a positive multiple of 128", name, (long long)hidden);
+    return SGLQ_EINVAL;
+  }
+  if (!(qmax > 0.f) || !(eps > 0.f) || s_stride_col < num_tokens) {
+    set_error("%s: eps and the 8-bit maximum must be positive, the scale column stride at least num_tokens", name);
+    return SGLQ_EINVAL;
+  }
+  if ((reinterpret_cast<uintptr_t>(input) & 15) || (reinterpret_cast<uintptr_t>(output_q) & 7) ||
+      (reinterpret_cast<uintptr_t>(output_s) & 3)) {
+    set_error("%s: input must be 16-byte, output_q 8-byte and output_s 4-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t gpr = hidden / 128, ng = num_tokens * gpr;
+  if (ng == 0) return SGLQ_OK;
+  if (ng >= (1ll << 32) - 65536) {
+    set_error("%s: too many groups (%lld)", name, (long long)ng);
+    return SGLQ_EINVAL;
+  }
+  FastDiv fd;
+  fd.init((uint32_t)gpr);
+  const dim3 grid((uint32_t)((ng + 15) / 16)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const char* xi = static_cast<const char*>(input);
+  char* qo = static_cast<char*>(output_q);
+  unsigned char* so = static_cast<unsigned char*>(output_s);
+  const float rq = 1.0f / qmax;
+  switch (in_dtype) {
+    case SGLQ_BF16: group_quant_ue8m0_kernel<SGLQ_BF16><<<grid, block, 0, st>>>(xi, qo, so, (uint32_t)ng, fd, s_stride_col, eps, qmin, qmax, rq); break;
+    case SGLQ_FP16: group_quant_ue8m0_kernel<SGLQ_FP16><<<grid, block, 0, st>>>(xi, qo, so, (uint32_t)ng, fd, s_stride_col, eps, qmin, qmax, rq); break;
+    case SGLQ_FP32: group_quant_ue8m0_kernel<SGLQ_FP32><<<grid, block, 0, st>>>(xi, qo, so, (uint32_t)ng, fd, s_stride_col, eps, qmin, qmax, rq); break;
+    default:
+      set_error("%s: input dtype must be bf16, fp16 or fp32", name);
+      return SGLQ_EUNSUPPORTED;
+  }
+  return check_launch(name);
+}
+
 template <int DT, int MODE>
 static int launch_token_quant(const char* name, const void* x, void* q, float* s, void* row_sum, int64_t rows,
                               int64_t hidden, hipStream_t st) {
@@ -689,6 +774,13 @@ extern "C" int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, v
   return sglq::group_quant_entry<false>("sgl_per_token_group_quant_fp8", input, in_dtype, output_q, output_s,
                                         num_tokens, hidden, group_size, s_stride_row, s_stride_col, eps, fp8_min,
                                         fp8_max, stream);
+}
+
+extern "C" int sglq_per_token_group_quant_fp8_ue8m0(const void* input, int in_dtype, void* output_q, void* output_s,
+                                                    int64_t num_tokens, int64_t hidden, int64_t s_stride_col, float eps,
+                                                    float fp8_min, float fp8_max, void* stream) {
+  return sglq::group_quant_ue8m0_entry(input, in_dtype, output_q, output_s, num_tokens, hidden, s_stride_col, eps, fp8_min,
+                                       fp8_max, stream);
 }
 
 extern "C" int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,

@@ -29,7 +29,14 @@ def create_per_token_group_quant_fp8_output_scale(
 ):
     """Scale buffer in the layout the consumer GEMM wants (fp8_kernel.py:300-341)."""
     if scale_ue8m0:
-        raise NotImplementedError("packed UE8M0 scales are not built")
+        # int32 words of four exponent bytes, [ceil4(K/128)/4, ceil4(M)] transposed; zero-filled as in the
+        # reference (:319-323), so that the bytes of groups beyond K/128 are defined
+        assert column_major_scales and scale_tma_aligned
+        x_q_mn, x_q_k = x_shape
+        x_s_mn, x_s_k = x_q_mn, x_q_k // 128
+        aligned_mn = (x_s_mn + 3) // 4 * 4
+        aligned_k = (x_s_k + 3) // 4 * 4
+        return torch.zeros((aligned_k // 4, aligned_mn), device=device, dtype=torch.int).transpose(0, 1)[:x_s_mn, :]
     if column_major_scales:
         if scale_tma_aligned:
             aligned_size = (x_shape[-2] + 3) // 4 * 4

@@ -224,7 +224,30 @@ def _group_quant_impl(fn_name, q_dtype, input, output_q, output_s, group_size, e
 
 def _sgl_per_token_group_quant_fp8_impl(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0):
     if scale_ue8m0:
-        raise NotImplementedError("sgl_per_token_group_quant_fp8: scale_ue8m0=True (packed power-of-two scales) is not built")
+        # power-of-two scales packed four exponent bytes to an int32 word, column-major
+        # (per_token_group_quant_8bit.cu:50-65,86-105; the reference asserts a column-major buffer, :190-191)
+        for name, t in (("input", input), ("output_q", output_q)):
+            _check(t.is_cuda, f"{name} must be a CUDA tensor")
+            _check(t.is_contiguous(), f"{name} must be contiguous")
+        _check(output_s.is_cuda, "output_s must be a CUDA tensor")
+        _check(input.dtype in DTYPE_CODE, "input must be Float, Half or BFloat16")
+        _check(output_q.dtype == FP8 and output_q.shape == input.shape, "output_q must be Float8_e4m3fn with the shape of input")
+        if group_size != 128:
+            raise NotImplementedError("sgl_per_token_group_quant_fp8: scale_ue8m0=True is built for group_size 128 only")
+        _check(input.dim() >= 1 and input.shape[-1] % 128 == 0, "the last dimension must be divisible by group_size")
+        _check(output_s.dim() == 2, "output_s must be a 2D tensor")
+        _check(output_s.dtype == torch.int32, "output_s must be Int32 (four UE8M0 scales per element)")
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        groups = input.shape[-1] // 128
+        _check(output_s.size(0) == rows and output_s.size(1) * 4 >= groups, "output_s has the wrong shape")
+        if rows == 0:
+            return
+        _check(output_s.stride(0) == 1 and output_s.stride(1) >= rows, "output_s must be column major (scale_ue8m0)")
+        rc = _lib.load().sglq_per_token_group_quant_fp8_ue8m0(
+            input.data_ptr(), DTYPE_CODE[input.dtype], output_q.data_ptr(), output_s.data_ptr(), rows, input.shape[-1],
+            output_s.stride(1), float(eps), float(fp8_min), float(fp8_max), _lib.stream_ptr(input.device))
+        _lib.check(rc, "sgl_per_token_group_quant_fp8")
+        return
     _group_quant_impl("sglq_per_token_group_quant_fp8", FP8, input, output_q, output_s, group_size, eps, fp8_min, fp8_max)
 
 

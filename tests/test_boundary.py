@@ -139,8 +139,9 @@ def test_scale_buffer_layouts_match_reference_allocator():
     assert tuple(s.shape) == (6, 4) and s.stride() == (1, 6)
     s = mk((6, 512), "cpu", 128, True, True, False)
     assert tuple(s.shape) == (6, 4) and s.stride() == (1, 8)
-    with pytest.raises(NotImplementedError):
-        mk((6, 512), "cpu", 128, True, True, True)
+    # scale_ue8m0: int32 words of four exponent bytes, zero-filled, column stride ceil4(M) (fp8_kernel.py:308-320)
+    s = mk((6, 1536), "cpu", 128, True, True, True)
+    assert s.dtype == torch.int32 and tuple(s.shape) == (6, 3) and s.stride() == (1, 8) and int(s.abs().max()) == 0
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():

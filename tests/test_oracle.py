@@ -237,6 +237,49 @@ def test_tensor_fp8_closed_form_and_zero_tensor(c_oracle):
     assert fp8_bits(q).unique().tolist() == [0x7E] and qc.unique().tolist() == [0x7E]
 
 
+# ------------------------------------------------------------------ f2 UE8M0 group scales
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_group_quant_ue8m0_pins(dtype):
+    """Power-of-two scales: the reference test's formula 2^ceil(log2(amax / 448))
+    (python/sglang/test/test_block_fp8_deep_gemm_blackwell.py:48-59) evaluated in float64, where
+    log2 of these fp32 quotients cannot round across an integer; exponent bytes, packing and
+    codes from first principles."""
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn((37, 640), generator=g) * torch.logspace(-6, 4, 37).unsqueeze(1)).to(dtype)
+    x[5, 128:256] = 0  # an all-zero group: eps / 448 < 1e-10, so the scale is the power of two >= 1e-10
+    q, exps, packed = O.per_token_group_quant_fp8_ue8m0(x)
+    amax = x.float().view(37, 5, 128).abs().amax(dim=2).clamp(min=1e-10)
+    y = (amax / 448.0).clamp(min=1e-10)  # fp32, as the kernel
+    want_scale = torch.pow(2.0, torch.ceil(torch.log2(y.double())))
+    got_scale = torch.pow(2.0, exps.double() - 127)
+    assert torch.equal(got_scale, want_scale)
+    # the regular scale amax / 448 is at most the power-of-two scale and more than half of it
+    assert bool((got_scale >= y.double()).all()) and bool((got_scale < 2 * y.double()).all())
+    assert exps[5, 1].item() == 127 + math.ceil(math.log2(1e-10))  # 2^-33
+    # codes: exact division by a power of two, then the e4m3fn cast that the other quant ops use
+    want_q = (x.float().view(37, 5, 128) / got_scale.float().unsqueeze(2)).clamp(-448, 448).to(FP8).view(37, 640)
+    assert_bits_equal(q, want_q, "codes")
+    assert float(q.float().abs().max()) <= 448.0 and float(q.float().abs().max()) > 224.0
+    # packing: byte g % 4 of word g / 4; words of groups that do not exist stay zero; column-major, stride ceil4(M)
+    assert tuple(packed.shape) == (37, 2) and packed.stride() == (1, 40) and packed.dtype == torch.int32
+    by = packed.contiguous().view(torch.uint8).view(37, 2, 4)
+    assert torch.equal(by[:, 0, :], exps[:, 0:4]) and torch.equal(by[:, 1, 0], exps[:, 4])
+    assert int(by[:, 1, 1:].max()) == 0
+
+
+def test_group_quant_ue8m0_exact_powers_of_two():
+    # amax = 448 * 2^e: the quotient is a power of two and stays; one ulp above it doubles the scale
+    for e in (-20, -3, 0, 5):
+        x = torch.zeros((1, 128))
+        x[0, 7] = 448.0 * 2.0 ** e
+        x[0, 9] = -3.0 * 2.0 ** e
+        q, exps, _ = O.per_token_group_quant_fp8_ue8m0(x)
+        assert exps.item() == 127 + e and q[0, 7].float().item() == 448.0 and q[0, 9].float().item() == -3.0
+        x[0, 7] = float(np.nextafter(np.float32(448.0 * 2.0 ** e), np.float32(np.inf)))
+        q, exps, _ = O.per_token_group_quant_fp8_ue8m0(x)
+        assert exps.item() == 127 + e + 1 and q[0, 7].float().item() == 224.0 and q[0, 9].float().item() == -1.5
+
+
 # ------------------------------------------------------------------ f2 static per-tensor quant
 @pytest.mark.parametrize("dtype", [torch.half, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("num_tokens,d", [(7, 512), (83, 4096), (33, 5120)])

@@ -271,6 +271,46 @@ def test_static_quant_fp8_shapes_and_errors(gpu):
     assert q.shape == (0, 64) and s.shape == (0, 1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 128), (7, 512), (83, 1536), (130, 7168), (2048, 640)])
+def test_group_quant_ue8m0_bit_exact(gpu, dtype, shape):
+    """scale_ue8m0: codes and the packed exponent words (the reference's int32 tensor, padding
+    words included) bit for bit against the oracle."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    say("group_quant ue8m0", dtype, shape)
+    m, k = shape
+    x = (O.gen_activation(m, k, seed=m + k, outliers=True).float() * torch.logspace(-4, 3, m).unsqueeze(1)).to(dtype)
+    if m > 2:
+        x[2, :128] = 0
+    q_ref, exps_ref, packed_ref = O.per_token_group_quant_fp8_ue8m0(x)
+    q, s = sglang_per_token_group_quant_fp8(x.to(gpu), 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    assert s.dtype == torch.int32 and tuple(s.shape) == tuple(packed_ref.shape) and s.stride() == packed_ref.stride()
+    assert_bits_equal(q, q_ref, "codes")
+    assert torch.equal(s.cpu(), packed_ref), "packed exponents"
+    # dequantized with the power-of-two scales: within half an e4m3 step of the input
+    scale = torch.pow(2.0, exps_ref.float() - 127).repeat_interleave(128, dim=1)
+    err = (q.cpu().float() * scale - x.float()).abs()
+    assert bool((err <= 0.0625 * x.float().abs() + scale * 2.0 ** -10).all())
+
+
+def test_group_quant_ue8m0_argument_checks(gpu):
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8
+
+    x = torch.randn((8, 256), device=gpu, dtype=torch.bfloat16)
+    q = torch.empty((8, 256), device=gpu, dtype=FP8)
+    row_major = torch.zeros((8, 1), device=gpu, dtype=torch.int32)
+    s = torch.zeros((1, 8), device=gpu, dtype=torch.int32).t()
+    with pytest.raises(RuntimeError, match="Int32"):
+        sgl_per_token_group_quant_fp8(x, q, torch.zeros((2, 8), device=gpu).t(), 128, 1e-10, -448.0, 448.0, True)
+    with pytest.raises(NotImplementedError, match="group_size 128"):
+        sgl_per_token_group_quant_fp8(x, q, s, 64, 1e-10, -448.0, 448.0, True)
+    sgl_per_token_group_quant_fp8(x, q, s, 128, 1e-10, -448.0, 448.0, True)
+    _, _, packed = O.per_token_group_quant_fp8_ue8m0(x.cpu())
+    assert torch.equal(s.cpu(), packed)
+    del row_major
+
+
 def test_tensor_quant_full_size_properties(gpu):
     """8192 x 16384 (the largest activation of the configurations): quantizing the dequantized
     tensor with the same static scale reproduces the codes; the maximum code is 448."""
