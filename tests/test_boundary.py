@@ -166,5 +166,23 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     rc = lib.sglq_per_tensor_quant_fp8(p, 0, p, None, 16, 0, None)
     assert rc == 1 and b"scale" in lib.sglq_last_error()
     assert lib.sglq_per_tensor_quant_fp8(None, 0, None, p, 0, 1, None) == 0
+    # the widened operator set
+    rc = lib.sglq_static_quant_fp8(p, 0, p, None, None, 4, 16, None)
+    assert rc == 1 and b"scale" in lib.sglq_last_error()
+    rc = lib.sglq_static_quant_fp8(p, 9, p, p, None, 4, 16, None)
+    assert rc == 2 and b"dtype" in lib.sglq_last_error()
+    assert lib.sglq_static_quant_fp8(None, 0, None, p, None, 0, 16, None) == 0
+    rc = lib.sglq_per_token_group_quant_fp8_ue8m0(p, 0, p, p, 4, 200, 4, 1e-10, -448.0, 448.0, None)
+    assert rc == 1 and b"multiple of 128" in lib.sglq_last_error()
+    rc = lib.sglq_per_token_group_quant_fp8_ue8m0(p, 0, p, p, 8, 256, 4, 1e-10, -448.0, 448.0, None)
+    assert rc == 1 and b"column stride" in lib.sglq_last_error()
+    # grouped GEMM: a [32, 128], 2 experts of [16, 128]; workspace too small, then K not a multiple of 128, then no output type
+    grouped = lambda k, ws_bytes, dt: lib.sglq_fp8_blockwise_scaled_grouped_mm(
+        p, k, p, k, 16 * k, p, 1, 1, p, 1, 1, 1, p, 16, dt, p, p, 2, 32, 16, k, p, ws_bytes, None)
+    assert grouped(128, 8, 0) == 1 and b"workspace" in lib.sglq_last_error()
+    assert grouped(64, 4096, 0) == 1 and b"multiple of 128" in lib.sglq_last_error()
+    assert grouped(128, 4096, 2) == 1 and b"bfloat16 or half" in lib.sglq_last_error()
+    assert lib.sglq_fp8_blockwise_scaled_grouped_mm(p, 128, p, 128, 2048, p, 1, 1, p, 1, 1, 1, p, 16, 0, p, p, 0, 32, 16, 128, p, 4096,
+                                                    None) == 0  # no experts
     # empty problems are a no-op
     assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0
