@@ -174,6 +174,16 @@ int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int
                                   int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                   int64_t workspace_bytes, void* stream);
 
+/* sglq_int8_blockwise_scaled_mm fused with the bias add of its caller
+ * (python/sglang/srt/layers/quantization/int8_utils.py:25-32: the matmul rounded to the
+ * output type, then `output + bias`): out = round(round(gemm) + bias), bias [N] in out_dtype
+ * or NULL. */
+int sglq_int8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                       int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                       int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out,
+                                       int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                       int64_t workspace_bytes, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.int8_scaled_mm
  * (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; schema common_extension.cc:101-104).
  * out = float(acc) * (scales_b[n] * scales_a[m]) + bias[n], acc exact int32.

@@ -39,6 +39,8 @@ SIGNATURES = {
                                              c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_int8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                       c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
+    "sglq_int8_blockwise_scaled_mm_bias": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                           c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_int8_scaled_mm": _ROWCOL_MM,
     "sglq_fp8_scaled_mm": _ROWCOL_MM,
     "sglq_int8_mm_i32": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],

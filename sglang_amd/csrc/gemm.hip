@@ -2485,6 +2485,16 @@ extern "C" int sglq_int8_blockwise_scaled_mm(const void* a, int64_t lda, const v
                                         workspace_bytes, stream);
 }
 
+extern "C" int sglq_int8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                                  int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                                  int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out,
+                                                  int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                                  void* workspace, int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_I8_BLOCK>("w8a8_block_int8_matmul_bias", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
+                                        sfb_stride_k, sfb_stride_n, bias, out, ldo, out_dtype, M, N, K, workspace,
+                                        workspace_bytes, stream);
+}
+
 static int rowcol_entry(const char* name, bool fp8, const void* a, int64_t lda, const void* b, int64_t ldb,
                         const float* scales_a, const float* scales_b, const void* bias, void* out, int64_t ldo,
                         int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,

@@ -5,7 +5,7 @@ w8a8_block_int8_matmul (:339-425)."""
 
 from __future__ import annotations
 
-from typing import List, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -67,9 +67,12 @@ def w8a8_block_int8_matmul(
     Bs: torch.Tensor,
     block_size: List[int],
     output_dtype: torch.dtype = torch.float16,
+    bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """int8_kernel.py:339-425: A int8 [..., K] contiguous, B int8 [N, K] contiguous (the
-    weight as stored), As fp32 [..., K/128], Bs fp32 [N/128, K/128]."""
+    weight as stored), As fp32 [..., K/128], Bs fp32 [N/128, K/128].  `bias` (not an argument of
+    the reference's function): the caller's `output + bias` (int8_utils.py:31-32) fused, [N] in
+    output_dtype, same two roundings."""
     assert len(block_size) == 2
     block_n, block_k = block_size[0], block_size[1]
     if block_n != 128 or block_k != 128:
@@ -97,6 +100,15 @@ def w8a8_block_int8_matmul(
     if not Bs.is_contiguous():
         Bs = Bs.contiguous()
     lib = _lib.load()
+    if bias is not None:
+        if not (bias.is_cuda and bias.is_contiguous() and bias.numel() == N and bias.dtype == output_dtype):
+            raise RuntimeError("w8a8_block_int8_matmul: bias must be a contiguous CUDA tensor of N elements in output_dtype")
+        rc = lib.sglq_int8_blockwise_scaled_mm_bias(
+            A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
+            Bs.data_ptr(), Bs.stride(1), Bs.stride(0), bias.data_ptr(), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,
+            *_lib.workspace(A.device), _lib.stream_ptr(A.device))
+        _lib.check(rc, "w8a8_block_int8_matmul")
+        return C
     rc = lib.sglq_int8_blockwise_scaled_mm(
         A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
         Bs.data_ptr(), Bs.stride(1), Bs.stride(0), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,

@@ -22,7 +22,11 @@ def apply_w8a8_block_int8_linear(
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[0]]
     q_input, x_scale = per_token_group_quant_int8(input_2d, block_size[1])
-    output = w8a8_block_int8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
-    if bias is not None:
-        output = output + bias
+    if bias is not None and bias.dtype == input.dtype and bias.is_contiguous() and bias.numel() == weight.shape[0]:
+        # the matmul and `output + bias` (int8_utils.py:26-32) in one kernel, same two roundings
+        output = w8a8_block_int8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype, bias=bias)
+    else:
+        output = w8a8_block_int8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
+        if bias is not None:
+            output = output + bias
     return output.to(dtype=input.dtype).view(*output_shape)

@@ -178,6 +178,23 @@ def test_w8a8_block_int8_matmul(gpu, tile, mnk, out_dtype):
     torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("mnk", [(5, 2112, 1536), (100, 640, 1024), (300, 2048, 1024), (1024, 640, 2048)])
+def test_w8a8_block_int8_matmul_fused_bias(gpu, tile, mnk):
+    """Block-scaled INT8 with the caller's `output + bias` (int8_utils.py:31-32) fused: bit-identical
+    to the two steps done apart, on every kernel selection."""
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    say("block int8 fused bias", mnk, "tile", tile)
+    m, n, k = mnk
+    xq, xs, wq, ws = make_block_int8_case(m, n, k, seed=m + n + k)
+    args = (xq.to(gpu), wq.to(gpu), xs.to(gpu), ws.to(gpu), [128, 128])
+    for dt in (torch.bfloat16, torch.float16):
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(dt).to(gpu)
+        plain = w8a8_block_int8_matmul(*args, dt)
+        fused = w8a8_block_int8_matmul(*args, dt, bias=bias)
+        assert torch.equal(fused.view(torch.int16), (plain + bias).view(torch.int16)), dt
+
+
 def test_w8a8_block_int8_unit_scales_exact_and_linear(gpu):
     """Unit scales and small integers: exact whatever the summation order; then the glue
     (per-token-group INT8 quant, GEMM, bias) against the oracle's same sequence."""
