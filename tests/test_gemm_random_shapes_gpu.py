@@ -107,3 +107,46 @@ def test_strided_operands(gpu, code, m):
         torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
     finally:
         lib.sglq_debug_force_tile(0)
+
+
+@pytest.mark.parametrize("code", [0, 128, 130, 256, 258, 257, 224, 192, 64, 16, 32], ids=lambda v: f"tile{v}")
+@pytest.mark.parametrize("mn", [(300, 520), (257, 1000), (64, 264), (9, 2112), (513, 776)], ids=lambda v: f"{v[0]}x{v[1]}")
+def test_output_written_only_inside_its_rows_and_columns(gpu, code, mn):
+    """The output is a [M, N] window inside a larger sentinel-filled buffer (row stride N + 24,
+    guard rows above and below): through the C ABI, with and without a workspace, every kernel
+    must write its window and nothing else."""
+    from sglang_amd import _lib
+
+    m, n = mn
+    if (code in (16, 32) and m > 32) or (code == 64 and m > 512):
+        pytest.skip("kernel not applicable to this M")
+    k = 1024
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(m * n + code)
+    a = (torch.randn((m, k), generator=g) * 2).to(FP8)
+    w = (torch.randn((n, k), generator=g) * 0.5).to(FP8)
+    sfa = torch.rand((m, k // 128), generator=g) * 0.05 + 0.01
+    sfb = torch.rand(((n + 127) // 128, k // 128), generator=g) * 0.01 + 0.001
+    ref = O.fp8_blockwise_scaled_mm(a, w.t(), sfa, sfb.t(), torch.float32, acc_dtype=torch.float64)
+    ag, wg, sag, sbg = a.to(gpu), w.to(gpu), sfa.to(gpu), sfb.to(gpu)
+    ldo, guard = n + 24, 3
+    ws_ptr, ws_bytes = _lib.workspace(gpu)
+    lib.sglq_debug_force_tile(code)
+    try:
+        for use_ws in (True, False):
+            print("output window", code, mn, "workspace" if use_ws else "no workspace", flush=True)
+            buf = torch.full((m + 2 * guard, ldo), 768.0, dtype=torch.bfloat16, device=gpu)
+            out_ptr = buf.data_ptr() + (guard * ldo + 8) * 2  # window starts 8 columns in: rows stay 16-byte aligned
+            rc = lib.sglq_fp8_blockwise_scaled_mm(
+                ag.data_ptr(), k, wg.data_ptr(), k, sag.data_ptr(), sag.stride(0), sag.stride(1), sbg.data_ptr(), sbg.stride(1),
+                sbg.stride(0), out_ptr, ldo, 0, m, n, k, ws_ptr if use_ws else None, ws_bytes if use_ws else 0,
+                _lib.stream_ptr(gpu))
+            assert rc == 0, lib.sglq_last_error()
+            torch.cuda.synchronize()
+            host = buf.cpu().float()
+            window = host[guard:guard + m, 8:8 + n]
+            torch.testing.assert_close(window, ref, rtol=RTOL, atol=ATOL)
+            host[guard:guard + m, 8:8 + n] = 768.0
+            assert bool((host == 768.0).all()), "a kernel wrote outside the output window"
+    finally:
+        lib.sglq_debug_force_tile(0)
