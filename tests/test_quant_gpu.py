@@ -360,3 +360,70 @@ def test_group_quant_full_size_properties(gpu):
     q2, s2 = sglang_per_token_group_quant_fp8(deq, 128, column_major_scales=True)
     assert bool((s2 == s).all())
     assert bool((q2.view(torch.uint8) == q.view(torch.uint8)).all())
+
+
+@pytest.mark.parametrize("shape", [(1, 128), (5, 384), (33, 1024), (257, 7168)])
+def test_quant_kernels_write_only_their_outputs(gpu, shape):
+    """Codes and scales land in windows of sentinel-filled buffers (guard bytes before and after):
+    every quantization entry point, through the C ABI, must leave the guards alone."""
+    from sglang_amd import _lib
+
+    lib = _lib.load()
+    m, k = shape
+    say("quant output windows", shape)
+    x = O.gen_activation(m, k, seed=m * 7 + k, outliers=True).to(torch.bfloat16).to(gpu)
+    st = _lib.stream_ptr(gpu)
+    G = 64  # guard elements on each side
+
+    def window(numel, dtype, fill):
+        buf = torch.full((numel + 2 * G,), fill, dtype=dtype, device=gpu)
+        return buf, buf[G:G + numel]
+
+    def guards_intact(buf, numel, fill):
+        host = buf.cpu()
+        return bool((host[:G] == fill).all()) and bool((host[G + numel:] == fill).all())
+
+    groups = k // 128
+    cases = []
+    # per-token-group FP8, row-major and column-major (padded) scales; INT8 twin
+    for col_major in (False, True):
+        qb, q = window(m * k, torch.uint8, 0xAB)
+        ld = (m + 3) // 4 * 4
+        sb, s = window(ld * groups if col_major else m * groups, torch.float32, -7.0)
+        sr, sc = (1, ld) if col_major else (groups, 1)
+        rc = lib.sglq_per_token_group_quant_fp8(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), m, k, 128, sr, sc, 1e-10, -448.0, 448.0, st)
+        cases.append(("group fp8", rc, qb, m * k, 0xAB, sb, s.numel(), -7.0))
+    qb, q = window(m * k, torch.uint8, 0xAB)
+    sb, s = window(m * groups, torch.float32, -7.0)
+    rc = lib.sglq_per_token_group_quant_int8(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), m, k, 128, groups, 1, 1e-10, -128.0, 127.0, st)
+    cases.append(("group int8", rc, qb, m * k, 0xAB, sb, m * groups, -7.0))
+    # UE8M0: packed int32 words, column stride ceil4(M)
+    qb, q = window(m * k, torch.uint8, 0xAB)
+    ld = (m + 3) // 4 * 4
+    words = (groups + 3) // 4
+    sb, s = window(ld * words, torch.int32, 0x55555555)
+    rc = lib.sglq_per_token_group_quant_fp8_ue8m0(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), m, k, ld, 1e-10, -448.0, 448.0, st)
+    cases.append(("ue8m0", rc, qb, m * k, 0xAB, sb, ld * words, 0x55555555))
+    # per-token FP8 / INT8
+    for name, fn in (("token fp8", lambda q, s: lib.sglq_per_token_quant_fp8(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), m, k, st)),
+                     ("token int8", lambda q, s: lib.sglq_per_token_quant_int8(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), None, m, k, st))):
+        qb, q = window(m * k, torch.uint8, 0xAB)
+        sb, s = window(m, torch.float32, -7.0)
+        cases.append((name, fn(q, s), qb, m * k, 0xAB, sb, m, -7.0))
+    # per-tensor dynamic / static, static with the repeated scale
+    qb, q = window(m * k, torch.uint8, 0xAB)
+    sb, s = window(1, torch.float32, -7.0)
+    s.zero_()
+    rc = lib.sglq_per_tensor_quant_fp8(x.data_ptr(), 0, q.data_ptr(), s.data_ptr(), m * k, 0, st)
+    cases.append(("tensor dynamic", rc, qb, m * k, 0xAB, sb, 1, -7.0))
+    qb, q = window(m * k, torch.uint8, 0xAB)
+    sb, s = window(m, torch.float32, -7.0)
+    scale = torch.tensor([0.05], device=gpu)
+    rc = lib.sglq_static_quant_fp8(x.data_ptr(), 0, q.data_ptr(), scale.data_ptr(), s.data_ptr(), m, k, st)
+    cases.append(("static repeat", rc, qb, m * k, 0xAB, sb, m, -7.0))
+    torch.cuda.synchronize()
+    for name, rc, qb, qn, qfill, sb, sn, sfill in cases:
+        assert rc == 0, (name, lib.sglq_last_error())
+        assert guards_intact(qb, qn, qfill), f"{name}: codes written outside the output"
+        assert guards_intact(sb, sn, sfill), f"{name}: scales written outside the output"
+    assert scale.item() == torch.tensor(0.05).item()
