@@ -107,22 +107,24 @@ def cpu_baseline(m_sample):
     cores = torch.get_num_threads()
     flops = 0.0
     secs = 0.0
+    PASSES = 2  # about 16 s of host time on the 16 cores of a one-GPU box
     for i, (n, k) in enumerate(DSV3_NK):
         x = O.gen_activation(m_sample, k, seed=2000 + i)
         w = torch.randn((n, k), generator=torch.Generator().manual_seed(i)) * 0.02
         wq, ws = O.block_quant_weight(w)
         del w
-        t0 = time.perf_counter()
-        xq, xs = O.per_token_group_quant_fp8(x, 128)
-        O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
-        secs += time.perf_counter() - t0
-        flops += 2.0 * m_sample * n * k
+        for _ in range(PASSES):
+            t0 = time.perf_counter()
+            xq, xs = O.per_token_group_quant_fp8(x, 128)
+            O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+            secs += time.perf_counter() - t0
+            flops += 2.0 * m_sample * n * k
     return {
         "value": round(flops / secs / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"{m_sample} of 4096 activation rows of each of the 5 shapes, full weights, one pass, {secs:.1f} s of CPU time",
+        "sample": f"{m_sample} of 4096 activation rows of each of the 5 shapes, full weights, {PASSES} passes, {secs:.1f} s of CPU time",
     }
 
 
