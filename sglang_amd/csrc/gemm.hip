@@ -1056,11 +1056,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         if constexpr (BLOCK) {
           part = block_mfma<KIND>(bf[j], a_cur);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, acc[i][j], 0, 0, 0, 0, 0, 0);
+          // (a tile's first step starts from zero instead of clearing 128 registers beforehand)
+          const v4f c0 = first ? v4f{0.f, 0.f, 0.f, 0.f} : acc[i][j];
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, c0, 0, 0, 0, 0, 0, 0);
         } else {
           const v4i b0 = {bf[j][0], bf[j][1], bf[j][2], bf[j][3]};
           const v4i a0 = {a_cur[0], a_cur[1], a_cur[2], a_cur[3]};
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+          const v4i c0 = first ? v4i{0, 0, 0, 0} : acc[i][j];
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, c0, 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!IS_FP8 && !BLOCK) {
@@ -1097,10 +1100,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
             const float s_use = (pi == i) ? sc : sc_prev;
-            acc[pi][pj][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), s_use, acc[pi][pj][0]);
-            acc[pi][pj][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), s_use, acc[pi][pj][1]);
-            acc[pi][pj][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), s_use, acc[pi][pj][2]);
-            acc[pi][pj][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), s_use, acc[pi][pj][3]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[pi][pj][e] = first ? block_value<KIND>(part_prev[e]) * s_use
+                                     : __builtin_fmaf(block_value<KIND>(part_prev[e]), s_use, acc[pi][pj][e]);
           }
           part_prev = part;
         }
@@ -1109,10 +1112,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       a_cur = a_nxt;
     }
     if constexpr (BLOCK) {
-      acc[MI - 1][NI - 1][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc, acc[MI - 1][NI - 1][0]);
-      acc[MI - 1][NI - 1][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc, acc[MI - 1][NI - 1][1]);
-      acc[MI - 1][NI - 1][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc, acc[MI - 1][NI - 1][2]);
-      acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[MI - 1][NI - 1][e] = first ? block_value<KIND>(part_prev[e]) * sc
+                                       : __builtin_fmaf(block_value<KIND>(part_prev[e]), sc, acc[MI - 1][NI - 1][e]);
     }
   };
 
@@ -1169,11 +1172,6 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   }
 
   while (true) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
-
     // The block's next unit; past its last one the prefetches are pointed at rows beyond M
     // and N, which the buffer bounds turn into zero fill without memory traffic.
     const int next_unit = unit + (int)gridDim.x;
