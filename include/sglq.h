@@ -159,6 +159,41 @@ int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, const void*
                                          int64_t num_experts, int64_t total_m, int64_t N, int64_t K, void* workspace,
                                          int64_t workspace_bytes, void* stream);
 
+/* The data movement around the grouped GEMM in an MoE layer
+ * (python/sglang/srt/layers/moe/cutlass_moe.py:140-222).
+ *
+ * sglq_prepare_moe_input replaces torch.ops.sgl_kernel.prepare_moe_input
+ * (sgl-kernel/csrc/moe/prepare_moe_input.cu:13-166; schema common_extension.cc:199-203):
+ * topk_ids [topk_length] int32, slot i belonging to token i / topk; outputs
+ * expert_offsets [num_experts + 1], blockscale_offsets [num_experts + 1] or NULL (offsets of
+ * the counts rounded up to 128), problem_sizes1 [num_experts, 3] = (count, 2 n, k),
+ * problem_sizes2 = (count, k, n), input_permutation [topk_length] (expert-major position ->
+ * token) and output_permutation [topk_length] (slot -> expert-major position).  Positions
+ * inside an expert follow slot order (the reference's order depends on thread timing); ids
+ * outside [0, num_experts) are routed nowhere.  No scratch buffer is needed.
+ *
+ * sglq_shuffle_rows replaces shuffle_rows (prepare_moe_input.cu:168-244):
+ * output row d = input row dst2src_map[d], rows of row_bytes bytes, any element type.
+ *
+ * sglq_silu_and_mul replaces silu_and_mul (sgl-kernel/csrc/elementwise/activation.cu:57-60,
+ * 85-103): input [num_tokens, 2 d], output [num_tokens, d] = T(silu(x[:, :d])) * x[:, d:],
+ * T = dtype (SGLQ_BF16 or SGLQ_FP16); 16 bytes per lane when d is a multiple of 8 and the
+ * pointers are 16-byte aligned, one element per lane otherwise.
+ *
+ * sglq_apply_shuffle_mul_sum replaces apply_shuffle_mul_sum (prepare_moe_input.cu:258-392):
+ * output [m, row] = sum_j factors[i topk + j] * input[permutation[i topk + j]], fp32
+ * accumulation in j order; factors [m topk] in dtype or NULL (all ones); input has
+ * num_src_rows rows. */
+int sglq_prepare_moe_input(const int32_t* topk_ids, int32_t* expert_offsets, int32_t* blockscale_offsets,
+                           int32_t* problem_sizes1, int32_t* problem_sizes2, int32_t* input_permutation,
+                           int32_t* output_permutation, int64_t topk_length, int64_t topk, int64_t num_experts,
+                           int64_t n, int64_t k, void* stream);
+int sglq_shuffle_rows(const void* input, const int32_t* dst2src_map, void* output, int64_t num_src_rows,
+                      int64_t num_dst_rows, int64_t row_bytes, void* stream);
+int sglq_silu_and_mul(const void* input, int dtype, void* output, int64_t num_tokens, int64_t d, void* stream);
+int sglq_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors,
+                               int dtype, int64_t m, int64_t topk, int64_t row, int64_t num_src_rows, void* stream);
+
 /* Replaces w8a8_block_int8_matmul, a Triton kernel in the reference
  * (python/sglang/srt/layers/quantization/int8_kernel.py:212-425; there is no
  * sgl_kernel C++ op): out[m,n] = sum_kb float(sum_{k in block kb} a[m,k] b[k,n])

@@ -323,6 +323,87 @@ def fp8_blockwise_scaled_grouped_mm(
 
 
 # ---------------------------------------------------------------------------
+# The data movement around the grouped GEMM in an MoE layer
+# ---------------------------------------------------------------------------
+def prepare_moe_input(topk_ids: torch.Tensor, num_experts: int, n: int, k: int):
+    """sgl-kernel/csrc/moe/prepare_moe_input.cu:13-139.  Returns expert_offsets [E + 1],
+    blockscale_offsets [E + 1] (:56-76), problem_sizes1 = (count, 2 n, k), problem_sizes2 =
+    (count, k, n) (:31-38), input_permutation and output_permutation (:78-96).  The reference
+    orders the slots of one expert by thread arrival; any order is a valid result, this one keeps
+    slot order.  Slots whose id is outside [0, E) get output_permutation -1 here (the operator
+    leaves those entries untouched)."""
+    ids = topk_ids.reshape(-1).to(torch.int64)
+    topk = topk_ids.shape[1]
+    counts = torch.zeros(num_experts, dtype=torch.int64)
+    valid = (ids >= 0) & (ids < num_experts)
+    counts.scatter_add_(0, ids[valid], torch.ones_like(ids[valid]))
+    offsets = torch.zeros(num_experts + 1, dtype=torch.int64)
+    offsets[1:] = torch.cumsum(counts, 0)
+    rounded = torch.zeros(num_experts + 1, dtype=torch.int64)
+    rounded[1:] = torch.cumsum((counts + 127) // 128 * 128, 0)
+    ps1 = torch.stack([counts, torch.full_like(counts, 2 * n), torch.full_like(counts, k)], dim=1)
+    ps2 = torch.stack([counts, torch.full_like(counts, k), torch.full_like(counts, n)], dim=1)
+    a_map = torch.full((ids.numel(),), -1, dtype=torch.int64)
+    c_map = torch.full((ids.numel(),), -1, dtype=torch.int64)
+    nxt = offsets[:-1].clone()
+    for i in range(ids.numel()):
+        e = int(ids[i])
+        if 0 <= e < num_experts:
+            pos = int(nxt[e])
+            nxt[e] += 1
+            a_map[pos] = i // topk
+            c_map[i] = pos
+    to32 = lambda t: t.to(torch.int32)
+    return to32(offsets), to32(rounded), to32(ps1), to32(ps2), to32(a_map), to32(c_map)
+
+
+def shuffle_rows(x: torch.Tensor, dst2src_map: torch.Tensor) -> torch.Tensor:
+    """prepare_moe_input.cu:168-190: output[d] = input[dst2src_map[d]]."""
+    return x[dst2src_map.to(torch.int64)]
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """sgl-kernel/csrc/elementwise/activation.cu:57-60 with the act_and_mul kernel it instantiates
+    (:85-103): silu(v) = v / (1 + exp(-v)) in fp32, rounded to the tensor's type; then the product
+    with the second half, rounded again."""
+    d = x.shape[-1] // 2
+    v = x[..., :d].to(torch.float32)
+    act = (v / (1.0 + torch.exp(-v))).to(x.dtype)
+    return (act.to(torch.float32) * x[..., d:].to(torch.float32)).to(x.dtype)
+
+
+def apply_shuffle_mul_sum(c2: torch.Tensor, c_map: torch.Tensor, factors: Optional[torch.Tensor], m: int) -> torch.Tensor:
+    """prepare_moe_input.cu:258-318: output[i] = sum_j factors[i, j] * c2[c_map[i topk + j]],
+    fp32 accumulation in j order, one fused multiply-add per term (the product of two 16-bit
+    floats is exact in fp32, so multiply-then-add rounds the same way), rounded to the type."""
+    topk = c_map.numel() // m
+    acc = torch.zeros((m, c2.shape[1]), dtype=torch.float32)
+    cm = c_map.to(torch.int64).reshape(m, topk)
+    for j in range(topk):
+        f = torch.ones(m, dtype=torch.float32) if factors is None else factors.reshape(m, topk)[:, j].to(torch.float32)
+        routed = (cm[:, j] >= 0) & (cm[:, j] < c2.shape[0])  # other entries name no row and add nothing
+        term = f.unsqueeze(1) * c2[cm[:, j].clamp(0, max(c2.shape[0] - 1, 0))].to(torch.float32)
+        acc = torch.where(routed.unsqueeze(1), acc + term, acc)
+    return acc.to(c2.dtype)
+
+
+def cutlass_fused_experts_fp8(a, w1_q, w2_q, w1_scale, w2_scale, topk_weights, topk_ids) -> torch.Tensor:
+    """python/sglang/srt/layers/moe/cutlass_moe.py:140-222 as a sequence of the restatements above:
+    a [m, k]; w1_q [E, k, 2 n], w2_q [E, n, k] e4m3fn; w1_scale [E, k/128, 2 n/128], w2_scale
+    [E, n/128, k/128]; topk_weights / topk_ids [m, topk]."""
+    num_experts, k, n = w1_q.shape[0], w1_q.shape[1], w2_q.shape[1]
+    m, topk = topk_ids.shape
+    offsets, _, ps1, ps2, a_map, c_map = prepare_moe_input(topk_ids, num_experts, n, k)
+    a_q, a1_scale = per_token_group_quant_fp8(a, 128)
+    rep_a_q, rep_a1_scales = shuffle_rows(a_q, a_map), shuffle_rows(a1_scale, a_map)
+    c1 = fp8_blockwise_scaled_grouped_mm(rep_a_q, w1_q, rep_a1_scales, w1_scale, ps1, offsets[:-1], a.dtype)
+    inter = silu_and_mul(c1)
+    inter_q, a2_scale = per_token_group_quant_fp8(inter, 128)
+    c2 = fp8_blockwise_scaled_grouped_mm(inter_q, w2_q, a2_scale, w2_scale, ps2, offsets[:-1], a.dtype)
+    return apply_shuffle_mul_sum(c2, c_map, topk_weights.to(a.dtype), m)
+
+
+# ---------------------------------------------------------------------------
 # a5  INT8 scaled GEMM
 # ---------------------------------------------------------------------------
 def w8a8_block_int8_matmul(

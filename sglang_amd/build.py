@@ -16,7 +16,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libsglq.so"
-SOURCES = ["common.hip", "quant.hip", "gemm.hip"]
+SOURCES = ["common.hip", "quant.hip", "moe.hip", "gemm.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

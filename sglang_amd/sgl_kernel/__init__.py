@@ -11,10 +11,14 @@ from .gemm import (
     sgl_per_tensor_quant_fp8,
     sgl_per_token_quant_fp8,
 )
-from .moe import fp8_blockwise_scaled_grouped_mm
+from .moe import apply_shuffle_mul_sum, fp8_blockwise_scaled_grouped_mm, prepare_moe_input, shuffle_rows, silu_and_mul
 
 __all__ = [
+    "apply_shuffle_mul_sum",
     "fp8_blockwise_scaled_grouped_mm",
+    "prepare_moe_input",
+    "shuffle_rows",
+    "silu_and_mul",
     "fp8_blockwise_scaled_mm",
     "fp8_scaled_mm",
     "int8_mm_i32",

@@ -1,8 +1,12 @@
-"""Grouped (MoE) block-scaled FP8 GEMM behind the reference's operator name and argument list
-(sgl-kernel/python/sgl_kernel/moe.py:131-170, checks of
-sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:606-641)."""
+"""Grouped (MoE) block-scaled FP8 GEMM and the data-movement operators around it, behind the
+reference's operator names and argument lists (sgl-kernel/python/sgl_kernel/moe.py:131-205,
+sgl-kernel/python/sgl_kernel/gemm.py:281-288, sgl-kernel/python/sgl_kernel/elementwise.py:171-183;
+checks of sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:606-641 and
+sgl-kernel/csrc/moe/prepare_moe_input.cu)."""
 
 from __future__ import annotations
+
+from typing import Optional
 
 import torch
 
@@ -94,3 +98,107 @@ def fp8_blockwise_scaled_grouped_mm(
         problem_sizes.data_ptr(), expert_offsets.data_ptr(), num_experts, total_m, n, k,
         workspace.data_ptr(), workspace.numel() * workspace.element_size(), _lib.stream_ptr(a.device))
     _lib.check(rc, "fp8_blockwise_scaled_grouped_mm")
+
+
+def _cuda_int32(name, t):
+    _check(t.is_cuda, f"{name} must be a CUDA tensor")
+    _check(t.dtype == torch.int32, f"{name} must be int32")
+    _check(t.is_contiguous(), f"{name} must be contiguous")
+
+
+def prepare_moe_input(
+    topk_ids,
+    expert_offsets,
+    problem_sizes1,
+    problem_sizes2,
+    input_permutation,
+    output_permutation,
+    num_experts,
+    n,
+    k,
+    blockscale_offsets: Optional[torch.Tensor] = None,
+):
+    """Routing tables from the top-k expert ids (sgl-kernel/python/sgl_kernel/moe.py:173-196):
+    fills expert_offsets [E + 1], problem_sizes1/2 [E, 3], input_permutation (a_map) and
+    output_permutation (c_map), both [m * topk], and blockscale_offsets [E + 1] if given."""
+    _check(topk_ids.dtype == torch.int32, "topk_ids must be int32")  # prepare_moe_input.cu:153
+    for name, t in (("topk_ids", topk_ids), ("expert_offsets", expert_offsets), ("problem_sizes1", problem_sizes1),
+                    ("problem_sizes2", problem_sizes2), ("input_permutation", input_permutation),
+                    ("output_permutation", output_permutation)):
+        _cuda_int32(name, t)
+    _check(topk_ids.dim() == 2, "topk_ids must be a [num_tokens, topk] tensor")
+    _check(expert_offsets.numel() >= num_experts + 1, "expert_offsets must hold num_experts + 1 entries")
+    _check(problem_sizes1.numel() >= 3 * num_experts and problem_sizes2.numel() >= 3 * num_experts,
+           "problem_sizes must have shape (num_experts, 3)")
+    _check(input_permutation.numel() >= topk_ids.numel() and output_permutation.numel() >= topk_ids.numel(),
+           "the permutations must hold one entry per element of topk_ids")
+    if blockscale_offsets is not None:
+        _cuda_int32("blockscale_offsets", blockscale_offsets)
+        _check(blockscale_offsets.numel() >= num_experts + 1, "blockscale_offsets must hold num_experts + 1 entries")
+    rc = _lib.load().sglq_prepare_moe_input(
+        topk_ids.data_ptr(), expert_offsets.data_ptr(), None if blockscale_offsets is None else blockscale_offsets.data_ptr(),
+        problem_sizes1.data_ptr(), problem_sizes2.data_ptr(), input_permutation.data_ptr(), output_permutation.data_ptr(),
+        topk_ids.numel(), max(topk_ids.size(1), 1), int(num_experts), int(n), int(k), _lib.stream_ptr(topk_ids.device))
+    _lib.check(rc, "prepare_moe_input")
+
+
+def shuffle_rows(input_tensor, dst2src_map, output_tensor_shape):
+    """output[d] = input[dst2src_map[d]] (sgl-kernel/python/sgl_kernel/gemm.py:281-288)."""
+    _check(input_tensor.is_cuda and dst2src_map.is_cuda, "input and dst2src_map must be CUDA tensors")
+    _check(input_tensor.dim() == 2 and input_tensor.is_contiguous(), "input must be a contiguous 2D tensor")
+    _check(dst2src_map.dtype == torch.int32 and dst2src_map.is_contiguous(), "dst2src_map must be a contiguous int32 tensor")
+    output_tensor = torch.empty(output_tensor_shape, device=input_tensor.device, dtype=input_tensor.dtype)
+    _check(output_tensor.dim() == 2 and output_tensor.size(1) == input_tensor.size(1), "output rows must have the input's length")
+    _check(dst2src_map.numel() >= output_tensor.size(0), "dst2src_map must hold one entry per output row")
+    rc = _lib.load().sglq_shuffle_rows(
+        input_tensor.data_ptr(), dst2src_map.data_ptr(), output_tensor.data_ptr(), input_tensor.size(0), output_tensor.size(0),
+        input_tensor.size(1) * input_tensor.element_size(), _lib.stream_ptr(input_tensor.device))
+    _lib.check(rc, "shuffle_rows")
+    return output_tensor
+
+
+def apply_shuffle_mul_sum(input, output, permutation, factors):
+    """output[i] = sum_j factors[i, j] * input[permutation[i * topk + j]]
+    (sgl-kernel/python/sgl_kernel/moe.py:199-207; checks of prepare_moe_input.cu:320-345)."""
+    _check(input.dim() == 2, "input_tensor must be 2D [m * topk, row_stride]")
+    _check(output.dim() == 2, "output_tensor must be 2D [m, row_stride]")
+    _check(permutation.dim() == 1, "permutation must be 1D [m * topk]")
+    _check(input.is_cuda and output.is_cuda and permutation.is_cuda, "tensors must be CUDA tensors")
+    _check(input.is_contiguous() and output.is_contiguous() and permutation.is_contiguous(), "tensors must be contiguous")
+    _check(output.dtype in (torch.bfloat16, torch.float16) and input.dtype == output.dtype, "input and output must be Half or BFloat16")
+    _check(permutation.dtype == torch.int32, "permutation must be int32")
+    m, row = output.shape
+    _check(input.size(1) == row, "input and output rows must have the same length")
+    if m == 0:
+        return
+    topk = permutation.size(0) // m
+    _check(permutation.size(0) == m * topk and topk > 0, "permutation size must match m * topk")
+    f_ptr = None
+    if factors is not None:
+        _check(factors.dtype == output.dtype, "Factors must match output dtype")
+        _check(factors.numel() == m * topk, "Factors must have shape [m * topk]")
+        _check(factors.is_cuda and factors.is_contiguous(), "factors must be a contiguous CUDA tensor")
+        f_ptr = factors.data_ptr()
+    rc = _lib.load().sglq_apply_shuffle_mul_sum(
+        input.data_ptr(), output.data_ptr(), permutation.data_ptr(), f_ptr, DTYPE_CODE[output.dtype], m, topk, row, input.size(0),
+        _lib.stream_ptr(input.device))
+    _lib.check(rc, "apply_shuffle_mul_sum")
+
+
+def silu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """out = silu(input[..., :d]) * input[..., d:] (sgl-kernel/python/sgl_kernel/elementwise.py:171-183)."""
+    if input.shape[-1] * input.element_size() % 16 != 0:
+        raise ValueError("The pointers must be multiple of 16 bytes.")
+    d = input.shape[-1] // 2
+    if out is not None:
+        assert input.ndim == out.ndim and input.shape[:-1] == out.shape[:-1] and input.shape[-1] == 2 * out.shape[-1]
+    else:
+        out = torch.empty(input.shape[:-1] + (d,), device=input.device, dtype=input.dtype)
+    _check(input.is_cuda and out.is_cuda, "input and out must be CUDA tensors")
+    _check(input.is_contiguous() and out.is_contiguous(), "input and out must be contiguous")
+    if input.dtype not in (torch.bfloat16, torch.float16) or out.dtype != input.dtype:
+        raise NotImplementedError("silu_and_mul: Half and BFloat16 are built")
+    tokens = input.numel() // input.shape[-1] if input.numel() else 0
+    rc = _lib.load().sglq_silu_and_mul(input.data_ptr(), DTYPE_CODE[input.dtype], out.data_ptr(), tokens, d, _lib.stream_ptr(input.device))
+    _lib.check(rc, "silu_and_mul")
+    return out

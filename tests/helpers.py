@@ -107,3 +107,24 @@ def calc_diff(x, y):
     # the reference test's criterion (sgl-kernel/tests/test_fp8_blockwise_moe.py:29-33)
     x, y = x.double(), y.double()
     return float(1 - 2 * (x * y).sum() / (x * x + y * y).sum())
+
+
+def moe_layer_case(m, topk, num_experts, n, k, seed, dtype=torch.bfloat16, w_std=0.1):
+    """One MoE expert layer's inputs in the layout python/sglang/srt/layers/moe/cutlass_moe.py:30-139
+    documents: x [m, k]; w1_q [E, k, 2 n] and w2_q [E, n, k] e4m3fn (transposed views of the
+    [E, 2 n, k] / [E, k, n] weights, quantized per 128 x 128 block); w1_s [E, k/128, 2 n/128] and
+    w2_s [E, n/128, k/128]; distinct expert ids per token and softmax weights."""
+    from oracle import w8a8_oracle as O
+
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((m, k), generator=g).to(dtype)
+    w1 = torch.randn((num_experts, 2 * n, k), generator=g) * w_std
+    w2 = torch.randn((num_experts, k, n), generator=g) * w_std
+    q = lambda w: [O.block_quant_weight(w[i]) for i in range(w.shape[0])]
+    w1q, w2q = q(w1), q(w2)
+    ids = torch.stack([torch.randperm(num_experts, generator=g)[:topk] for _ in range(m)]).to(torch.int32).reshape(m, topk)
+    tw = torch.softmax(torch.rand((m, topk), generator=g), dim=-1)
+    return dict(
+        x=x, ids=ids, tw=tw,
+        w1_q=torch.stack([t[0] for t in w1q]).transpose(1, 2), w1_s=torch.stack([t[1] for t in w1q]).transpose(1, 2),
+        w2_q=torch.stack([t[0] for t in w2q]).transpose(1, 2), w2_s=torch.stack([t[1] for t in w2q]).transpose(1, 2))

@@ -184,5 +184,19 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert grouped(128, 4096, 2) == 1 and b"bfloat16 or half" in lib.sglq_last_error()
     assert lib.sglq_fp8_blockwise_scaled_grouped_mm(p, 128, p, 128, 2048, p, 1, 1, p, 1, 1, 1, p, 16, 0, p, p, 0, 32, 16, 128, p, 4096,
                                                     None) == 0  # no experts
+    # the operators around the grouped GEMM
+    assert lib.sglq_prepare_moe_input(p, p, None, p, p, p, p, 8, 0, 4, 128, 128, None) == 1 and b"bad sizes" in lib.sglq_last_error()
+    assert lib.sglq_prepare_moe_input(p, None, None, p, p, p, p, 8, 2, 4, 128, 128, None) == 1 and b"null" in lib.sglq_last_error()
+    assert lib.sglq_prepare_moe_input(p, p, None, p, p, p, p, 8, 2, 0, 128, 128, None) == 0  # no experts
+    assert lib.sglq_shuffle_rows(p, p, p, 4, -1, 16, None) == 1 and b"negative" in lib.sglq_last_error()
+    assert lib.sglq_shuffle_rows(p, None, p, 4, 4, 16, None) == 1 and b"null" in lib.sglq_last_error()
+    assert lib.sglq_shuffle_rows(p, p, p, 4, 0, 16, None) == 0
+    assert lib.sglq_silu_and_mul(p, 2, p, 4, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
+    assert lib.sglq_silu_and_mul(None, 0, p, 4, 8, None) == 1 and b"null" in lib.sglq_last_error()
+    assert lib.sglq_silu_and_mul(p, 0, p, 0, 8, None) == 0
+    assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 0, 8, 8, None) == 1 and b"bad sizes" in lib.sglq_last_error()
+    assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 2, 12, 8, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
+    assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 2, 4, 2, 8, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
+    assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 0, 2, 8, 8, None) == 0
     # empty problems are a no-op
     assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0

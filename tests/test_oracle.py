@@ -395,6 +395,92 @@ def test_grouped_mm_oracle_reduces_to_dense_and_leaves_gaps():
     assert float(out[16:20].abs().max()) == 0.0 and float(out[25:32].abs().max()) == 0.0 and float(out[40:].abs().max()) == 0.0
 
 
+def test_moe_routing_tables_from_their_definition():
+    """prepare_moe_input (prepare_moe_input.cu:13-139): counts are a histogram, offsets their
+    running sums (and those of the counts rounded up to 128), every routed slot owns exactly one
+    expert-major position inside its expert's range, and the two permutations invert each other."""
+    g = torch.Generator().manual_seed(8)
+    m, topk, e, n, k = 37, 4, 9, 256, 512
+    ids = torch.randint(0, e, (m, topk), generator=g, dtype=torch.int32)
+    ids[3, 1] = -1  # routed nowhere
+    ids[5, 0] = e   # out of range as well
+    offsets, rounded, ps1, ps2, a_map, c_map = O.prepare_moe_input(ids, e, n, k)
+    flat = ids.reshape(-1).long()
+    hist = torch.bincount(flat[(flat >= 0) & (flat < e)], minlength=e)
+    assert torch.equal(ps1[:, 0].long(), hist) and torch.equal(ps2[:, 0].long(), hist)
+    assert ps1[:, 1].unique().tolist() == [2 * n] and ps1[:, 2].unique().tolist() == [k]
+    assert ps2[:, 1].unique().tolist() == [k] and ps2[:, 2].unique().tolist() == [n]
+    assert offsets.tolist() == [0] + torch.cumsum(hist, 0).tolist()
+    assert rounded.tolist() == [0] + torch.cumsum((hist + 127) // 128 * 128, 0).tolist()
+    routed = (flat >= 0) & (flat < e)
+    pos = c_map[routed].long()
+    assert sorted(pos.tolist()) == list(range(int(hist.sum())))  # a bijection onto the used positions
+    for i in routed.nonzero().flatten().tolist():
+        ex, p = int(flat[i]), int(c_map[i])
+        assert offsets[ex] <= p < offsets[ex + 1] and int(a_map[p]) == i // topk
+    assert c_map[~routed].tolist() == [-1, -1]
+    # slot order is kept inside an expert
+    for ex in range(e):
+        mine = c_map[(flat == ex)].tolist()
+        assert mine == sorted(mine)
+
+
+def test_moe_combine_and_activation_from_their_definitions():
+    g = torch.Generator().manual_seed(9)
+    m, topk, row = 11, 3, 64
+    c2 = torch.randn((m * topk, row), generator=g).to(torch.bfloat16)
+    c_map = torch.randperm(m * topk, generator=g).to(torch.int32)
+    w = torch.softmax(torch.rand((m, topk), generator=g), dim=-1).to(torch.bfloat16)
+    out = O.apply_shuffle_mul_sum(c2, c_map, w, m)
+    # the reference's own description of the operator (prepare_moe_input.cu:368-373), in float64
+    want = (c2[c_map.long()].view(m, topk, row).double() * w.view(m, topk, 1).double()).sum(dim=1)
+    torch.testing.assert_close(out.double(), want, rtol=2 ** -8, atol=1e-6)
+    assert torch.equal(O.apply_shuffle_mul_sum(c2, c_map, None, m), O.apply_shuffle_mul_sum(c2, c_map, torch.ones_like(w), m))
+    # silu_and_mul: x * sigmoid(x) times the gate, two roundings to the 16-bit type
+    x = (torch.randn((5, 96), generator=g) * 3).to(torch.bfloat16)
+    got = O.silu_and_mul(x)
+    silu = torch.nn.functional.silu(x[:, :48].double())
+    want = silu.to(torch.bfloat16).double() * x[:, 48:].double()
+    torch.testing.assert_close(got.double(), want, rtol=2 ** -8, atol=1e-30)
+    assert O.silu_and_mul(torch.zeros((1, 16), dtype=torch.float16)).abs().max().item() == 0.0
+    assert torch.equal(O.shuffle_rows(c2, torch.tensor([2, 2, 0], dtype=torch.int32)), c2[[2, 2, 0]])
+
+
+def test_moe_layer_oracle_vs_dequantized_float_reference():
+    """The whole expert layer against the same layer computed in float64 on dequantized weights
+    and unquantized activations.  The reference's check has the form max |err| / max(|ref|, c) < 0.5
+    (python/sglang/test/test_cutlass_moe.py:241-254, c = 1e-2 on outputs of the order of 1e-7);
+    here c is the outputs' root mean square, plus bounds on the mean and the largest error that
+    FP8 quantization of activations and weights explains (a few per cent)."""
+    g = torch.Generator().manual_seed(10)
+    m, topk, e, n, k = 24, 2, 4, 128, 256
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    w1 = torch.randn((e, 2 * n, k), generator=g) * 0.1
+    w2 = torch.randn((e, k, n), generator=g) * 0.1
+    q = lambda w: [O.block_quant_weight(w[i]) for i in range(w.shape[0])]
+    w1q, w2q = q(w1), q(w2)
+    w1_q = torch.stack([t[0] for t in w1q]).transpose(1, 2)       # [E, k, 2n]
+    w1_s = torch.stack([t[1] for t in w1q]).transpose(1, 2)       # [E, k/128, 2n/128]
+    w2_q = torch.stack([t[0] for t in w2q]).transpose(1, 2)       # [E, n, k]
+    w2_s = torch.stack([t[1] for t in w2q]).transpose(1, 2)       # [E, n/128, k/128]
+    ids = torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+    tw = torch.softmax(torch.rand((m, topk), generator=g), dim=-1).to(torch.bfloat16)
+    out = O.cutlass_fused_experts_fp8(x, w1_q, w2_q, w1_s, w2_s, tw, ids)
+    deq = lambda wq, ws: wq.float().double() * ws.double().repeat_interleave(128, 0).repeat_interleave(128, 1)[: wq.shape[0], : wq.shape[1]]
+    ref = torch.zeros((m, k), dtype=torch.float64)
+    for t in range(m):
+        for j in range(topk):
+            ex = int(ids[t, j])
+            h = deq(*w1q[ex]) @ x[t].double()
+            act = torch.nn.functional.silu(h[:n]) * h[n:]
+            ref[t] += tw[t, j].double() * (deq(*w2q[ex]) @ act)
+    err = (out.double() - ref).abs()
+    rms = float(ref.pow(2).mean().sqrt())
+    print("moe layer oracle: rms", rms, "mean err", float(err.mean()), "max err", float(err.max()))
+    assert float((err / ref.abs().clamp(min=rms)).max()) < 0.5  # the reference's form, clamped at the outputs' scale
+    assert float(err.mean()) < 0.04 * rms and float(err.max()) < 0.25 * rms
+
+
 def test_block_int8_mm_pins(c_oracle):
     """w8a8_block_int8_matmul: unit scales reduce to the exact integer product, one-hot rows select
     scaled weight rows, a double-precision C brute force on N % 128 != 0 and K % 128 != 0, and the
