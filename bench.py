@@ -437,6 +437,60 @@ def run_sweep(args):
                      gemm_GBs=round(nbytes / tg / 1e6, 1), gemm_frac_hbm=round(nbytes / tg / 1e6 / PEAK_HBM_GBS, 4))
             del b
             torch.cuda.empty_cache()
+    # the whole expert layer (routing tables, gathers, two grouped GEMMs, SiLU-and-multiply, quantization, combine) on
+    # DeepSeek-V3's expert shape, 32 local experts, top-8 routing among them: per-step device times and the layer's
+    if want("moe_layer"):
+        from sglang_amd.moe.cutlass_moe import cutlass_fused_experts_fp8
+        from sglang_amd.sgl_kernel import apply_shuffle_mul_sum, prepare_moe_input, shuffle_rows, silu_and_mul
+
+        e, k, n, topk = 32, 7168, 2048, 8
+        g = torch.Generator(device=dev).manual_seed(6000)
+        w1 = (torch.randn((e, 2 * n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn).transpose(1, 2)
+        w2 = (torch.randn((e, k, n), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn).transpose(1, 2)
+        s1 = torch.rand((e, k // 128, 2 * n // 128), generator=g, device=dev) * 1e-3 + 1e-4
+        s2 = torch.rand((e, n // 128, k // 128), generator=g, device=dev) * 1e-3 + 1e-4
+        i64 = torch.empty((e,), dtype=torch.int64, device=dev)
+        lay = torch.zeros((e, 5), dtype=torch.int32, device=dev)
+        ws = torch.empty((1 << 20,), dtype=torch.uint8, device=dev)
+        offs = torch.empty((e + 1,), dtype=torch.int32, device=dev)
+        ps1, ps2 = torch.empty((e, 3), dtype=torch.int32, device=dev), torch.empty((e, 3), dtype=torch.int32, device=dev)
+        for m in (16, 512, 4096):
+            x = make_activation(m, k, 6000 + m, dev)
+            ids = torch.rand((m, e), generator=g, device=dev).argsort(dim=1)[:, :topk].to(torch.int32).contiguous()
+            tw = torch.softmax(torch.rand((m, topk), generator=g, device=dev), dim=-1)
+            rows = m * topk
+            a_map = torch.empty((rows,), dtype=torch.int32, device=dev)
+            c_map = torch.empty((rows,), dtype=torch.int32, device=dev)
+            iters = max(2, args.iters // 4)
+            t = {}
+            t["prepare"] = time_kernel(lambda j: prepare_moe_input(ids, offs, ps1, ps2, a_map, c_map, e, n, k), iters)
+            t["quant1"] = time_kernel(lambda j: sglang_per_token_group_quant_fp8(x, 128), iters)
+            a_q, a_s = sglang_per_token_group_quant_fp8(x, 128)
+            t["gather_codes"] = time_kernel(lambda j: shuffle_rows(a_q, a_map, (rows, k)), iters)
+            t["gather_scales"] = time_kernel(lambda j: shuffle_rows(a_s, a_map, (rows, k // 128)), iters)
+            rq, rs = shuffle_rows(a_q, a_map, (rows, k)), shuffle_rows(a_s, a_map, (rows, k // 128))
+            c1 = torch.empty((rows, 2 * n), dtype=torch.bfloat16, device=dev)
+            c2 = torch.empty((rows, k), dtype=torch.bfloat16, device=dev)
+            gmm = lambda out, a, b, sa, sb, ps: fp8_blockwise_scaled_grouped_mm(out, i64, i64, i64, i64, i64, a, b, sa, sb, i64, i64, i64,
+                                                                                lay, lay, ps, offs[:-1], ws)
+            t["gemm1"] = time_kernel(lambda j: gmm(c1, rq, w1, rs, s1, ps1), iters)
+            t["silu_and_mul"] = time_kernel(lambda j: silu_and_mul(c1), iters)
+            inter = silu_and_mul(c1)
+            t["quant2"] = time_kernel(lambda j: sglang_per_token_group_quant_fp8(inter, 128), iters)
+            iq, isc = sglang_per_token_group_quant_fp8(inter, 128)
+            t["gemm2"] = time_kernel(lambda j: gmm(c2, iq, w2, isc, s2, ps2), iters)
+            res = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+            twb = tw.to(torch.bfloat16)
+            t["combine"] = time_kernel(lambda j: apply_shuffle_mul_sum(c2, res, c_map, twb), iters)
+            layer = time_kernel(lambda j: cutlass_fused_experts_fp8(x, w1, w2, s1, s2, tw, ids, i64, i64, i64, i64, ws, i64, i64, i64, i64,
+                                                                    i64, offs, ps1, ps2), iters)
+            fl = 2.0 * rows * (2 * n * k + n * k)
+            moved = {"gather_codes": 2 * rows * k, "gather_scales": 8 * rows * (k // 128), "silu_and_mul": 6 * rows * n,
+                     "quant1": group_quant_bytes(m, k), "quant2": group_quant_bytes(rows, n), "combine": 2 * rows * k + 2 * m * k}
+            emit(cfg="moe_layer", op="cutlass_fused_experts_fp8", experts=e, topk=topk, M=m, hidden=k, intermediate=n,
+                 layer_us=round(layer * 1e3, 1), layer_TFLOPs=round(fl / layer / 1e9, 2),
+                 steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(t.values()) * 1e3, 1),
+                 steps_GBs={s: round(b / t[s] / 1e6, 1) for s, b in moved.items()})
     f.close()
 
 
@@ -452,7 +506,7 @@ def main():
     ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--sweep-only", type=str, default=None,
-                    help="with --sweep: comma-separated configurations to run (0, 1, 2, 3, 4, moe); default all")
+                    help="with --sweep: comma-separated configurations to run (0, 1, 2, 3, 4, moe, moe_layer); default all")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is measured on one GPU only (it needs no exchange between GPUs; "

@@ -255,7 +255,8 @@ void sglq_debug_force_tile(int tile);
  * with sglq_debug_force_tile(64 / 128 / 256): 64 = always the M <= 64 kernel where it applies. */
 void sglq_debug_force_splits(int splits);
 /* Test hook: fixes the grouped GEMM's row tile height (32, 64, 128: the 128-row kernel; 256: the
- * pipelined 256-row kernel); anything else restores the choice from the average group size. */
+ * pipelined 256-row kernel; 130: the pipelined kernel with 128-row tiles); anything else restores
+ * the choice from the average group size. */
 void sglq_debug_grouped_tile(int rows);
 /* Test and measurement hook: name of the GEMM kernel that the calling thread's last GEMM
  * call launched ("" before the first call); the string is static. */

@@ -1920,7 +1920,7 @@ static int num_cus() {
 }
 
 static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
-static int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile (0 = from the average group)
+static int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile, 130 = 128 rows pipelined (0 = from the average group)
 static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
 
 template <int KIND, int OUT_DT>
@@ -2322,7 +2322,9 @@ using namespace sglq;
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
-extern "C" void sglq_debug_grouped_tile(int rows) { g_grouped_tile = (rows == 32 || rows == 64 || rows == 128 || rows == 256) ? rows : 0; }
+extern "C" void sglq_debug_grouped_tile(int rows) {
+  g_grouped_tile = (rows == 32 || rows == 64 || rows == 128 || rows == 130 || rows == 256) ? rows : 0;
+}
 extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel; }
 
 template <int KIND>
@@ -2412,15 +2414,25 @@ extern "C" int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, 
   }
   // Row tile height from the average group: the experts' row counts are device data.
   // Measured with 256 experts of 4096 x 7168 (one launch streams every expert's weight once,
-  // 7.5 GB): 64-row tiles are fastest below about 12 rows per expert (1.27-1.31 ms, 5.7-5.9
-  // TB/s), 128-row tiles up to about 64 (1.47-2.19 ms), and from there the pipelined 256-row
-  // kernel even with its tiles partly empty (2.2-2.3 ms whatever the fill, against 3.0 ms for
-  // 128-row tiles at 96 rows per expert).
+  // 7.5 GB) and equal groups: below about 12 rows per expert the 128-row kernel's 64-row tiles
+  // are fastest (1.30-1.32 ms, 5.7-5.8 TB/s, against 1.43-1.45 ms); from there to 128 rows per
+  // expert the pipelined kernel with 128-row tiles (1.46 ms at 16 rows, 1.57 ms at 64, 1.76 ms
+  // at 128, where the unpipelined 128-row tiles need 1.48, 2.23 and 3.99 ms and the pipelined
+  // 256-row ones 2.1-2.2 ms whatever their fill); above 128 rows per expert two 128-row tiles
+  // cost what one 256-row tile costs and the 256-row tile computes faster (2.26 against
+  // 2.51 ms at 256 rows, 7.7 against 8.1 ms at 1024).
   const int64_t avg = total_m / num_experts;
-  const bool pipelined = g_grouped_tile == 256 || (g_grouped_tile == 0 && avg >= 64 && K >= 384);
-  const int bm = g_grouped_tile ? g_grouped_tile : pipelined ? 256 : avg < 12 ? 64 : 128;
-  if (g_grouped_tile == 256 && K < 384) {
-    set_error("%s: the 256-row kernel needs K >= 384", name);
+  bool pipelined;
+  int bm;
+  if (g_grouped_tile) {  // test hook; 130 = the pipelined kernel with 128-row tiles
+    pipelined = g_grouped_tile == 256 || g_grouped_tile == 130;
+    bm = g_grouped_tile == 130 ? 128 : g_grouped_tile;
+  } else {
+    pipelined = avg >= 12 && K >= 384;
+    bm = pipelined ? (avg > 128 ? 256 : 128) : avg < 12 ? 64 : 128;
+  }
+  if (pipelined && K < 384) {
+    set_error("%s: the pipelined kernel needs K >= 384", name);
     return SGLQ_EINVAL;
   }
   const int64_t max_tiles = total_m / bm + num_experts;
@@ -2449,15 +2461,20 @@ extern "C" int sglq_fp8_blockwise_scaled_grouped_mm(const void* a, int64_t lda, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   grouped_plan_kernel<<<dim3(1), dim3(256), 0, st>>>(problem_sizes, expert_offsets, (int)num_experts, (int)total_m, bm,
                                                      (int)max_tiles, static_cast<int*>(workspace));
-  if (bm == 256) {
-    g_last_kernel = "grouped_plan_kernel+gemm_pipe_kernel<grouped>";
+  if (pipelined) {
+    g_last_kernel = bm == 256 ? "grouped_plan_kernel+gemm_pipe_kernel<grouped>" : "grouped_plan_kernel+gemm_pipe_kernel<grouped, 128 rows>";
     p.tiles_m = (int)max_tiles;
     p.tiles_n = (int)((N + 255) / 256);
     p.splits = 1;
     const int64_t units = max_tiles * p.tiles_n;
     const dim3 grid((uint32_t)(units < num_cus() ? units : num_cus())), block(512);
-    if (out_dtype == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_BF16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
-    else gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_FP16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
+    if (bm == 256) {
+      if (out_dtype == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_BF16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
+      else gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_FP16, PIPE_GROUPED><<<grid, block, 0, st>>>(p);
+    } else {
+      if (out_dtype == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_BF16, PIPE_GROUPED, 128><<<grid, block, 0, st>>>(p);
+      else gemm_pipe_kernel<KIND_FP8_BLOCK, SGLQ_FP16, PIPE_GROUPED, 128><<<grid, block, 0, st>>>(p);
+    }
     return finish(name);
   }
   g_last_kernel = "grouped_plan_kernel+gemm_kernel<grouped>";

@@ -17,8 +17,8 @@ def say(*a):
     print(*a, flush=True)
 
 
-# the row tile: chosen from the average group, the 128-row kernel's tiles, the pipelined 256-row kernel
-@pytest.fixture(params=[0, 32, 64, 128, 256], ids=["rows_auto", "rows32", "rows64", "rows128", "rows256"])
+# the row tile: chosen from the average group, the 128-row kernel's tiles, the pipelined kernel with 128 and 256 rows
+@pytest.fixture(params=[0, 32, 64, 128, 130, 256], ids=["rows_auto", "rows32", "rows64", "rows128", "rows128_pipelined", "rows256"])
 def gtile(request):
     from sglang_amd import _lib
 
@@ -117,11 +117,12 @@ def test_grouped_mm_gaps_order_and_scale_strides(gpu, gtile):
     assert bool((out[~owned] == SENTINEL).all())
 
 
-@pytest.mark.parametrize("rows_per_tile", [128, 256])
+@pytest.mark.parametrize("rows_per_tile", [128, 130, 256])
 def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu, rows_per_tile):
     """DeepSeek-V3-shaped expert GEMM (N = 4096, K = 7168, 32 experts, 8192 routed rows): every
     expert's rows equal the dense operator's result on that expert with the same kernel (the
-    128 x 128 one, the pipelined 256 x 256 one) and no split-K, bit for bit (same summation order)."""
+    128 x 128 one, the pipelined one with 128 x 256 and 256 x 256 tiles) and no split-K, bit for bit (same
+    summation order)."""
     from sglang_amd import _lib
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
@@ -145,9 +146,10 @@ def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu, rows_per_tile):
         out = run_grouped(gpu, c, torch.bfloat16)
     finally:
         lib.sglq_debug_grouped_tile(0)
-    want_kernel = "grouped_plan_kernel+gemm_kernel<grouped>" if rows_per_tile == 128 else "grouped_plan_kernel+gemm_pipe_kernel<grouped>"
+    want_kernel = {128: "grouped_plan_kernel+gemm_kernel<grouped>", 130: "grouped_plan_kernel+gemm_pipe_kernel<grouped, 128 rows>",
+                   256: "grouped_plan_kernel+gemm_pipe_kernel<grouped>"}[rows_per_tile]
     assert lib.sglq_debug_last_gemm_kernel().decode() == want_kernel
-    lib.sglq_debug_force_tile(128 if rows_per_tile == 128 else 258)
+    lib.sglq_debug_force_tile({128: 128, 130: 130, 256: 258}[rows_per_tile])
     lib.sglq_debug_force_splits(1)
     try:
         for x in (0, 5, 17, 31):
@@ -156,7 +158,8 @@ def test_grouped_mm_matches_dense_operator_bit_for_bit(gpu, rows_per_tile):
             sl = slice(int(cuts[x]), int(cuts[x + 1]))
             sa_cm = sa[sl].t().contiguous().t()  # the dense operator takes M-major activation scales
             dense = fp8_blockwise_scaled_mm(a[sl], b[x].t(), sa_cm, sb[x].t().contiguous().t(), torch.bfloat16)  # K-major weight scales
-            assert lib.sglq_debug_last_gemm_kernel().decode() == ("gemm_kernel" if rows_per_tile == 128 else "gemm_pipe_kernel")
+            assert lib.sglq_debug_last_gemm_kernel().decode() == {128: "gemm_kernel", 130: "gemm_pipe_kernel<128 rows>",
+                                                                  256: "gemm_pipe_kernel"}[rows_per_tile]
             assert torch.equal(out[sl].view(torch.int16), dense.view(torch.int16)), x
     finally:
         lib.sglq_debug_force_tile(0)
