@@ -26,21 +26,48 @@ static int check_moe_launch(const char* what) {
 // threads arrive; here slots keep their order (position = number of earlier slots of the same
 // expert), so the tables are the same on every run.  Ids outside [0, E) belong to nobody: their
 // output_permutation entries are left as they are, as in the reference.
-// One block per expert; the counts of every expert must be known before any offset, hence
-// three launches: count, offsets (one thread block scanning E values), place.
+// The counts of every expert must be known before any offset, hence three launches: count
+// (one block per expert), offsets (one block scanning E values), place.  A thread looks at
+// four consecutive slots at a time, a block of 1024 threads at 4096.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void moe_count_kernel(const int* __restrict__ topk_ids, int* __restrict__ ps1,
-                                                        int* __restrict__ ps2, int64_t topk_length, int n, int k) {
-  __shared__ int red[4];
-  const int e = blockIdx.x;
+constexpr int MOE_THREADS = 1024, MOE_SWEEP = 4 * MOE_THREADS;
+
+// Slots i .. i + 3; slots past the end read as -1, which is nobody's id.
+SGLQ_DEV v4i load_ids4(const int* __restrict__ ids, int64_t i, int64_t n, bool aligned) {
+  if (aligned && i + 3 < n) return *reinterpret_cast<const v4i*>(ids + i);
+  v4i v = {-1, -1, -1, -1};
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    if (i + q < n) v[q] = ids[i + q];
+  return v;
+}
+
+// Number of slots in [0, end) that name expert e; every thread of the block gets the sum.
+SGLQ_DEV int block_count_ids(const int* __restrict__ ids, int64_t end, int e, bool aligned, int* red) {
   int c = 0;
-  for (int64_t i = threadIdx.x; i < topk_length; i += 256) c += topk_ids[i] == e;
+#pragma unroll 4
+  for (int64_t i = 4 * (int64_t)threadIdx.x; i < end; i += MOE_SWEEP) {
+    const v4i v = load_ids4(ids, i, end, aligned);
+    c += (v[0] == e) + (v[1] == e) + (v[2] == e) + (v[3] == e);
+  }
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) c += __shfl_xor(c, o);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
   __syncthreads();
+  c = 0;
+#pragma unroll
+  for (int w = 0; w < MOE_THREADS / 64; ++w) c += red[w];
+  __syncthreads();
+  return c;
+}
+
+__global__ __launch_bounds__(MOE_THREADS) void moe_count_kernel(const int* __restrict__ topk_ids, int* __restrict__ ps1,
+                                                                int* __restrict__ ps2, int64_t topk_length, int n, int k,
+                                                                int aligned) {
+  __shared__ int red[MOE_THREADS / 64];
+  const int e = blockIdx.x;
+  const int c = block_count_ids(topk_ids, topk_length, e, aligned != 0, red);
   if (threadIdx.x == 0) {
-    c = red[0] + red[1] + red[2] + red[3];
     ps1[3 * e] = c;
     ps1[3 * e + 1] = 2 * n;
     ps1[3 * e + 2] = k;
@@ -89,35 +116,57 @@ __global__ __launch_bounds__(256) void moe_offsets_kernel(const int* __restrict_
   }
 }
 
-__global__ __launch_bounds__(256) void moe_place_kernel(const int* __restrict__ topk_ids,
-                                                        const int* __restrict__ expert_offsets,
-                                                        int* __restrict__ input_permutation,
-                                                        int* __restrict__ output_permutation, int64_t topk_length,
-                                                        int topk) {
-  __shared__ int wave_count[4];
+// Block (e, part) places expert e's slots of the part-th range of `span` slots (a multiple of
+// 4096); it first counts the expert's slots in the ranges before its own, which is where its
+// positions start.  Inside a sweep a slot's position follows from the matches before it:
+// those of earlier waves, of earlier lanes of its wave (one ballot per slot of the four), and
+// of the thread's own earlier slots.
+__global__ __launch_bounds__(MOE_THREADS) void moe_place_kernel(const int* __restrict__ topk_ids,
+                                                                const int* __restrict__ expert_offsets,
+                                                                int* __restrict__ input_permutation,
+                                                                int* __restrict__ output_permutation, int64_t topk_length,
+                                                                int topk, int64_t span, int aligned) {
+  __shared__ int red[MOE_THREADS / 64];
+  __shared__ int wave_count[2][MOE_THREADS / 64];
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int next = expert_offsets[e];  // position of the expert's next slot
-  for (int64_t i0 = 0; i0 < topk_length; i0 += 256) {
-    const int64_t i = i0 + threadIdx.x;
-    const bool mine = i < topk_length && topk_ids[i] == e;
-    const uint64_t ballot = __ballot(mine);
-    const int before = __popcll(ballot & ((1ull << lane) - 1ull));  // earlier slots of this wave
-    if (lane == 0) wave_count[wave] = __popcll(ballot);
-    __syncthreads();
+  const int64_t begin = (int64_t)blockIdx.y * span;
+  if (begin >= topk_length) return;
+  const int64_t end = begin + span < topk_length ? begin + span : topk_length;
+  int next = expert_offsets[e] + block_count_ids(topk_ids, begin, e, aligned != 0, red);
+  const uint64_t below = (1ull << lane) - 1ull;
+  int buf = 0;
+  v4i v = load_ids4(topk_ids, begin + 4 * (int64_t)threadIdx.x, end, aligned != 0);
+  for (int64_t i0 = begin; i0 < end; i0 += MOE_SWEEP, buf ^= 1) {
+    const int64_t i = i0 + 4 * (int64_t)threadIdx.x;
+    const v4i cur = v;
+    if (i0 + MOE_SWEEP < end) v = load_ids4(topk_ids, i + MOE_SWEEP, end, aligned != 0);  // the next sweep's, ahead of the barrier
+    int before = 0, in_wave = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint64_t ballot = __ballot(cur[q] == e);
+      before += __popcll(ballot & below);
+      in_wave += __popcll(ballot);
+    }
+    if (lane == 0) wave_count[buf][wave] = in_wave;
+    __syncthreads();  // (the buffer written two sweeps ago was last read before the previous sweep's barrier)
     int earlier_waves = 0, total = 0;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      if (w < wave) earlier_waves += wave_count[w];
-      total += wave_count[w];
+    for (int w = 0; w < MOE_THREADS / 64; ++w) {
+      const int c = wave_count[buf][w];
+      earlier_waves += w < wave ? c : 0;
+      total += c;
     }
-    if (mine) {
-      const int pos = next + earlier_waves + before;
-      input_permutation[pos] = (int)(i / topk);
-      output_permutation[i] = pos;
+    int pos = next + earlier_waves + before;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (cur[q] == e) {
+        input_permutation[pos] = (int)((i + q) / topk);
+        output_permutation[i + q] = pos;
+        ++pos;
+      }
     }
     next += total;
-    __syncthreads();
   }
 }
 
@@ -201,26 +250,48 @@ __global__ __launch_bounds__(256) void silu_and_mul_scalar_kernel(const uint16_t
 // apply_shuffle_mul_sum (prepare_moe_input.cu:258-392): output[i, :] = sum over j < topk of
 // factors[i * topk + j] * input[permutation[i * topk + j], :], accumulated in fp32 in j order
 // with one fused multiply-add per term (:293-295), rounded once to the 16-bit type.
-// One block per token, 8 elements per lane.
+// A lane owns 8 consecutive elements of one output row; lanes walk (row, chunk) pairs linearly,
+// so rows of any length fill the waves.
 // ---------------------------------------------------------------------------
 template <int DT>
 __global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
                                                               const int* __restrict__ perm,
                                                               const uint16_t* __restrict__ factors, int64_t m, int topk,
                                                               int64_t row, int64_t num_src_rows) {
-  const int64_t i = blockIdx.x;
-  for (int64_t c = threadIdx.x; c * 8 < row; c += 256) {
+  const int64_t cpr = row >> 3;  // chunks per row
+  const int64_t total = m * cpr;
+  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+    const int64_t i = id / cpr, c = id - i * cpr;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int j = 0; j < topk; ++j) {
-      const int64_t slot = i * topk + j;
-      const int64_t src = perm[slot];
-      if (src < 0 || src >= num_src_rows) continue;  // a slot that was routed to nobody contributes nothing
-      const float f = factors ? to_f32_16<DT>(factors[slot]) : 1.0f;
-      const v4u v = *reinterpret_cast<const v4u*>(in + src * row + c * 8);
+    // Eight slots at a time: their table entries, then their rows, are loaded together so that one
+    // memory round trip covers eight terms; the sum still runs in slot order.  A slot that names
+    // no row (routed to nobody, or past topk) reads row 0 and enters as 0 * 0, which leaves the
+    // sum as it is (the sum is never -0: it starts from +0).
+    for (int j0 = 0; j0 < topk; j0 += 8) {
+      int64_t src[8];
+      float f[8];
+      bool ok[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        acc[2 * q] = __builtin_fmaf(f, to_f32_16<DT>((uint16_t)(v[q] & 0xffffu)), acc[2 * q]);
-        acc[2 * q + 1] = __builtin_fmaf(f, to_f32_16<DT>((uint16_t)(v[q] >> 16)), acc[2 * q + 1]);
+      for (int u = 0; u < 8; ++u) {
+        const int64_t slot = i * topk + (j0 + u < topk ? j0 + u : topk - 1);
+        src[u] = perm[slot];
+        f[u] = factors ? to_f32_16<DT>(factors[slot]) : 1.0f;
+      }
+      v4u v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        ok[u] = j0 + u < topk && src[u] >= 0 && src[u] < num_src_rows;
+        v[u] = *reinterpret_cast<const v4u*>(in + (ok[u] ? src[u] : 0) * row + c * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fu = ok[u] ? f[u] : 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w = ok[u] ? v[u][q] : 0u;
+          acc[2 * q] = __builtin_fmaf(fu, to_f32_16<DT>((uint16_t)(w & 0xffffu)), acc[2 * q]);
+          acc[2 * q + 1] = __builtin_fmaf(fu, to_f32_16<DT>((uint16_t)(w >> 16)), acc[2 * q + 1]);
+        }
       }
     }
     v4u o;
@@ -250,12 +321,20 @@ extern "C" int sglq_prepare_moe_input(const int32_t* topk_ids, int32_t* expert_o
     return SGLQ_EINVAL;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  moe_count_kernel<<<dim3((uint32_t)num_experts), dim3(256), 0, st>>>(topk_ids, problem_sizes1, problem_sizes2, topk_length, (int)n,
-                                                                      (int)k);
+  const int aligned = (reinterpret_cast<uintptr_t>(topk_ids) & 15) == 0;
+  moe_count_kernel<<<dim3((uint32_t)num_experts), dim3(MOE_THREADS), 0, st>>>(topk_ids, problem_sizes1, problem_sizes2, topk_length,
+                                                                              (int)n, (int)k, aligned);
   moe_offsets_kernel<<<dim3(1), dim3(256), 0, st>>>(problem_sizes1, expert_offsets, blockscale_offsets, (int)num_experts);
-  if (topk_length > 0)
-    moe_place_kernel<<<dim3((uint32_t)num_experts), dim3(256), 0, st>>>(topk_ids, expert_offsets, input_permutation,
-                                                                        output_permutation, topk_length, (int)topk);
+  if (topk_length > 0) {
+    // few experts: several blocks per expert, each with its own range of slots (about one block per CU in all)
+    const int64_t sweeps = (topk_length + MOE_SWEEP - 1) / MOE_SWEEP;
+    int64_t parts = 256 / num_experts;
+    if (parts > sweeps) parts = sweeps;
+    if (parts < 1) parts = 1;
+    const int64_t span = (sweeps + parts - 1) / parts * MOE_SWEEP;
+    moe_place_kernel<<<dim3((uint32_t)num_experts, (uint32_t)parts), dim3(MOE_THREADS), 0, st>>>(
+        topk_ids, expert_offsets, input_permutation, output_permutation, topk_length, (int)topk, span, aligned);
+  }
   return check_moe_launch(name);
 }
 
@@ -328,6 +407,10 @@ extern "C" int sglq_apply_shuffle_mul_sum(const void* input, void* output, const
     return SGLQ_EINVAL;
   }
   if (m == 0 || row == 0) return SGLQ_OK;
+  if (num_src_rows == 0) {
+    set_error("%s: input has no rows", name);
+    return SGLQ_EINVAL;
+  }
   if (!input || !output || !permutation) {
     set_error("%s: null pointer", name);
     return SGLQ_EINVAL;
@@ -337,7 +420,9 @@ extern "C" int sglq_apply_shuffle_mul_sum(const void* input, void* output, const
     return SGLQ_EINVAL;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid((uint32_t)m), block(256);
+  int64_t blocks = (m * (row / 8) + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  const dim3 grid((uint32_t)blocks), block(256);
   const uint16_t* in = static_cast<const uint16_t*>(input);
   uint16_t* out = static_cast<uint16_t*>(output);
   const uint16_t* f = static_cast<const uint16_t*>(factors);

@@ -18,10 +18,16 @@ def say(*a):
     print(*a, flush=True)
 
 
-def run_prepare(gpu, ids, num_experts, n, k, with_blockscale=True, fill=-7):
+def run_prepare(gpu, ids, num_experts, n, k, with_blockscale=True, fill=-7, shift=0):
+    """`shift` moves topk_ids off its 16-byte alignment by that many elements."""
     from sglang_amd.sgl_kernel import prepare_moe_input
 
     i32 = lambda *shape: torch.full(shape, fill, dtype=torch.int32, device=gpu)
+    if shift:
+        holder = torch.full((ids.numel() + shift + 8,), 0, dtype=torch.int32)
+        holder[shift:shift + ids.numel()] = ids.reshape(-1)
+        ids = holder.to(gpu)[shift:shift + ids.numel()].view(ids.shape)
+        assert ids.data_ptr() % 16 != 0
     offsets, rounded = i32(num_experts + 1), i32(num_experts + 1)
     ps1, ps2 = i32(num_experts, 3), i32(num_experts, 3)
     a_map, c_map = i32(ids.numel()), i32(ids.numel())
@@ -31,7 +37,7 @@ def run_prepare(gpu, ids, num_experts, n, k, with_blockscale=True, fill=-7):
 
 
 @pytest.mark.parametrize("m,topk,num_experts", [(1, 1, 1), (1, 8, 256), (33, 2, 8), (257, 8, 64), (1000, 6, 160),
-                                                (4096, 8, 256), (77, 4, 384), (300, 1, 3)])
+                                                (4096, 8, 256), (77, 4, 384), (300, 1, 3), (4099, 7, 8), (9000, 3, 2)])
 def test_prepare_moe_input_tables(gpu, m, topk, num_experts):
     """Every table equals the oracle's, which keeps slot order inside an expert (the operator's
     documented order); ids outside [0, E) leave their output_permutation entry and the tail of
@@ -50,6 +56,9 @@ def test_prepare_moe_input_tables(gpu, m, topk, num_experts):
     for name, g_t, w_t in zip(names, got, want):
         w_t = torch.where(w_t < 0, torch.full_like(w_t, -7), w_t) if name.endswith("permutation") else w_t
         assert torch.equal(g_t, w_t.reshape(g_t.shape)), name
+    # ids that do not start on a 16-byte boundary (scalar loads)
+    for a, b in zip(got, run_prepare(gpu, ids, num_experts, n, k, shift=1)):
+        assert torch.equal(a, b)
     # without the optional table
     got2 = run_prepare(gpu, ids, num_experts, n, k, with_blockscale=False)
     assert bool((got2[1] == -7).all())
