@@ -139,3 +139,68 @@ def scaled_fp8_quant(
         assert scale.numel() == 1, f"Expected scalar scale, got numel={scale.numel()}"
         sgl_per_tensor_quant_fp8(input, q, scale, is_static=True)
     return output, scale
+
+
+def w8a8_block_fp8_matmul(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    block_size,
+    output_dtype: torch.dtype = torch.float16,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """fp8_kernel.py:801-846,870-967 (w8a8_block_fp8_matmul and its Triton twin): A e4m3fn
+    [..., K] contiguous, B e4m3fn [N, K] contiguous (the weight as stored), As fp32 [..., K/128]
+    (row-major, as per_token_group_quant_fp8 returns it without column_major_scales), Bs fp32
+    [N/128, K/128]; N and K need not be multiples of 128 (K of 16 and N of 4).  `bias` (not an argument of the
+    reference's function): the caller's `output += bias` (fp8_utils.py:307-308) fused, [N] in
+    output_dtype, same two roundings.  UE8M0-packed (int32) scales are not accepted."""
+    assert len(block_size) == 2
+    block_n, block_k = block_size[0], block_size[1]
+    if block_n != 128 or block_k != 128:
+        raise NotImplementedError("w8a8_block_fp8_matmul: only 128 x 128 weight blocks are built")
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1]
+    assert A.is_contiguous()
+    if As.dtype != torch.float32 or Bs.dtype != torch.float32:
+        raise NotImplementedError("w8a8_block_fp8_matmul: scales must be Float32")
+    assert -(-A.shape[-1] // block_k) == As.shape[-1]
+    M = A.numel() // A.shape[-1]
+    assert B.ndim == 2
+    assert B.is_contiguous()
+    assert Bs.ndim == 2
+    N, K = B.shape
+    assert -(-N // block_n) == Bs.shape[0]
+    assert -(-K // block_k) == Bs.shape[1]
+    if not (A.is_cuda and B.is_cuda and As.is_cuda and Bs.is_cuda):
+        raise RuntimeError("w8a8_block_fp8_matmul: tensors must be CUDA tensors")
+    if A.dtype != fp8_dtype or B.dtype != fp8_dtype:
+        raise RuntimeError("w8a8_block_fp8_matmul: A and B must be Float8_e4m3fn")
+    if output_dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError("w8a8_block_fp8_matmul: output_dtype must be Half or BFloat16")
+    C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
+    if M == 0 or N == 0:
+        return C
+    As2 = As.reshape(M, As.shape[-1])
+    if not Bs.is_contiguous():
+        Bs = Bs.contiguous()
+    lib = _lib.load()
+    if bias is not None:
+        if not (bias.is_cuda and bias.is_contiguous() and bias.numel() == N and bias.dtype == output_dtype):
+            raise RuntimeError("w8a8_block_fp8_matmul: bias must be a contiguous CUDA tensor of N elements in output_dtype")
+        rc = lib.sglq_fp8_blockwise_scaled_mm_bias(
+            A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
+            Bs.data_ptr(), Bs.stride(1), Bs.stride(0), bias.data_ptr(), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,
+            *_lib.workspace(A.device), _lib.stream_ptr(A.device))
+    else:
+        rc = lib.sglq_fp8_blockwise_scaled_mm(
+            A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
+            Bs.data_ptr(), Bs.stride(1), Bs.stride(0), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,
+            *_lib.workspace(A.device), _lib.stream_ptr(A.device))
+    _lib.check(rc, "w8a8_block_fp8_matmul")
+    return C
+
+
+# the Triton kernel behind it (:870-948) computes the same sums
+w8a8_block_fp8_matmul_triton = w8a8_block_fp8_matmul

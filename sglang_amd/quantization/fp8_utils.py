@@ -9,7 +9,7 @@ import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from ..sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
-from .fp8_kernel import per_token_group_quant_fp8, sglang_per_token_quant_fp8, static_quant_fp8
+from .fp8_kernel import per_token_group_quant_fp8, sglang_per_token_quant_fp8, static_quant_fp8, w8a8_block_fp8_matmul
 
 
 def w8a8_block_fp8_linear(
@@ -36,6 +36,29 @@ def w8a8_block_fp8_linear(
         output = fp8_blockwise_scaled_mm_bias(q_input, weight.T, x_scale, weight_scale.T, input_2d.dtype, bias)
     else:
         output = fp8_blockwise_scaled_mm(q_input, weight.T, x_scale, weight_scale.T, out_dtype=input_2d.dtype)
+        if bias is not None:
+            output += bias
+    return output.to(dtype=input_2d.dtype).view(*output_shape)
+
+
+def triton_w8a8_block_fp8_linear(
+    input: torch.Tensor,
+    weight: torch.Tensor,
+    block_size: List[int],
+    weight_scale: torch.Tensor,
+    input_scale: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """The call sequence of triton_w8a8_block_fp8_linear (fp8_utils.py:289-309): row-major
+    activation scales, the weight and its scales as stored, any N and K."""
+    assert input_scale is None
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=False)
+    if bias is not None and bias.dtype == input_2d.dtype and bias.is_contiguous() and bias.numel() == weight.shape[0]:
+        output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input_2d.dtype, bias=bias)
+    else:
+        output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input_2d.dtype)
         if bias is not None:
             output += bias
     return output.to(dtype=input_2d.dtype).view(*output_shape)

@@ -67,3 +67,61 @@ def test_fp8_static_activation_scale_linear(gpu):
     ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16, bias)
     out = apply_fp8_linear(x.to(gpu), wq.to(gpu).t(), ws.to(gpu), input_scale=in_scale.to(gpu), bias=bias.to(gpu))
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("mnk", [(1, 128, 128), (5, 2112, 1536), (40, 200, 1008), (127, 512, 7168), (300, 2048, 1024), (1024, 640, 2048),
+                                 (4096, 1536, 512)])
+def test_w8a8_block_fp8_matmul_row_major_scales(gpu, mnk):
+    """w8a8_block_fp8_matmul (fp8_kernel.py:801-846,951-967): the weight and its scales as stored,
+    row-major activation scales, N and K that are not multiples of 128; the same values as the
+    sgl_kernel operator on transposed views, bit for bit, where that operator's K rule allows."""
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul, w8a8_block_fp8_matmul_triton
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    m, n, k = mnk
+    print("w8a8_block_fp8_matmul", mnk, flush=True)
+    g = torch.Generator().manual_seed(m + n + k)
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=n + k))
+    xq = (torch.randn((m, k), generator=g) * 100).clamp(-448, 448).to(torch.float8_e4m3fn)
+    xs = torch.rand((m, (k + 127) // 128), generator=g) * 1e-2 + 1e-3
+    assert w8a8_block_fp8_matmul_triton is w8a8_block_fp8_matmul
+    for dt in (torch.bfloat16, torch.float16):
+        out = w8a8_block_fp8_matmul(xq.to(gpu), wq.to(gpu), xs.to(gpu), ws.to(gpu), [128, 128], dt)
+        assert out.dtype == dt and tuple(out.shape) == (m, n)
+        ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
+        torch.testing.assert_close(out.cpu().float(), ref, rtol=1e-2, atol=1e-2)
+        if k % 128 == 0:
+            xs_cm = xs.to(gpu).t().contiguous().t()
+            same = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), dt)
+            assert torch.equal(out.view(torch.int16), same.view(torch.int16))
+        bias = (torch.randn(n, generator=g) * 0.5).to(dt).to(gpu)
+        fused = w8a8_block_fp8_matmul(xq.to(gpu), wq.to(gpu), xs.to(gpu), ws.to(gpu), [128, 128], dt, bias=bias)
+        assert torch.equal(fused.view(torch.int16), (out + bias).view(torch.int16))
+    # leading dimensions are kept
+    out3 = w8a8_block_fp8_matmul(xq.to(gpu).view(1, m, k), wq.to(gpu), xs.to(gpu).view(1, m, -1), ws.to(gpu), [128, 128], torch.bfloat16)
+    assert tuple(out3.shape) == (1, m, n)
+
+
+def test_triton_path_block_fp8_linear(gpu):
+    """triton_w8a8_block_fp8_linear (fp8_utils.py:289-309) against the oracle's same sequence, and
+    against the column-major-scale path of the same layer bit for bit (same kernels, same sums)."""
+    from sglang_amd.quantization.fp8_utils import triton_w8a8_block_fp8_linear, w8a8_block_fp8_linear
+
+    print("triton-path block fp8 linear", flush=True)
+    x = O.gen_activation(96, 2048, seed=3, outliers=True)
+    wq, ws = O.block_quant_weight(O.gen_weight(1536, 2048, seed=4))
+    bias = (torch.randn(1536, generator=torch.Generator().manual_seed(5)) * 0.1).to(torch.bfloat16)
+    xq, xs = O.per_token_group_quant_fp8(x, 128)
+    mm = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32)
+    ref = mm + bias.float()
+    for b in (None, bias.to(gpu)):
+        out = triton_w8a8_block_fp8_linear(x.to(gpu).view(2, 48, 2048), wq.to(gpu), [128, 128], ws.to(gpu), bias=b)
+        assert tuple(out.shape) == (2, 48, 1536) and out.dtype == torch.bfloat16
+        want = ref if b is not None else mm
+        tol = 1e-2 + 1e-2 * want.abs() + mm.abs() * 2.0**-8
+        err = (out.cpu().view(96, 1536).float() - want).abs()
+        assert bool((err <= tol).all()), f"max excess {(err - tol).max().item()}"
+        other = w8a8_block_fp8_linear(x.to(gpu).view(2, 48, 2048), wq.to(gpu), [128, 128], ws.to(gpu), bias=b)
+        assert torch.equal(out.view(torch.int16), other.view(torch.int16))
+    with pytest.raises(NotImplementedError):
+        triton_w8a8_block_fp8_linear(x.to(gpu), wq.to(gpu), [64, 64], ws.to(gpu))
