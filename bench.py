@@ -439,9 +439,12 @@ def run_sweep(args):
             torch.cuda.empty_cache()
     # the whole expert layer (routing tables, gathers, two grouped GEMMs, SiLU-and-multiply, quantization, combine) on
     # DeepSeek-V3's expert shape, 32 local experts, top-8 routing among them: per-step device times and the layer's
+    # (the layer runs SiLU-and-multiply and the second quantization as one kernel, "silu_quant_fused"; the two
+    # separate operators are timed beside it and left out of the steps' sum)
     if want("moe_layer"):
         from sglang_amd.moe.cutlass_moe import cutlass_fused_experts_fp8
         from sglang_amd.sgl_kernel import apply_shuffle_mul_sum, prepare_moe_input, shuffle_rows, silu_and_mul
+        from sglang_amd.sgl_kernel.moe import silu_and_mul_per_token_group_quant_fp8
 
         e, k, n, topk = 32, 7168, 2048, 8
         g = torch.Generator(device=dev).manual_seed(6000)
@@ -477,6 +480,7 @@ def run_sweep(args):
             t["silu_and_mul"] = time_kernel(lambda j: silu_and_mul(c1), iters)
             inter = silu_and_mul(c1)
             t["quant2"] = time_kernel(lambda j: sglang_per_token_group_quant_fp8(inter, 128), iters)
+            t["silu_quant_fused"] = time_kernel(lambda j: silu_and_mul_per_token_group_quant_fp8(c1, 128), iters)
             iq, isc = sglang_per_token_group_quant_fp8(inter, 128)
             t["gemm2"] = time_kernel(lambda j: gmm(c2, iq, w2, isc, s2, ps2), iters)
             res = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
@@ -486,10 +490,11 @@ def run_sweep(args):
                                                                     i64, offs, ps1, ps2), iters)
             fl = 2.0 * rows * (2 * n * k + n * k)
             moved = {"gather_codes": 2 * rows * k, "gather_scales": 8 * rows * (k // 128), "silu_and_mul": 6 * rows * n,
-                     "quant1": group_quant_bytes(m, k), "quant2": group_quant_bytes(rows, n), "combine": 2 * rows * k + 2 * m * k}
+                     "quant1": group_quant_bytes(m, k), "quant2": group_quant_bytes(rows, n),
+                     "silu_quant_fused": 5 * rows * n + 4 * rows * (n // 128), "combine": 2 * rows * k + 2 * m * k}
             emit(cfg="moe_layer", op="cutlass_fused_experts_fp8", experts=e, topk=topk, M=m, hidden=k, intermediate=n,
                  layer_us=round(layer * 1e3, 1), layer_TFLOPs=round(fl / layer / 1e9, 2),
-                 steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(t.values()) * 1e3, 1),
+                 steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(v for s, v in t.items() if s not in ("silu_and_mul", "quant2")) * 1e3, 1),
                  steps_GBs={s: round(b / t[s] / 1e6, 1) for s, b in moved.items()})
     f.close()
 

@@ -194,6 +194,16 @@ int sglq_silu_and_mul(const void* input, int dtype, void* output, int64_t num_to
 int sglq_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors,
                                int dtype, int64_t m, int64_t topk, int64_t row, int64_t num_src_rows, void* stream);
 
+/* silu_and_mul (activation.cu:57-60) followed by sgl_per_token_group_quant_fp8 with group 128
+ * (per_token_group_quant_8bit.cu:72-113), the pair of calls of
+ * python/sglang/srt/layers/moe/cutlass_moe.py:187-194, in one kernel that never writes the
+ * intermediate: input [num_tokens, 2 d] in dtype (SGLQ_BF16 or SGLQ_FP16), output_q
+ * [num_tokens, d] e4m3fn, output_s [num_tokens, d / 128] fp32 row-major, d a multiple of 128.
+ * Codes and scales are bit-identical to sglq_silu_and_mul followed by
+ * sglq_per_token_group_quant_fp8(group 128, eps, -448, 448). */
+int sglq_silu_and_mul_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
+                                      int64_t num_tokens, int64_t d, float eps, void* stream);
+
 /* Replaces w8a8_block_int8_matmul, a Triton kernel in the reference
  * (python/sglang/srt/layers/quantization/int8_kernel.py:212-425; there is no
  * sgl_kernel C++ op): out[m,n] = sum_kb float(sum_{k in block kb} a[m,k] b[k,n])

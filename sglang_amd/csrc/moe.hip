@@ -196,17 +196,6 @@ __global__ __launch_bounds__(256) void shuffle_rows_kernel(const char* __restric
 // product rounded to T again; silu(v) = v / (1 + expf(-v)) in fp32.  16 bytes per lane.
 // ---------------------------------------------------------------------------
 template <int DT>
-SGLQ_DEV float to_f32_16(uint16_t h) {
-  if constexpr (DT == SGLQ_BF16) return u2f((uint32_t)h << 16);
-  else return (float)__builtin_bit_cast(_Float16, h);
-}
-template <int DT>
-SGLQ_DEV uint16_t from_f32_16(float v) {
-  if constexpr (DT == SGLQ_BF16) return __builtin_bit_cast(uint16_t, (__bf16)v);
-  else return __builtin_bit_cast(uint16_t, (_Float16)v);
-}
-
-template <int DT>
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
                                                            int64_t tokens, int64_t d) {
   const int64_t cpr = d >> 3;  // 8-element chunks per output row
@@ -221,10 +210,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
       uint32_t w = 0;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const float x = to_f32_16<DT>((uint16_t)(xv[q] >> (16 * h)));
-        const float y = to_f32_16<DT>((uint16_t)(yv[q] >> (16 * h)));
-        const float act = to_f32_16<DT>(from_f32_16<DT>(x / (1.0f + __builtin_expf(-x))));
-        w |= (uint32_t)from_f32_16<DT>(act * y) << (16 * h);
+        w |= (uint32_t)silu_mul_16<DT>((uint16_t)(xv[q] >> (16 * h)), (uint16_t)(yv[q] >> (16 * h))) << (16 * h);
       }
       o[q] = w;
     }
@@ -239,10 +225,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_scalar_kernel(const uint16_t
   const int64_t total = tokens * d;
   for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
     const int64_t t = id / d, c = id - t * d;
-    const float x = to_f32_16<DT>(in[t * 2 * d + c]);
-    const float y = to_f32_16<DT>(in[t * 2 * d + d + c]);
-    const float act = to_f32_16<DT>(from_f32_16<DT>(x / (1.0f + __builtin_expf(-x))));
-    out[id] = from_f32_16<DT>(act * y);
+    out[id] = silu_mul_16<DT>(in[t * 2 * d + c], in[t * 2 * d + d + c]);
   }
 }
 

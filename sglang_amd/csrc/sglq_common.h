@@ -80,4 +80,37 @@ SGLQ_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
+// 16-bit floats (dtype code SGLQ_BF16 or SGLQ_FP16) as raw bits <-> fp32, round to nearest even.
+template <int DT>
+SGLQ_DEV float to_f32_16(uint16_t h) {
+  if constexpr (DT == SGLQ_BF16) return u2f((uint32_t)h << 16);
+  else return (float)__builtin_bit_cast(_Float16, h);
+}
+template <int DT>
+SGLQ_DEV uint16_t from_f32_16(float v) {
+  if constexpr (DT == SGLQ_BF16) return __builtin_bit_cast(uint16_t, (__bf16)v);
+  else return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+
+// silu(v) = v / (1 + exp(-v)) in fp32 with the hardware's exp2 and reciprocal (each within one
+// unit in the last place; the reference writes v / (1 + expf(-v)),
+// sgl-kernel/csrc/elementwise/activation.cu:57-60, and builds with -use_fast_math,
+// sgl-kernel/CMakeLists.txt:190, which makes both approximate as well).  exp2 overflows to +inf for v below
+// about -88, where the result is -0 like the exact quotient's.
+SGLQ_DEV float silu_f32(float v) {
+  const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896340736f);
+  return v * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+// T(T(silu(x)) * y): both roundings of the reference's activation kernel (activation.cu:57-60,85-103).
+template <int DT>
+SGLQ_DEV uint16_t silu_mul_16(uint16_t xb, uint16_t yb) {
+  float s = silu_f32(to_f32_16<DT>(xb));
+  // (keeps the product and its rounding to 16 bits apart: fused into one mixed-precision
+  // multiply-add with a +0 addend, silu(-0) would come out as +0)
+  asm volatile("" : "+v"(s));
+  const float act = to_f32_16<DT>(from_f32_16<DT>(s));
+  return from_f32_16<DT>(act * to_f32_16<DT>(yb));
+}
+
 }  // namespace sglq

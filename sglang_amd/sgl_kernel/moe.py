@@ -202,3 +202,24 @@ def silu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     rc = _lib.load().sglq_silu_and_mul(input.data_ptr(), DTYPE_CODE[input.dtype], out.data_ptr(), tokens, d, _lib.stream_ptr(input.device))
     _lib.check(rc, "silu_and_mul")
     return out
+
+
+def silu_and_mul_per_token_group_quant_fp8(input: torch.Tensor, group_size: int = 128, eps: float = 1e-10):
+    """silu_and_mul(input) followed by sglang_per_token_group_quant_fp8(., 128) in one kernel
+    (the two calls of python/sglang/srt/layers/moe/cutlass_moe.py:187-194); the intermediate
+    is not materialised.  input [..., 2 d] Half / BFloat16, d a multiple of 128; returns
+    (codes [..., d] e4m3fn, scales [..., d / 128] fp32 row-major), bit-identical to the two calls."""
+    if group_size != 128:
+        raise NotImplementedError("silu_and_mul_per_token_group_quant_fp8: group size 128 is built")
+    _check(input.is_cuda and input.is_contiguous(), "input must be a contiguous CUDA tensor")
+    if input.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError("silu_and_mul_per_token_group_quant_fp8: Half and BFloat16 are built")
+    d = input.shape[-1] // 2
+    _check(input.shape[-1] == 2 * d and d % 128 == 0, "the last dimension must be 2 d with d a multiple of 128")
+    out_q = torch.empty(input.shape[:-1] + (d,), device=input.device, dtype=FP8)
+    out_s = torch.empty(input.shape[:-1] + (d // 128,), device=input.device, dtype=torch.float32)
+    tokens = input.numel() // input.shape[-1] if input.numel() else 0
+    rc = _lib.load().sglq_silu_and_mul_group_quant_fp8(input.data_ptr(), DTYPE_CODE[input.dtype], out_q.data_ptr(), out_s.data_ptr(),
+                                                       tokens, d, eps, _lib.stream_ptr(input.device))
+    _lib.check(rc, "silu_and_mul_per_token_group_quant_fp8")
+    return out_q, out_s

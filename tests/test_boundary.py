@@ -194,6 +194,10 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.sglq_silu_and_mul(p, 2, p, 4, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
     assert lib.sglq_silu_and_mul(None, 0, p, 4, 8, None) == 1 and b"null" in lib.sglq_last_error()
     assert lib.sglq_silu_and_mul(p, 0, p, 0, 8, None) == 0
+    assert lib.sglq_silu_and_mul_group_quant_fp8(p, 0, p, p, 4, 192, 1e-10, None) == 1 and b"multiple of 128" in lib.sglq_last_error()
+    assert lib.sglq_silu_and_mul_group_quant_fp8(p, 2, p, p, 4, 128, 1e-10, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
+    assert lib.sglq_silu_and_mul_group_quant_fp8(p, 0, p, None, 4, 128, 1e-10, None) == 1 and b"null" in lib.sglq_last_error()
+    assert lib.sglq_silu_and_mul_group_quant_fp8(p, 0, p, p, 0, 128, 1e-10, None) == 0
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 0, 8, 8, None) == 1 and b"bad sizes" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 2, 12, 8, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 2, 4, 2, 8, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()

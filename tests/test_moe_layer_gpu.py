@@ -138,6 +138,38 @@ def test_silu_and_mul(gpu, dtype, tokens, d):
     assert torch.equal(buf.cpu().reshape(tokens, d), out)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.half])
+@pytest.mark.parametrize("tokens,d", [(1, 128), (7, 2048), (333, 256), (4096, 384)])
+def test_silu_and_mul_fused_with_group_quant(gpu, dtype, tokens, d):
+    """One kernel for SiLU-and-multiply and the group quantization after it: codes and scales equal
+    those of the two operators called one after the other, bit for bit (zero rows, large values
+    and rows whose activation underflows included)."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import silu_and_mul
+    from sglang_amd.sgl_kernel.moe import silu_and_mul_per_token_group_quant_fp8
+
+    g = torch.Generator().manual_seed(tokens + d)
+    x = (torch.randn((tokens, 2 * d), generator=g) * 3).to(dtype)
+    x[0, :128] = 0
+    x[tokens - 1, :64] = -40.0
+    x[tokens // 2, d:d + 32] = 200.0
+    say("silu_and_mul + group quant", dtype, tokens, d)
+    xg = x.to(gpu)
+    q2, s2 = sglang_per_token_group_quant_fp8(silu_and_mul(xg), 128)
+    q1, s1 = silu_and_mul_per_token_group_quant_fp8(xg, 128)
+    assert q1.shape == (tokens, d) and s1.shape == (tokens, d // 128) and s1.is_contiguous()
+    assert_bits_equal(q1, q2, "codes")
+    assert_bits_equal(s1, s2, "scales")
+    # and the oracle's two steps on the device's activation (the exponential is the device's)
+    oq, os_ = O.per_token_group_quant_fp8(silu_and_mul(xg).cpu(), 128)
+    assert_bits_equal(q1, oq, "codes against the oracle")
+    assert_bits_equal(s1, os_, "scales against the oracle")
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        silu_and_mul_per_token_group_quant_fp8(torch.zeros((2, 192), dtype=dtype, device=gpu))
+    with pytest.raises(NotImplementedError):
+        silu_and_mul_per_token_group_quant_fp8(torch.zeros((2, 256), dtype=torch.float32, device=gpu))
+
+
 def test_silu_and_mul_argument_checks(gpu):
     from sglang_amd.sgl_kernel import silu_and_mul
 
