@@ -439,12 +439,14 @@ def run_sweep(args):
             torch.cuda.empty_cache()
     # the whole expert layer (routing tables, gathers, two grouped GEMMs, SiLU-and-multiply, quantization, combine) on
     # DeepSeek-V3's expert shape, 32 local experts, top-8 routing among them: per-step device times and the layer's
-    # (the layer runs SiLU-and-multiply and the second quantization as one kernel, "silu_quant_fused"; the two
-    # separate operators are timed beside it and left out of the steps' sum)
+    # (the layer runs the first quantization and the two gathers as one kernel, "quant_to_expert_rows_fused", and
+    # SiLU-and-multiply and the second quantization as another, "silu_quant_fused"; the separate operators are timed
+    # beside them and left out of the steps' sum)
+    SEPARATE = ("quant1", "gather_codes", "gather_scales", "silu_and_mul", "quant2")
     if want("moe_layer"):
         from sglang_amd.moe.cutlass_moe import cutlass_fused_experts_fp8
         from sglang_amd.sgl_kernel import apply_shuffle_mul_sum, prepare_moe_input, shuffle_rows, silu_and_mul
-        from sglang_amd.sgl_kernel.moe import silu_and_mul_per_token_group_quant_fp8
+        from sglang_amd.sgl_kernel.moe import per_token_group_quant_fp8_to_expert_rows, silu_and_mul_per_token_group_quant_fp8
 
         e, k, n, topk = 32, 7168, 2048, 8
         g = torch.Generator(device=dev).manual_seed(6000)
@@ -471,6 +473,7 @@ def run_sweep(args):
             a_q, a_s = sglang_per_token_group_quant_fp8(x, 128)
             t["gather_codes"] = time_kernel(lambda j: shuffle_rows(a_q, a_map, (rows, k)), iters)
             t["gather_scales"] = time_kernel(lambda j: shuffle_rows(a_s, a_map, (rows, k // 128)), iters)
+            t["quant_to_expert_rows_fused"] = time_kernel(lambda j: per_token_group_quant_fp8_to_expert_rows(x, c_map, topk, 128), iters)
             rq, rs = shuffle_rows(a_q, a_map, (rows, k)), shuffle_rows(a_s, a_map, (rows, k // 128))
             c1 = torch.empty((rows, 2 * n), dtype=torch.bfloat16, device=dev)
             c2 = torch.empty((rows, k), dtype=torch.bfloat16, device=dev)
@@ -491,10 +494,11 @@ def run_sweep(args):
             fl = 2.0 * rows * (2 * n * k + n * k)
             moved = {"gather_codes": 2 * rows * k, "gather_scales": 8 * rows * (k // 128), "silu_and_mul": 6 * rows * n,
                      "quant1": group_quant_bytes(m, k), "quant2": group_quant_bytes(rows, n),
-                     "silu_quant_fused": 5 * rows * n + 4 * rows * (n // 128), "combine": 2 * rows * k + 2 * m * k}
+                     "silu_quant_fused": 5 * rows * n + 4 * rows * (n // 128),
+                     "quant_to_expert_rows_fused": 2 * m * k + rows * k + 4 * rows * (k // 128), "combine": 2 * rows * k + 2 * m * k}
             emit(cfg="moe_layer", op="cutlass_fused_experts_fp8", experts=e, topk=topk, M=m, hidden=k, intermediate=n,
                  layer_us=round(layer * 1e3, 1), layer_TFLOPs=round(fl / layer / 1e9, 2),
-                 steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(v for s, v in t.items() if s not in ("silu_and_mul", "quant2")) * 1e3, 1),
+                 steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(v for s, v in t.items() if s not in SEPARATE) * 1e3, 1),
                  steps_GBs={s: round(b / t[s] / 1e6, 1) for s, b in moved.items()})
     f.close()
 

@@ -194,6 +194,17 @@ int sglq_silu_and_mul(const void* input, int dtype, void* output, int64_t num_to
 int sglq_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors,
                                int dtype, int64_t m, int64_t topk, int64_t row, int64_t num_src_rows, void* stream);
 
+/* sgl_per_token_group_quant_fp8 with group 128 (per_token_group_quant_8bit.cu:72-113) followed by
+ * the two shuffle_rows calls that replicate codes and scales into expert-major order
+ * (python/sglang/srt/layers/moe/cutlass_moe.py:156-158), in one kernel: input [num_tokens, hidden];
+ * token t's codes go to rows slot_map[t * topk + j] (j < topk) of output_q [num_dst_rows, hidden]
+ * and its scales to the same rows of output_s [num_dst_rows, hidden / 128] (row-major); slot_map is
+ * prepare_moe_input's output_permutation; entries outside [0, num_dst_rows) are skipped.  Rows that
+ * no slot names are left untouched.  Bit-identical to the three calls. */
+int sglq_per_token_group_quant_fp8_scatter(const void* input, int in_dtype, void* output_q, float* output_s,
+                                           const int32_t* slot_map, int64_t num_tokens, int64_t hidden, int64_t topk,
+                                           int64_t num_dst_rows, float eps, void* stream);
+
 /* silu_and_mul (activation.cu:57-60) followed by sgl_per_token_group_quant_fp8 with group 128
  * (per_token_group_quant_8bit.cu:72-113), the pair of calls of
  * python/sglang/srt/layers/moe/cutlass_moe.py:187-194, in one kernel that never writes the

@@ -41,6 +41,7 @@ SIGNATURES = {
                                c_int64, c_void_p],
     "sglq_shuffle_rows": [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p],
     "sglq_silu_and_mul": [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p],
+    "sglq_per_token_group_quant_fp8_scatter": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_void_p],
     "sglq_silu_and_mul_group_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p],
     "sglq_apply_shuffle_mul_sum": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p],
     "sglq_int8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,

@@ -200,6 +200,56 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict
 }
 
 // ---------------------------------------------------------------------------
+// Per-token-group FP8 quantization (group 128) whose result goes straight to the expert-major
+// rows an MoE layer gathers it into (python/sglang/srt/layers/moe/cutlass_moe.py:156-158:
+// quantize once per token, then shuffle_rows codes and scales by a_map): token t's codes and
+// row-major scales are written to every row slot_map[t * topk + j], j < topk, that lies in
+// [0, num_dst_rows); other entries (slots routed to nobody) are skipped.  Same arithmetic as
+// group_quant_kernel; each token is read once and written topk times instead of being
+// written once, read topk times and written topk times.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void group_quant_scatter_kernel(const char* __restrict__ x, char* __restrict__ q,
+                                                                  float* __restrict__ s, const int* __restrict__ slot_map,
+                                                                  uint32_t num_groups, FastDiv groups_per_row, int topk,
+                                                                  int64_t num_dst_rows, float eps, float qmax, float rqmax) {
+  constexpr int GROUP = 128, NCH = 2, LPG = GROUP / (8 * NCH), GPB = 256 / LPG;
+  constexpr int EB = elem_bytes<DT>();
+  const uint32_t t = threadIdx.x;
+  const uint32_t sub = t % LPG;
+  const uint32_t gid = blockIdx.x * GPB + t / LPG;
+  if (gid >= num_groups) return;
+  const uint32_t row = groups_per_row.div(gid);
+  const uint32_t col = gid - row * groups_per_row.d;
+  const int64_t hidden = (int64_t)groups_per_row.d * GROUP;
+  Chunk8<DT> ch[NCH];
+  const char* px = x + ((int64_t)gid * GROUP + sub * 8) * EB;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) ch[c].load(px + c * (GROUP / NCH) * EB);
+  uint32_t mb = umax(ch[0].amax_bits(), ch[1].amax_bits());
+  mb = group_umax<LPG>(mb);
+  const float amax = u2f(umax(mb, f2u(eps)));
+  const float y_s = div_by(amax, qmax, rqmax);
+  const float r = 1.0f / y_s;
+  v2u o[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = quantize_elem<false>(ch[c].get(i), y_s, r, -qmax, qmax);
+    o[c] = Fp8Pack::pack(v);
+  }
+  for (int j = 0; j < topk; ++j) {
+    const int64_t dst = slot_map[(int64_t)row * topk + j];
+    if (dst < 0 || dst >= num_dst_rows) continue;
+    char* qp = q + dst * hidden + (int64_t)col * GROUP + sub * 8;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) *reinterpret_cast<v2u*>(qp + c * (GROUP / NCH)) = o[c];
+    if (sub == 0) s[dst * groups_per_row.d + col] = y_s;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // SiLU-and-multiply fused with the per-token-group FP8 quantization that follows it in an MoE
 // expert layer (python/sglang/srt/layers/moe/cutlass_moe.py:187-194): input [tokens, 2 d] in a
 // 16-bit type, codes [tokens, d] and row-major scales [tokens, d / 128] of
@@ -813,6 +863,54 @@ static int static_quant_entry(const void* input, int in_dtype, void* output_q, c
 }
 
 }  // namespace sglq
+
+extern "C" int sglq_per_token_group_quant_fp8_scatter(const void* input, int in_dtype, void* output_q, float* output_s,
+                                                      const int32_t* slot_map, int64_t num_tokens, int64_t hidden,
+                                                      int64_t topk, int64_t num_dst_rows, float eps, void* stream) {
+  using namespace sglq;
+  const char* name = "per_token_group_quant_fp8_scatter";
+  if (num_tokens < 0 || hidden <= 0 || hidden % 128 != 0 || topk <= 0 || topk >= (1 << 20) || num_dst_rows < 0) {
+    set_error("%s: hidden (%lld) must be a positive multiple of 128, topk positive", name, (long long)hidden);
+    return SGLQ_EINVAL;
+  }
+  if (num_tokens == 0 || num_dst_rows == 0) return SGLQ_OK;
+  if (!input || !output_q || !output_s || !slot_map) {
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (!(eps > 0.f)) {
+    set_error("%s: eps must be positive", name);
+    return SGLQ_EINVAL;
+  }
+  if ((reinterpret_cast<uintptr_t>(input) & 15) || (reinterpret_cast<uintptr_t>(output_q) & 7)) {
+    set_error("%s: input must be 16-byte and output_q 8-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t gpr = hidden / 128, ng = num_tokens * gpr;
+  if (ng >= (1ll << 32) - 65536) {
+    set_error("%s: too many groups (%lld)", name, (long long)ng);
+    return SGLQ_EINVAL;
+  }
+  FastDiv fd;
+  fd.init((uint32_t)gpr);
+  const float qmax = 448.0f;
+  const dim3 grid((uint32_t)((ng + 31) / 32)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const char* xi = static_cast<const char*>(input);
+  char* qo = static_cast<char*>(output_q);
+#define SGLQ_SCATTER(DT)                                                                                               \
+  group_quant_scatter_kernel<DT><<<grid, block, 0, st>>>(xi, qo, output_s, slot_map, (uint32_t)ng, fd, (int)topk, num_dst_rows, \
+                                                         eps, qmax, 1.0f / qmax)
+  if (in_dtype == SGLQ_BF16) SGLQ_SCATTER(SGLQ_BF16);
+  else if (in_dtype == SGLQ_FP16) SGLQ_SCATTER(SGLQ_FP16);
+  else if (in_dtype == SGLQ_FP32) SGLQ_SCATTER(SGLQ_FP32);
+  else {
+    set_error("%s: unsupported in_dtype %d", name, in_dtype);
+    return SGLQ_EUNSUPPORTED;
+  }
+#undef SGLQ_SCATTER
+  return check_launch(name);
+}
 
 extern "C" int sglq_silu_and_mul_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
                                                  int64_t num_tokens, int64_t d, float eps, void* stream) {

@@ -223,3 +223,28 @@ def silu_and_mul_per_token_group_quant_fp8(input: torch.Tensor, group_size: int 
                                                        tokens, d, eps, _lib.stream_ptr(input.device))
     _lib.check(rc, "silu_and_mul_per_token_group_quant_fp8")
     return out_q, out_s
+
+
+def per_token_group_quant_fp8_to_expert_rows(x: torch.Tensor, slot_map: torch.Tensor, topk: int, group_size: int = 128,
+                                             eps: float = 1e-10):
+    """sglang_per_token_group_quant_fp8(x, 128) followed by shuffle_rows of codes and scales with
+    a_map (python/sglang/srt/layers/moe/cutlass_moe.py:156-158) in one kernel: token t is quantized
+    once and written to the rows slot_map[t * topk + j], j < topk (slot_map = prepare_moe_input's
+    output_permutation; entries outside [0, m * topk) are skipped and rows that no slot names stay
+    uninitialised).  x [m, k] Half / BFloat16 / Float; returns (codes [m * topk, k] e4m3fn, scales
+    [m * topk, k / 128] fp32 row-major), bit-identical to the three calls on every row a slot names."""
+    if group_size != 128:
+        raise NotImplementedError("per_token_group_quant_fp8_to_expert_rows: group size 128 is built")
+    _check(x.is_cuda and x.dim() == 2 and x.is_contiguous(), "x must be a contiguous 2D CUDA tensor")
+    _check(x.dtype in DTYPE_CODE, "x must be Float, Half or BFloat16")
+    _check(x.size(1) % 128 == 0, "the last dimension must be divisible by group_size")
+    _cuda_int32("slot_map", slot_map)
+    m, k = x.shape
+    _check(topk > 0 and slot_map.numel() >= m * topk, "slot_map must hold m * topk entries")
+    out_q = torch.empty((m * topk, k), device=x.device, dtype=FP8)
+    out_s = torch.empty((m * topk, k // 128), device=x.device, dtype=torch.float32)
+    rc = _lib.load().sglq_per_token_group_quant_fp8_scatter(x.data_ptr(), DTYPE_CODE[x.dtype], out_q.data_ptr(), out_s.data_ptr(),
+                                                            slot_map.data_ptr(), m, k, int(topk), m * topk, eps,
+                                                            _lib.stream_ptr(x.device))
+    _lib.check(rc, "per_token_group_quant_fp8_to_expert_rows")
+    return out_q, out_s

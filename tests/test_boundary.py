@@ -198,6 +198,10 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.sglq_silu_and_mul_group_quant_fp8(p, 2, p, p, 4, 128, 1e-10, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
     assert lib.sglq_silu_and_mul_group_quant_fp8(p, 0, p, None, 4, 128, 1e-10, None) == 1 and b"null" in lib.sglq_last_error()
     assert lib.sglq_silu_and_mul_group_quant_fp8(p, 0, p, p, 0, 128, 1e-10, None) == 0
+    assert lib.sglq_per_token_group_quant_fp8_scatter(p, 0, p, p, p, 4, 200, 2, 8, 1e-10, None) == 1 and b"multiple of 128" in lib.sglq_last_error()
+    assert lib.sglq_per_token_group_quant_fp8_scatter(p, 0, p, p, None, 4, 128, 2, 8, 1e-10, None) == 1 and b"null" in lib.sglq_last_error()
+    assert lib.sglq_per_token_group_quant_fp8_scatter(p, 5, p, p, p, 4, 128, 2, 8, 1e-10, None) == 2 and b"in_dtype" in lib.sglq_last_error()
+    assert lib.sglq_per_token_group_quant_fp8_scatter(p, 0, p, p, p, 0, 128, 2, 0, 1e-10, None) == 0
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 0, 8, 8, None) == 1 and b"bad sizes" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 2, 12, 8, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 2, 4, 2, 8, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()

@@ -170,6 +170,47 @@ def test_silu_and_mul_fused_with_group_quant(gpu, dtype, tokens, d):
         silu_and_mul_per_token_group_quant_fp8(torch.zeros((2, 256), dtype=torch.float32, device=gpu))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.half, torch.float32])
+@pytest.mark.parametrize("m,topk,e,k", [(1, 1, 1, 128), (9, 2, 4, 256), (333, 8, 32, 384), (2048, 6, 16, 1024)])
+def test_group_quant_written_to_expert_rows(gpu, dtype, m, topk, e, k):
+    """One kernel for the per-token-group quantization and the two row gathers after it: on every
+    row that a slot names, codes and scales equal those of the three operators called in turn, bit
+    for bit; rows that no slot names (ids outside [0, E)) are not written."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import shuffle_rows
+    from sglang_amd.sgl_kernel.moe import per_token_group_quant_fp8_to_expert_rows
+
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn((m, k), generator=g) * 2).to(dtype)
+    x[0, :128] = 0
+    ids = torch.randint(0, e, (m, topk), generator=g, dtype=torch.int32)
+    if m > 4:
+        ids[1, 0] = -1
+        ids[m - 1, topk - 1] = e
+    say("group quant to expert rows", dtype, m, topk, e, k)
+    offsets, _, _, _, a_map, c_map = run_prepare(gpu, ids, e, 64, k, fill=-1)
+    total = int(offsets[-1])
+    xg, a_map, c_map = x.to(gpu), a_map.to(gpu), c_map.to(gpu)
+    q, s = sglang_per_token_group_quant_fp8(xg, 128)
+    want_q, want_s = shuffle_rows(q, a_map, (m * topk, k)), shuffle_rows(s, a_map, (m * topk, k // 128))
+    got_q, got_s = per_token_group_quant_fp8_to_expert_rows(xg, c_map, topk, 128)
+    assert got_q.shape == (m * topk, k) and got_s.shape == (m * topk, k // 128)
+    assert_bits_equal(got_q[:total], want_q[:total], "codes")
+    assert_bits_equal(got_s[:total], want_s[:total], "scales")
+    # nothing outside the named rows: through the C ABI into sentinel-filled buffers
+    from sglang_amd import _lib
+    from sglang_amd._lib import DTYPE_CODE
+
+    out_q = torch.full((m * topk + 2, k), 0x55, dtype=torch.uint8, device=gpu)
+    out_s = torch.full((m * topk + 2, k // 128), -3.0, dtype=torch.float32, device=gpu)
+    rc = _lib.load().sglq_per_token_group_quant_fp8_scatter(xg.data_ptr(), DTYPE_CODE[dtype], out_q[1:].data_ptr(), out_s[1:].data_ptr(),
+                                                            c_map.data_ptr(), m, k, topk, m * topk, 1e-10, _lib.stream_ptr(gpu))
+    assert rc == 0
+    assert torch.equal(out_q[1:1 + total], want_q[:total].view(torch.uint8))
+    assert bool((out_q[0] == 0x55).all()) and bool((out_q[1 + total:] == 0x55).all())
+    assert bool((out_s[0] == -3.0).all()) and bool((out_s[1 + total:] == -3.0).all())
+
+
 def test_silu_and_mul_argument_checks(gpu):
     from sglang_amd.sgl_kernel import silu_and_mul
 
