@@ -261,6 +261,22 @@ int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, c
                        const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
                        int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Tuned kernel selections, the counterpart of the reference's per-(N, K) JSON tables for its
+ * Triton GEMMs (get_w8a8_block_fp8_configs, python/sglang/srt/layers/quantization/fp8_kernel.py:
+ * 738-776, files under layers/quantization/configs/): for GEMMs of `kind` with exactly these N and
+ * K and m_lo <= M <= m_hi, use kernel `tile` (a code of sglq_debug_force_tile, 0 = by shape) and
+ * split-K factor `splits` (0 = by shape) instead of the built-in heuristics.  The first matching
+ * entry wins; a kernel that does not apply to a shape falls through to the next one that does, so
+ * no entry can make a call fail.  Results do not depend on the table beyond the summation order
+ * that each kernel has anyway.  Fill the table before GEMMs are launched from other threads. */
+#define SGLQ_KIND_FP8_BLOCK 0  /* sglq_fp8_blockwise_scaled_mm(_bias) */
+#define SGLQ_KIND_FP8_ROWCOL 1 /* sglq_fp8_scaled_mm */
+#define SGLQ_KIND_I8_ROWCOL 2  /* sglq_int8_scaled_mm */
+#define SGLQ_KIND_I8_RAW 3     /* sglq_int8_mm_i32 */
+#define SGLQ_KIND_I8_BLOCK 4   /* sglq_int8_blockwise_scaled_mm(_bias) */
+int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits);
+int sglq_tuned_clear(void);
+
 /* Test hook without a reference counterpart: non-zero (default) makes the GEMMs
  * copy global memory straight into LDS with buffer loads, zero stages the same
  * bytes through registers.  Both must give identical results. */

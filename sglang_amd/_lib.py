@@ -41,6 +41,8 @@ SIGNATURES = {
                                c_int64, c_void_p],
     "sglq_shuffle_rows": [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p],
     "sglq_silu_and_mul": [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p],
+    "sglq_tuned_add": [c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int],
+    "sglq_tuned_clear": [],
     "sglq_per_token_group_quant_fp8_scatter": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_void_p],
     "sglq_silu_and_mul_group_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p],
     "sglq_apply_shuffle_mul_sum": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p],
@@ -86,6 +88,11 @@ def load() -> ctypes.CDLL:
     lib.sglq_debug_last_gemm_kernel.argtypes = []
     lib.sglq_debug_last_gemm_kernel.restype = ctypes.c_char_p
     _lib = lib
+    if os.environ.get("SGLQ_NO_TUNED_CONFIGS", "0") != "1":
+        # per-(N, K) kernel selections shipped beside the package (sglang_amd/quantization/configs/)
+        from .quantization.tuned_configs import load_tuned_configs
+
+        load_tuned_configs()
     return lib
 
 

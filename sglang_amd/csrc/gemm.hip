@@ -1920,6 +1920,9 @@ static int num_cus() {
 }
 
 static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
+// The selection in force for the call being launched on this thread: the test hooks, else a
+// matching entry of the tuned table, else 0 = the built-in heuristics.
+static thread_local int t_tile = 0, t_splits = 0;
 static int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile, 130 = 128 rows pipelined (0 = from the average group)
 static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
 
@@ -2001,7 +2004,7 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     if (splits > by_steps) splits = by_steps;
     if (splits > by_traffic) splits = (int)(by_traffic > 0 ? by_traffic : 1);
   }
-  if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
+  if (t_splits > 0) splits = t_splits < nkb ? t_splits : nkb;
   const int64_t per_split = (int64_t)p.M * p.N * 4;
   if (!p.ws || ws_bytes < per_split * 2) splits = 1;
   else if (splits * per_split > ws_bytes) splits = (int)(ws_bytes / per_split);
@@ -2020,6 +2023,8 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 // 130 = the pipelined kernel with 128-row tiles (K >= 384, else the 128 x 128 kernel)
 static int g_force_tile = 0;
 
+static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws_bytes, int& splits);
+
 template <int KIND, int OUT_DT>
 static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + 255) / 256;
@@ -2028,25 +2033,26 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // persistent: one block per CU walks the tiles blockIdx, blockIdx + gridDim, ...
   const int tiles = p.tiles_m * p.tiles_n;
   // the pipelined kernel needs three K blocks; 256 forces the plain one (test hook)
-  if (g_force_tile != 256 && p.K >= 384) {
+  if (t_tile != 256 && p.K >= 384) {
     // Too few tiles for the chip: split K into equal contiguous ranges of at least four K
     // blocks, as many as fill the CUs and the workspace holds; the partial sums cost
     // 8 M N splits bytes of traffic, which must stay well under the operands'.
     const int nkb = p.K >> 7;
     int splits = 1;
-    if (2 * tiles <= num_cus() || g_force_splits > 0) {
-      int want = g_force_splits > 0 ? g_force_splits : num_cus() / tiles;
+    if (t_splits > 0) {
+      int want = t_splits;
       const int64_t per_split = (int64_t)p.M * p.N * 4;
       // (the kernel addresses a split's partial sums, tile padding included, with 31 bits)
       if (!p.ws || ws_bytes < 2 * per_split || (int64_t)(p.M + 256) * p.N * 4 >= (int64_t)1 << 31) want = 1;
       else if (want * per_split > ws_bytes) want = (int)(ws_bytes / per_split);
-      const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
-      if (g_force_splits == 0 && want > by_traffic) want = (int)(by_traffic > 0 ? by_traffic : 1);
       for (int s = want; s >= 2; --s)
-        if (nkb % s == 0 && nkb / s >= (g_force_splits > 0 ? 3 : 4)) {
+        if (nkb % s == 0 && nkb / s >= 3) {
           splits = s;
           break;
         }
+    } else if (2 * tiles <= num_cus()) {
+      // too few tiles for the chip: equal contiguous K ranges, as many as the cost model favours
+      model_pipe_splits(p, 256, ws_bytes, splits);
     }
     p.splits = splits;
     const int units = tiles * splits;
@@ -2072,7 +2078,34 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   }
 }
 
-// The pipelined kernel with 128-row tiles: (tile, K range) work units, about one per CU.
+// Split-K factor of the pipelined kernel by a cost model in microseconds, fitted to measurements
+// over M = 256 ... 3072 on the DeepSeek-V3 and Llama-70B shapes: the work units (tiles x splits)
+// run in rounds over the CUs; a unit costs its K steps (0.85 us each with 128-row tiles, 1.3 us
+// with 256-row tiles) plus a fixed 8 / 10 us (the first blocks' arrival, the epilogue); splitting
+// adds the reduction launch (4 us) and the partial sums' round trip (8 M N s bytes at 5 TB/s).
+// Returns the modelled time; `splits` gets the factor (a divisor of the K blocks, at least four per unit).
+static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws_bytes, int& splits) {
+  const int tiles = ((p.M + rows_per_tile - 1) / rows_per_tile) * ((p.N + 255) / 256);
+  const int nkb = p.K >> 7;
+  const double step_us = rows_per_tile == 128 ? 0.85 : 1.3, fixed_us = rows_per_tile == 128 ? 8.0 : 10.0;
+  const int64_t per_split = (int64_t)p.M * p.N * 4;
+  const bool can_split = p.ws && ws_bytes >= 2 * per_split && (int64_t)(p.M + 256) * p.N * 4 < ((int64_t)1 << 31);
+  double best = 1e30;
+  splits = 1;
+  for (int s = 1; s <= 16; ++s) {
+    if (s > 1 && (!can_split || nkb % s != 0 || nkb / s < 4 || s * per_split > ws_bytes)) continue;
+    const int rounds = (tiles * s + num_cus() - 1) / num_cus();
+    double cost = rounds * ((nkb / s) * step_us + fixed_us);
+    if (s > 1) cost += 4.0 + 8.0 * p.M * p.N * s / 5e6;
+    if (cost < best) {
+      best = cost;
+      splits = s;
+    }
+  }
+  return best;
+}
+
+// The pipelined kernel with 128-row tiles: (tile, K range) work units.
 template <int KIND, int OUT_DT>
 static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + 127) / 128;
@@ -2080,18 +2113,18 @@ static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const int tiles = p.tiles_m * p.tiles_n;
   const int nkb = p.K >> 7;
   int splits = 1;
-  if (tiles < num_cus() || g_force_splits > 0) {
-    int want = g_force_splits > 0 ? g_force_splits : (num_cus() + tiles / 2) / tiles;
+  if (t_splits > 0) {
     const int64_t per_split = (int64_t)p.M * p.N * 4;
+    int want = t_splits;
     if (!p.ws || ws_bytes < 2 * per_split || (int64_t)(p.M + 256) * p.N * 4 >= (int64_t)1 << 31) want = 1;
     else if (want * per_split > ws_bytes) want = (int)(ws_bytes / per_split);
-    const int64_t by_traffic = ((int64_t)(p.M + p.N) * p.K) / (8 * (int64_t)p.M * p.N / 2 + 1);
-    if (g_force_splits == 0 && want > by_traffic) want = (int)(by_traffic > 0 ? by_traffic : 1);
     for (int s = want; s >= 2; --s)
-      if (nkb % s == 0 && nkb / s >= (g_force_splits > 0 ? 3 : 4)) {
+      if (nkb % s == 0 && nkb / s >= 3) {
         splits = s;
         break;
       }
+  } else {
+    model_pipe_splits(p, 128, ws_bytes, splits);
   }
   p.splits = splits;
   const int units = tiles * splits;
@@ -2166,7 +2199,7 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
   if (splits > by_steps) splits = by_steps;
   if (splits < 1) splits = 1;
-  if (g_force_splits > 0) splits = g_force_splits < nkb ? g_force_splits : nkb;
+  if (t_splits > 0) splits = t_splits < nkb ? t_splits : nkb;
   const int64_t per_split = (int64_t)p.M * p.N * 4;
   if (!p.ws || ws_bytes < per_split * 2) splits = 1;
   else if (splits * per_split > ws_bytes) splits = (int)(ws_bytes / per_split);
@@ -2186,10 +2219,12 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   // 16-row blocks win for M <= 16 up to N = 16384, 32-row blocks beyond and for M > 16.  With
   // fewer K blocks a wave's ring never fills and the split-K kernel is faster.
   int nib = 0;
-  if (g_force_tile == 16) nib = 1;
-  else if (g_force_tile == 32) nib = 2;
+  if (t_tile == 16) nib = 1;
+  else if (t_tile == 32) nib = 2;
   else if (p.K >= 2048) {
-    nib = (p.M <= 16 && p.N <= 16384) ? 1 : 2;
+    // (measured: 16-row blocks up to M = 8 whatever N, e.g. 8 x 57344 x 8192 83 against 93 us; at M = 16 up to
+    // N = 16384; for 16 < M <= 32 only on small N, e.g. 32 x 4096 x 7168 8.4 against 9.1 us)
+    nib = (p.M <= 8 || (p.M <= 16 && p.N <= 16384) || p.N <= 4096) ? 1 : 2;
     if (p.N < 64 * 16 * nib) nib = 0;
   }
   if (nib == 0) return false;
@@ -2208,16 +2243,48 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   return true;
 }
 
+// Tuned kernel selections per problem, the counterpart of the reference's per-(N, K) JSON
+// tables for its Triton kernels (python/sglang/srt/layers/quantization/fp8_kernel.py:738-776,
+// layers/quantization/configs/): an entry names the kernel (a code of sglq_debug_force_tile)
+// and the split-K factor for kind, N, K and a range of M.  Filled once at start-up through
+// sglq_tuned_add (not while GEMMs are being launched from other threads); read-only afterwards.
+struct TunedEntry {
+  int kind;
+  int64_t n, k, m_lo, m_hi;
+  int tile, splits;
+};
+constexpr int MAX_TUNED = 1024;
+static TunedEntry g_tuned[MAX_TUNED];
+static int g_num_tuned = 0;
+
+static const TunedEntry* tuned_lookup(int kind, int64_t m, int64_t n, int64_t k) {
+  for (int i = 0; i < g_num_tuned; ++i) {
+    const TunedEntry& e = g_tuned[i];
+    if (e.kind == kind && e.n == n && e.k == k && m >= e.m_lo && m <= e.m_hi) return &e;
+  }
+  return nullptr;
+}
+
 template <int KIND, int OUT_DT>
 static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
-  if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (g_force_tile == 0 || g_force_tile == 16 || g_force_tile == 32) &&
+  t_tile = g_force_tile;
+  t_splits = g_force_splits;
+  if (t_tile == 0 && t_splits == 0 && g_num_tuned > 0) {
+    if (const TunedEntry* e = tuned_lookup(KIND, p.M, p.N, p.K)) {
+      t_tile = e->tile;
+      t_splits = e->splits;
+    }
+  }
+  if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (t_tile == 0 || t_tile == 16 || t_tile == 32) &&
       launch_stream<KIND, OUT_DT>(p, st))
     return;
   // ... and up to 128 rows (two 64-row tiles side by side) with K <= 8192 it still beats the
   // 128 x 128 kernel (measured, e.g. 128 x 24576 x 1536: 28.3 -> 16.3 us, 128 x 4096 x 7168:
   // 21.2 -> 17.9 us; at K = 16384 the 128 x 128 kernel wins, 35 against 49 us).
-  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192) || (g_force_tile == 64 && p.M <= 512);
-  if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (g_force_tile == 0 || g_force_tile == 64)) {
+  // (not with large weights: 96 x 57344 x 8192 takes 194 us there against 115 us on the pipelined kernel)
+  const int64_t weight_bytes = (int64_t)p.N * p.K;
+  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) || (t_tile == 64 && p.M <= 512);
+  if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
@@ -2228,10 +2295,16 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // ... unless the problem is large and deep enough for the pipelined kernel with K split over
   // (tile, K range) units: 512 x 7168 x 16384 90.6 -> 75.6 us, 1024 x 7168 x 16384 164.5 -> 122.6 us,
   // but 1024 x 4096 x 7168 49 -> 56 us (measured).
-  const bool deep = p.M > 256 && (p.K >> 7) >= 64 && 2.0 * p.M * p.N * p.K >= 1e11;
-  const bool forced_256 = g_force_tile == 256 || g_force_tile == 258 || g_force_tile == 192 || g_force_tile == 224 || g_force_tile == 257;
-  if ((p.K & 127) == 0 && (forced_256 || (g_force_tile == 0 && g_use_dma && p.M > 64 && (big_tiles >= 140 || deep)))) {
-    int width = g_force_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p) : 256) : g_force_tile;
+  bool deep = p.M > 256 && (p.K >> 7) >= 64 && 2.0 * p.M * p.N * p.K >= 1e11;
+  if (deep && big_tiles < 140 && t_tile == 0 && p.K >= 384) {
+    // ... and the 128-row tiles do not fill the chip better (1024 x 8192 x 8192: 81 us with 256-row tiles and
+    // K split in two, 66 us with 128-row tiles, one per CU)
+    int s128, s256;
+    if (model_pipe_splits(p, 128, ws_bytes, s128) < model_pipe_splits(p, 256, ws_bytes, s256)) deep = false;
+  }
+  const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 192 || t_tile == 224 || t_tile == 257;
+  if ((p.K & 127) == 0 && (forced_256 || (t_tile == 0 && g_use_dma && p.M > 64 && (big_tiles >= 140 || deep)))) {
+    int width = t_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p) : 256) : t_tile;
     if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
@@ -2243,8 +2316,8 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // Measured against the 128 x 128 kernel: 256 x 7168 x 16384 64 -> 44 us, 1024 x 7168 x 2048
   // 26 -> 20 us, 2048 x 4096 x 7168 74 -> 58 us, 2048 x 2112 x 7168 64 -> 48 us; below 256 rows
   // it only wins on large weights (256 x 24576 x 1536 22 -> 17 us, but 256 x 2112 x 7168 19 -> 21 us).
-  const bool mid = p.M > 256 || (p.M > 128 && (int64_t)p.N * p.K >= (24 << 20));
-  if ((p.K & 127) == 0 && p.K >= 384 && (g_force_tile == 130 || (g_force_tile == 0 && g_use_dma && mid))) {
+  const bool mid = p.M > 256 || (p.M > 128 && weight_bytes >= (24 << 20)) || (p.M > 64 && weight_bytes >= (48 << 20));
+  if ((p.K & 127) == 0 && p.K >= 384 && (t_tile == 130 || (t_tile == 0 && g_use_dma && mid))) {
     launch_pipe128<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
@@ -2322,6 +2395,26 @@ using namespace sglq;
 extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
+extern "C" int sglq_tuned_clear(void) {
+  g_num_tuned = 0;
+  return SGLQ_OK;
+}
+extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
+  static const int tiles[] = {0, 16, 32, 64, 128, 130, 192, 224, 256, 257, 258};
+  bool known = false;
+  for (int t : tiles) known = known || t == tile;
+  if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {
+    set_error("tuned_add: kind 0..4, positive N and K, 0 <= m_lo <= m_hi, a known kernel code and 0 <= splits <= 64 expected");
+    return SGLQ_EINVAL;
+  }
+  if (g_num_tuned >= MAX_TUNED) {
+    set_error("tuned_add: the table holds %d entries", MAX_TUNED);
+    return SGLQ_EUNSUPPORTED;
+  }
+  g_tuned[g_num_tuned++] = TunedEntry{kind, N, K, m_lo, m_hi, tile, splits};
+  return SGLQ_OK;
+}
+
 extern "C" void sglq_debug_grouped_tile(int rows) {
   g_grouped_tile = (rows == 32 || rows == 64 || rows == 128 || rows == 130 || rows == 256) ? rows : 0;
 }

@@ -1,0 +1,117 @@
+"""Tunes the kernel selection of the block-scaled FP8 GEMM for given (N, K) over a grid of batch
+sizes and writes the table that tuned_configs.load_tuned_configs reads: the counterpart of the
+reference's benchmark/kernels/quantization/tuning_block_wise_kernel.py for its Triton kernel.
+
+    python -m sglang_amd.quantization.tune_block_fp8 --N 4096 --K 7168 [--M 1 8 64 ...] [--out DIR]
+
+Every candidate (kernel code, split-K factor) is timed from HIP-graph replays with the weights
+rotated through more than the last-level cache; an entry is written only where a candidate beats
+the built-in selection by more than --margin (default 3 %), otherwise {"tile": 0, "splits": 0}."""
+
+from __future__ import annotations
+
+import argparse
+import json
+
+import torch
+
+DEFAULT_M = [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 256, 512, 1024, 1536, 2048, 3072, 4096, 8192]
+
+
+def candidates(m: int, n: int, k: int):
+    """(tile code, splits) pairs worth timing for this shape."""
+    out = [(0, 0)]
+    nkb = k // 128
+    if k % 128:
+        return out
+    if m <= 32 and k >= 512:
+        out += [(16, 0), (32, 0)]
+    if m <= 512:
+        out += [(64, s) for s in (0, 2, 4, 8) if s == 0 or s <= nkb // 2]
+    out += [(128, s) for s in (0, 2, 4) if s == 0 or s <= nkb // 4]
+    if k >= 384 and m > 64:
+        out += [(130, s) for s in (0, 1, 2, 4, 8) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]
+        out += [(258, s) for s in (0, 1, 2, 4) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]
+        if m > 256:
+            out += [(192, 0), (224, 0), (257, 0)]
+    return out
+
+
+def tune(n: int, k: int, ms, iters: int, margin: float, dev):
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lib = _lib.load()
+    lib.sglq_tuned_clear()
+    g = torch.Generator(device=dev).manual_seed(n + k)
+    w = (torch.randn((n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
+    ws = torch.rand(((n + 127) // 128, (k + 127) // 128), generator=g, device=dev) * 1e-2 + 1e-3
+    copies = max(1, min(8, int(600e6 // (n * k))))
+    wq = [w] + [w.clone() for _ in range(copies - 1)]
+    table = {}
+    for m in ms:
+        a = (torch.randn((m, k), generator=g, device=dev) * 2).to(torch.float8_e4m3fn)
+        sa = (torch.rand((k // 128, m), generator=g, device=dev) * 1e-2 + 1e-3).t()  # column-major [m, k / 128]
+
+        def run(j):
+            return fp8_blockwise_scaled_mm(a, wq[j].t(), sa, ws.t(), torch.bfloat16)
+
+        def time_it():
+            for j in range(max(2, copies)):
+                run(j % copies)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(iters):
+                    run(i % copies)
+            graph.replay()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            best = float("inf")
+            for _ in range(3):
+                s.record()
+                graph.replay()
+                e.record()
+                torch.cuda.synchronize()
+                best = min(best, s.elapsed_time(e) / iters)
+            return best
+
+        results = {}
+        try:
+            for tile, splits in candidates(m, n, k):
+                lib.sglq_debug_force_tile(tile)
+                lib.sglq_debug_force_splits(splits)
+                results[(tile, splits)] = (time_it(), lib.sglq_debug_last_gemm_kernel().decode())
+        finally:
+            lib.sglq_debug_force_tile(0)
+            lib.sglq_debug_force_splits(0)
+        base = results[(0, 0)][0]
+        (tile, splits), (t, name) = min(results.items(), key=lambda kv: kv[1][0])
+        if t < base * (1.0 - margin):
+            table[m] = {"tile": tile, "splits": splits}
+        else:
+            table[m] = {"tile": 0, "splits": 0}
+        print(json.dumps({"M": m, "N": n, "K": k, "default_us": round(base * 1e3, 2), "default_kernel": results[(0, 0)][1],
+                          "best_us": round(t * 1e3, 2), "best": [tile, splits], "best_kernel": name, "chosen": table[m]}), flush=True)
+    return table
+
+
+def main():
+    from sglang_amd.quantization.tuned_configs import save_config
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--N", type=int, required=True)
+    ap.add_argument("--K", type=int, required=True)
+    ap.add_argument("--M", type=int, nargs="*", default=DEFAULT_M)
+    ap.add_argument("--iters", type=int, default=8)
+    ap.add_argument("--margin", type=float, default=0.03)
+    ap.add_argument("--out", type=str, default=None, help="directory for the table (default: the package's configs/)")
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    table = tune(args.N, args.K, args.M, args.iters, args.margin, dev)
+    path = save_config(args.N, args.K, table, args.out)
+    print("wrote", path)
+
+
+if __name__ == "__main__":
+    main()

@@ -208,3 +208,40 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 0, 2, 8, 8, None) == 0
     # empty problems are a no-op
     assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0
+
+
+def test_tuned_config_tables(tmp_path):
+    """Per-(N, K) kernel selections (the counterpart of fp8_kernel.py:738-776): file naming, the
+    closest-M rule turned into ranges, and what the library's table accepts."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization import tuned_configs as T
+
+    name = T.config_file_name(4096, 7168)
+    assert name == "N=4096,K=7168,device_name=AMD_Instinct_MI355X,dtype=fp8_w8a8,block_shape=[128, 128].json"
+    assert T.parse_file_name(name) == (4096, 7168, "AMD_Instinct_MI355X", "fp8_w8a8")
+    assert T.parse_file_name("README.md") is None
+    table = {1: {"tile": 16, "splits": 0}, 64: {"tile": 64, "splits": 4}, 512: {"tile": 0, "splits": 0}, 4096: {"tile": 258, "splits": 1}}
+    assert T.ranges_of(table) == [(0, 32, 16, 0), (33, 288, 64, 4), (289, 2304, 0, 0), (2305, T.M_MAX, 258, 1)]
+    # every M goes to its closest key, ties to the smaller one
+    for m in (1, 32, 33, 288, 289, 2304, 2305, 100000):
+        closest = min(sorted(table), key=lambda key: abs(key - m))
+        lo_hi = [r for r in T.ranges_of(table) if r[0] <= m <= r[1]]
+        assert len(lo_hi) == 1 and lo_hi[0][2] == table[closest]["tile"], m
+    path = T.save_config(4096, 7168, table, tmp_path)
+    assert path.name == name and T.get_w8a8_block_fp8_configs(4096, 7168, 128, 128, tmp_path) == table
+    assert T.get_w8a8_block_fp8_configs(4096, 7168, 64, 64, tmp_path) is None
+    assert T.get_w8a8_block_fp8_configs(1, 2, 128, 128, tmp_path) is None
+    T.save_config(2048, 512, {8: {"tile": 128, "splits": 2}}, tmp_path, dtype="int8_w8a8")
+    (tmp_path / "N=8,K=8,device_name=other,dtype=fp8_w8a8,block_shape=[128, 128].json").write_text('{"1": {"tile": 64, "splits": 0}}')
+    try:
+        assert T.load_tuned_configs(tmp_path) == 4  # three selections of the first table, one of the second; the other device's file is skipped
+        lib = _lib.load()
+        assert lib.sglq_tuned_add(0, 4096, 7168, 0, 10, 77, 0) == 1 and b"known kernel code" in lib.sglq_last_error()
+        assert lib.sglq_tuned_add(9, 4096, 7168, 0, 10, 64, 0) == 1
+        assert lib.sglq_tuned_add(0, 4096, 7168, 11, 10, 64, 0) == 1
+        assert lib.sglq_tuned_clear() == 0
+        for i in range(1024):
+            assert lib.sglq_tuned_add(0, 128 * (i + 1), 128, 0, 10, 64, 0) == 0
+        assert lib.sglq_tuned_add(0, 128, 128, 0, 10, 64, 0) == 2 and b"1024 entries" in lib.sglq_last_error()
+    finally:
+        T.load_tuned_configs()  # back to the tables shipped with the package

@@ -484,3 +484,42 @@ def test_gemm_empty_m(gpu):
     w = torch.zeros((16, 128), dtype=torch.int8, device=gpu)
     out = int8_scaled_mm(a, w.t(), torch.empty((0, 1), device=gpu), torch.ones((16, 1), device=gpu), torch.bfloat16)
     assert tuple(out.shape) == (0, 16)
+
+
+def test_tuned_table_selects_the_kernel(gpu):
+    """An entry of the tuned table (the counterpart of the reference's per-(N, K) JSON configs) picks
+    the kernel and split-K factor for its N, K and range of M only; the test hooks still override it;
+    the results stay within tolerance of the oracle whatever kernel runs."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization.tuned_configs import load_tuned_configs
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lib = _lib.load()
+    m, n, k = 300, 512, 1024
+    x, xq, xs, wq, ws = make_block_case(m, n, k, seed=31)
+    args = (xq.to(gpu), wq.to(gpu).t(), xs.to(gpu).t().contiguous().t(), ws.to(gpu).t(), torch.bfloat16)
+    ref = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32, acc_dtype=torch.float64)
+    try:
+        lib.sglq_tuned_clear()
+        fp8_blockwise_scaled_mm(*args)
+        default_kernel = lib.sglq_debug_last_gemm_kernel().decode()
+        other_n = (args[0], args[1][:, :256], args[2], args[3][:, :2], torch.bfloat16)
+        fp8_blockwise_scaled_mm(*other_n)
+        default_other_n = lib.sglq_debug_last_gemm_kernel().decode()
+        assert lib.sglq_tuned_add(0, n, k, 200, 400, 258, 1) == 0   # this shape: the pipelined 256 x 256 kernel
+        assert lib.sglq_tuned_add(0, n, k, 0, 199, 64, 2) == 0      # smaller M of the same (N, K)
+        assert lib.sglq_tuned_add(4, n, k, 0, 1 << 30, 128, 0) == 0  # another kind: no effect here
+        out = fp8_blockwise_scaled_mm(*args)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_pipe_kernel" != default_kernel
+        torch.testing.assert_close(out.cpu().float(), ref, rtol=RTOL, atol=ATOL)
+        small = fp8_blockwise_scaled_mm(args[0][:50], args[1], args[2][:50], args[3], torch.bfloat16)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_skinny_kernel+splitk_reduce_kernel"
+        torch.testing.assert_close(small.cpu().float(), ref[:50], rtol=RTOL, atol=ATOL)
+        fp8_blockwise_scaled_mm(*other_n)  # another N: no entry
+        assert lib.sglq_debug_last_gemm_kernel().decode() == default_other_n != "gemm_pipe_kernel"
+        lib.sglq_debug_force_tile(128)
+        fp8_blockwise_scaled_mm(*args)
+        assert lib.sglq_debug_last_gemm_kernel().decode().startswith("gemm_kernel")
+    finally:
+        lib.sglq_debug_force_tile(0)
+        load_tuned_configs()
