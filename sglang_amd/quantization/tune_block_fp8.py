@@ -6,7 +6,8 @@ reference's benchmark/kernels/quantization/tuning_block_wise_kernel.py for its T
 
 Every candidate (kernel code, split-K factor) is timed from HIP-graph replays with the weights
 rotated through more than the last-level cache; an entry is written only where a candidate beats
-the built-in selection by more than --margin (default 3 %), otherwise {"tile": 0, "splits": 0}."""
+the built-in selection by more than --margin (default 4 %; its slowest of three runs against the built-in
+selection's fastest of three), otherwise {"tile": 0, "splits": 0}."""
 
 from __future__ import annotations
 
@@ -77,16 +78,26 @@ def tune(n: int, k: int, ms, iters: int, margin: float, dev):
             return best
 
         results = {}
+
+        def timed(tile, splits):
+            lib.sglq_debug_force_tile(tile)
+            lib.sglq_debug_force_splits(splits)
+            return time_it(), lib.sglq_debug_last_gemm_kernel().decode()
+
         try:
             for tile, splits in candidates(m, n, k):
-                lib.sglq_debug_force_tile(tile)
-                lib.sglq_debug_force_splits(splits)
-                results[(tile, splits)] = (time_it(), lib.sglq_debug_last_gemm_kernel().decode())
+                results[(tile, splits)] = timed(tile, splits)
+            (tile, splits), (t, name) = min(results.items(), key=lambda kv: kv[1][0])
+            base = results[(0, 0)][0]
+            if (tile, splits) != (0, 0) and t < base * (1.0 - margin):
+                # the same pair measured twice can differ by a few per cent: confirm the winner against the
+                # built-in selection in alternation before it is written down
+                for _ in range(2):
+                    base = min(base, timed(0, 0)[0])
+                    t = max(t, timed(tile, splits)[0])
         finally:
             lib.sglq_debug_force_tile(0)
             lib.sglq_debug_force_splits(0)
-        base = results[(0, 0)][0]
-        (tile, splits), (t, name) = min(results.items(), key=lambda kv: kv[1][0])
         if t < base * (1.0 - margin):
             table[m] = {"tile": tile, "splits": splits}
         else:
@@ -104,7 +115,7 @@ def main():
     ap.add_argument("--K", type=int, required=True)
     ap.add_argument("--M", type=int, nargs="*", default=DEFAULT_M)
     ap.add_argument("--iters", type=int, default=8)
-    ap.add_argument("--margin", type=float, default=0.03)
+    ap.add_argument("--margin", type=float, default=0.04)
     ap.add_argument("--out", type=str, default=None, help="directory for the table (default: the package's configs/)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
