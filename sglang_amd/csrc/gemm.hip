@@ -1720,7 +1720,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------
-// Decode kernel for M <= 32 and N large enough to give every CU a block without
+// Decode kernel for M <= 32 (M <= 64 with 16-row blocks) and N large enough to give every CU a block without
 // splitting K across blocks: a block owns BN = 16 NIB weight rows and the whole of K; its
 // four waves take the K blocks w, w + 4, w + 8, ... and add their partial sums through LDS
 // at the end, so no workspace and no second launch are needed.  Every wave has a ring of
@@ -2210,10 +2210,13 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   else launch_skinny_mi<KIND, 4, OUT_DT>(p, st);  // (64-row tiles for any M > 32)
 }
 
-// Decode path without split-K: blocks of 16 or 32 weight rows over the whole of K.
+// Decode path without split-K: blocks of 16 or 32 weight rows over the whole of K (M <= 32; M <= 64 on small weights).
 template <int KIND, int OUT_DT>
 static bool launch_stream(GemmArgs& p, hipStream_t st) {
-  if (p.M > 32 || p.K < 512) return false;
+  // 32 < M <= 64: on weights of up to 32 MB only, where the split-K kernel's second launch and partial sums
+  // weigh most (64 x 4096 x 7168: 14.1 -> 10.3 us, 64 x 4096 x 4096: 14.8 -> 8.3 us; but 64 x 8192 x 8192: 22 -> 27 us)
+  const bool small_weight = (int64_t)p.N * p.K <= (32 << 20);
+  if (p.M > 64 || (p.M > 32 && t_tile != 16 && !(t_tile == 0 && small_weight)) || p.K < 512) return false;
   // Measured (weights rotated through more than the last-level cache): with K >= 2048 this
   // kernel beats the split-K one by 5-15 % on large N and 2x on small N (no second launch);
   // 16-row blocks win for M <= 16 up to N = 16384, 32-row blocks beyond and for M > 16.  With
@@ -2224,9 +2227,10 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   else if (p.K >= 2048) {
     // (measured: 16-row blocks up to M = 8 whatever N, e.g. 8 x 57344 x 8192 83 against 93 us; at M = 16 up to
     // N = 16384; for 16 < M <= 32 only on small N, e.g. 32 x 4096 x 7168 8.4 against 9.1 us)
-    nib = (p.M <= 8 || (p.M <= 16 && p.N <= 16384) || p.N <= 4096) ? 1 : 2;
+    nib = (p.M <= 8 || (p.M <= 16 && p.N <= 16384) || p.N <= 4096 || p.M > 32) ? 1 : 2;
     if (p.N < 64 * 16 * nib) nib = 0;
   }
+  if (p.M > 32) nib = nib == 0 ? 0 : 1;  // (64 activation rows are built with 16-row blocks only)
   if (nib == 0) return false;
   p.splits = 1;
   p.tiles_m = 1;
@@ -2236,9 +2240,11 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   if (p.M <= 16) {
     if (nib == 1) gemm_stream_kernel<KIND, 1, 1, OUT_DT><<<grid, block, 0, st>>>(p);
     else gemm_stream_kernel<KIND, 1, 2, OUT_DT><<<grid, block, 0, st>>>(p);
-  } else {
+  } else if (p.M <= 32) {
     if (nib == 1) gemm_stream_kernel<KIND, 2, 1, OUT_DT><<<grid, block, 0, st>>>(p);
     else gemm_stream_kernel<KIND, 2, 2, OUT_DT><<<grid, block, 0, st>>>(p);
+  } else {
+    gemm_stream_kernel<KIND, 4, 1, OUT_DT><<<grid, block, 0, st>>>(p);
   }
   return true;
 }
