@@ -1577,9 +1577,9 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 // flight per CU).  All copies of a stage are vector-memory loads that retire in
 // order, so "stage t has landed" is a vmcnt wait that leaves the younger stages'
 // loads outstanding.  With splits > 1 the partial sums go to a workspace and
-// splitk_reduce_kernel applies the epilogue.  For 64 < M <= 512 the grid has a second
-// dimension of 64-row tiles (blockIdx.y): the tiles of one weight tile run side by side, so
-// the weights still come from HBM once and from the caches after that.
+// splitk_reduce_kernel applies the epilogue.  For 64 < M <= 512 there are several 64-row
+// tiles per weight tile; they run side by side on one XCD, so the weights still come from
+// HBM once and from that XCD's L2 after that.
 // ---------------------------------------------------------------------------
 template <int KIND, int MI, int OUT_DT>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
@@ -1602,9 +1602,17 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4, l8 = lane >> 3;
 
-  const int tile_n = blockIdx.x % p.tiles_n, split = blockIdx.x / p.tiles_n;
+  // Block id -> (weight tile and split, row tile): the row tiles of one weight tile get ids 8 apart
+  // inside a group of eight weight tiles, so they are dispatched together and (blocks go to the
+  // eight XCDs round-robin) to the same XCD: its L2 serves the weight tile's second reader.
+  const int cols = p.tiles_n * p.splits;
+  const int group = (int)blockIdx.x / (8 * p.tiles_m);
+  const int in_group = (int)blockIdx.x - group * 8 * p.tiles_m;
+  const int width = cols - group * 8 < 8 ? cols - group * 8 : 8;
+  const int col = group * 8 + in_group % width;
+  const int tile_n = col % p.tiles_n, split = col / p.tiles_n;
   const int n0 = tile_n * BN;
-  const int m_base = (int)blockIdx.y * 64;
+  const int m_base = (in_group / width) * 64;
   const int nkb = p.K >> 7;
   // Split s takes the K blocks s, s + splits, s + 2 splits, ...: the blocks that share a
   // weight tile then read neighbouring 128-byte pieces of the same rows at about the same
@@ -2182,7 +2190,7 @@ static void launch_reduce(GemmArgs& p, hipStream_t st) {
 template <int KIND, int MI, int OUT_DT>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
   g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
-  const dim3 grid((uint32_t)(p.tiles_n * p.splits), (uint32_t)p.tiles_m), block(256);
+  const dim3 grid((uint32_t)(p.tiles_n * p.splits * p.tiles_m)), block(256);
   gemm_skinny_kernel<KIND, MI, OUT_DT><<<grid, block, 0, st>>>(p);
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
@@ -2289,7 +2297,13 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // 21.2 -> 17.9 us; at K = 16384 the 128 x 128 kernel wins, 35 against 49 us).
   // (not with large weights: 96 x 57344 x 8192 takes 194 us there against 115 us on the pipelined kernel)
   const int64_t weight_bytes = (int64_t)p.N * p.K;
-  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) || (t_tile == 64 && p.M <= 512);
+  // The kinds without block scales (no scale folds between the MFMAs) keep it longer: up to 128 rows on
+  // weights below 64 MB (128 x 14336 x 4096 INT8: 28.7 us on the pipelined kernel, 23.5 us here) and up to
+  // 512 rows on weights of up to 26 MB (512 x 4096 x 4096 FP8: 24.9 -> 19.5 us).
+  const bool plain_scales = !is_block(KIND);
+  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) ||
+                           (plain_scales && p.M <= 128 && weight_bytes < (64 << 20)) ||
+                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20)) || (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
