@@ -164,14 +164,36 @@ def run_headline(args):
         torch.cuda.synchronize()
         del src, dst
 
+    # The chip needs about 60 steps (60 ms) of this load before its step time settles (962 us per step over
+    # steps 10-20, 933 over 20-30, 890-900 from step 60 on; measured): run untimed steps for 150 ms first, so
+    # that W and K of any size see the settled clocks.  Then W untimed steps and exactly K timed ones.
+    prewarm_steps = 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < args.prewarm_ms * 1e-3:
+        step()
+        torch.cuda.synchronize()
+        prewarm_steps += 1
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    wall_graph = None
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    if args.graph:
+        # the same K steps replayed as one HIP graph, for comparison (measured: no faster than the launches above)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(args.steps):
+                step()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        wall_graph = time.perf_counter() - t0
 
     # per-kernel durations on the launch stream (separate pass so the events do not perturb the wall clock above)
     tq, tg = [Timer() for _ in layers], [Timer() for _ in layers]
@@ -238,6 +260,7 @@ def run_headline(args):
                         "{(24576,1536),(32768,512),(7168,16384),(4096,7168),(2112,7168)}: "
                         "per-token-group-128 FP8 quant + 128x128 block-scaled FP8 GEMM, bf16 in/out",
             "value_is": "sum of 2MNK over the 5 GEMMs / wall time of the whole step (quant kernels included)",
+            "prewarm": f"{prewarm_steps} untimed steps over {args.prewarm_ms} ms before the {args.warmup} warm-up steps (clock settling)",
         },
         "roofline": {
             "kernel": f"fp8_blockwise_scaled_mm: sglq::{kernel_of.get(dom, '')} (block-scaled FP8, bf16 out) on "
@@ -271,6 +294,7 @@ def run_headline(args):
             "same_launch_inside_the_step_GBs": quant_in_step_gbs,
             "all_launches_inside_the_step_GBs": round(quant_gbs, 1),
         },
+        "graph_ms_per_step": None if wall_graph is None else round(wall_graph * 1e3 / args.steps, 4),
         "per_shape": per_shape,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
@@ -512,6 +536,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (reference point for the rocprofv3 byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true", help="also time the K steps replayed as one HIP graph (graph_ms_per_step)")
+    ap.add_argument("--prewarm-ms", type=float, default=150.0, help="untimed steps for this long before the warm-up steps")
     ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--sweep-only", type=str, default=None,
