@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import time
 
 import torch
 
@@ -45,8 +46,6 @@ def tune(n: int, k: int, ms, iters: int, margin: float, dev):
     lib = _lib.load()
     lib.sglq_tuned_clear()
     # untimed load for 150 ms first: the chip's clocks take that long to settle
-    import time
-
     spin = torch.randn((4096, 4096), device=dev)
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < 0.15:
@@ -74,8 +73,12 @@ def tune(n: int, k: int, ms, iters: int, margin: float, dev):
             with torch.cuda.graph(graph):
                 for i in range(iters):
                     run(i % copies)
-            graph.replay()
-            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while True:  # untimed replays for 10 ms: a kernel timed right after a different one runs slower
+                graph.replay()
+                torch.cuda.synchronize()
+                if time.perf_counter() - t0 >= 0.01:
+                    break
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             best = float("inf")
             for _ in range(3):
