@@ -2204,7 +2204,15 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
   // more blocks only add partial-sum traffic.
   int splits = 256 / (p.tiles_n * p.tiles_m);
-  const int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
+  int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
+  if (p.tiles_m > 1) {
+    // several row tiles share a weight tile's traffic: somewhat more blocks pay (96 x 6144 x 4096: 19.3 us
+    // with two splits, 17.9 with three), no more than eight splits (96 x 1536 x 7168: 16.9 us with 13, 14.8
+    // with 8), at least four K blocks per split
+    splits = 320 / (p.tiles_n * p.tiles_m);
+    if (splits > 8) splits = 8;
+    by_steps = nkb / 4 > 0 ? nkb / 4 : 1;
+  }
   if (splits > by_steps) splits = by_steps;
   if (splits < 1) splits = 1;
   if (t_splits > 0) splits = t_splits < nkb ? t_splits : nkb;
@@ -2221,24 +2229,42 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 // Decode path without split-K: blocks of 16 or 32 weight rows over the whole of K (M <= 32; M <= 64 on small weights).
 template <int KIND, int OUT_DT>
 static bool launch_stream(GemmArgs& p, hipStream_t st) {
-  // 32 < M <= 64: on weights of up to 32 MB only, where the split-K kernel's second launch and partial sums
-  // weigh most (64 x 4096 x 7168: 14.1 -> 10.3 us, 64 x 4096 x 4096: 14.8 -> 8.3 us; but 64 x 8192 x 8192: 22 -> 27 us)
-  const bool small_weight = (int64_t)p.N * p.K <= (32 << 20);
-  if (p.M > 64 || (p.M > 32 && t_tile != 16 && !(t_tile == 0 && small_weight)) || p.K < 512) return false;
-  // Measured (weights rotated through more than the last-level cache): with K >= 2048 this
-  // kernel beats the split-K one by 5-15 % on large N and 2x on small N (no second launch);
-  // 16-row blocks win for M <= 16 up to N = 16384, 32-row blocks beyond and for M > 16.  With
-  // fewer K blocks a wave's ring never fills and the split-K kernel is faster.
+  if (p.M > 64 || p.K < 512) return false;
+  // Rows of weight per block (16 or 32; 0 = leave the shape to the split-K kernel), from a sweep over
+  // N = 1024 ... 57344, K = 512 ... 28672 and M = 1 ... 64 with the weights rotated through more than the
+  // last-level cache.  Against the split-K kernel this one saves the second launch and the partial sums,
+  // which is worth a factor of up to two on small weights (1 x 3072 x 1536: 7.7 -> 4.3 us) and 5-15 % on
+  // large ones; the split-K kernel is ahead where it needs no split (N >= 16384) and K is short, and for
+  // more than 16 rows on large N, where this kernel's per-wave activation copies weigh more.
   int nib = 0;
   if (t_tile == 16) nib = 1;
-  else if (t_tile == 32) nib = 2;
-  else if (p.K >= 2048) {
-    // (measured: 16-row blocks up to M = 8 whatever N, e.g. 8 x 57344 x 8192 83 against 93 us; at M = 16 up to
-    // N = 16384; for 16 < M <= 32 only on small N, e.g. 32 x 4096 x 7168 8.4 against 9.1 us)
-    nib = (p.M <= 8 || (p.M <= 16 && p.N <= 16384) || p.N <= 4096 || p.M > 32) ? 1 : 2;
-    if (p.N < 64 * 16 * nib) nib = 0;
+  else if (t_tile == 32) nib = p.M <= 32 ? 2 : 0;
+  else if (t_tile == 0) {
+    // 32-row blocks move half the activation bytes per weight byte; they lose where they leave half of the
+    // CUs idle (N <= 4096) or their last round is less than half full (N = 10240: 320 blocks on 256 CUs)
+    const int blocks32 = (p.N + 31) / 32, rounds32 = (blocks32 + num_cus() - 1) / num_cus();
+    const bool wide_ok = p.N > 4096 && (rounds32 * num_cus() - blocks32 < num_cus() / 2 || rounds32 > 3);
+    const bool short_k_no_split = p.K < 2048 && p.N >= 16384;
+    if (p.M <= 16) {
+      if (short_k_no_split) nib = 0;
+      // (long K: 16-row blocks except where they fill between one and one and a half rounds of the CUs;
+      // 8 x 57344 x 8192: 83 against 93 us, 8 x 5120 x 13824: 19.1 against 16.3 us)
+      else if (p.K >= 8192) nib = (p.N > 4096 && p.N <= 6144) ? 2 : 1;
+      else nib = wide_ok ? 2 : 1;
+    } else if (p.M <= 32) {
+      if (short_k_no_split || p.N >= 18432 || (p.N >= 10240 && p.K >= 7168)) nib = 0;
+      else if (p.K >= 8192) nib = p.N <= 4096 ? 1 : 2;
+      else nib = wide_ok ? 2 : 1;
+    } else {
+      // 64 activation rows (8 KiB per K block and wave, one block per CU): on weights of up to 30 MB with few
+      // enough blocks (64 x 4096 x 7168: 14.1 -> 10.3 us, 64 x 4096 x 4096: 14.8 -> 8.3 us; but
+      // 64 x 8192 x 8192: 22 -> 27 us and 64 x 13824 x 2048: 14.4 -> 15.8 us)
+      nib = ((int64_t)p.N * p.K <= (30 << 20) && p.N <= 10240) ? 1 : 0;
+    }
+    if (nib == 2 && p.N < 2048) nib = 1;
+    if (p.N < 1024) nib = 0;
   }
-  if (p.M > 32) nib = nib == 0 ? 0 : 1;  // (64 activation rows are built with 16-row blocks only)
+  if (p.M > 32 && nib == 2) nib = 0;  // (64 activation rows are built with 16-row blocks only)
   if (nib == 0) return false;
   p.splits = 1;
   p.tiles_m = 1;
@@ -2303,7 +2329,9 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const bool plain_scales = !is_block(KIND);
   const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) ||
                            (plain_scales && p.M <= 128 && weight_bytes < (64 << 20)) ||
-                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20)) || (t_tile == 64 && p.M <= 512);
+                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20)) ||
+                           (p.M <= 256 && weight_bytes < (16 << 20)) ||  // (256 x 7168 x 2048 block-FP8: 21.2 -> 15.5 us)
+                           (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
