@@ -115,9 +115,11 @@ int sglq_per_token_quant_int8(const void* input, int in_dtype, void* output_q, f
  *
  * workspace (all four GEMM entry points): optional device scratch of
  * workspace_bytes bytes, 16-byte aligned, owned by the caller and not shared
- * with a call running concurrently on another stream.  For M <= 64 the weight
- * matrix is streamed by several blocks per output tile (split-K) whose fp32 /
- * int32 partial sums pass through it; it plays the part of the per-call
+ * with a call running concurrently on another stream.  Where a shape has too
+ * few output tiles to fill the chip, several blocks share a tile, each with a
+ * part of K (split-K), and their fp32 / int32 partial sums pass through it
+ * (4 * splits * M * N bytes; the split factor is capped by what fits); it plays
+ * the part of the per-call
  * workspace tensor that the reference's launchers allocate
  * (fp8_blockwise_gemm_kernel.cu:153-155).  NULL or too small only costs speed. */
 int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,

@@ -109,10 +109,13 @@ WORKSPACE_BYTES = 64 << 20
 
 
 def workspace(device: torch.device):
-    """Per-device scratch for the split-K partial sums of the M <= 64 GEMM kernels,
+    """Scratch for the split-K partial sums of the GEMM kernels, one buffer per device and
+    stream (two streams may run GEMMs at the same time and must not share partial sums),
     allocated on first use (the reference caches its GEMM workspaces the same way,
-    sgl-kernel/python/sgl_kernel/utils.py `_get_cache_buf`).  Returns (pointer, bytes)."""
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    sgl-kernel/python/sgl_kernel/utils.py `_get_cache_buf`).  Returns (pointer, bytes) for
+    the device's current stream."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (device.type, index, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None:
         buf = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device)

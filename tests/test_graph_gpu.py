@@ -20,7 +20,7 @@ def test_graph_replay_matches_eager(gpu, m):
 
     print("graph replay", m, flush=True)
     n, k = 2112, 4096
-    _lib.workspace(gpu)  # allocated before capture, as a server would at start-up
+    _lib.workspace(gpu)  # the eager calls' workspace; the capture stream gets one of its own from the graph's pool
     wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=1))
     w8, ws8 = O.block_quant_weight_int8(O.gen_weight(n, k, seed=2))
     wq, ws, w8, ws8 = wq.to(gpu), ws.to(gpu), w8.to(gpu), ws8.to(gpu)
@@ -108,3 +108,38 @@ def test_graph_replay_grouped_mm(gpu, rows_per_expert):
             ref = O.fp8_blockwise_scaled_mm(c["a"][first:first + rows], c["b"][2], c["scales_a"][first:first + rows], c["scales_b"][2],
                                             torch.float32, acc_dtype=torch.float64)
             torch.testing.assert_close(got[first:first + rows].cpu().float(), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_two_streams_do_not_share_partial_sums(gpu):
+    """Split-K GEMMs enqueued on two streams at the same time each use a workspace of their own
+    stream, so both give what a call alone gives."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    print("two streams", flush=True)
+    lib = _lib.load()
+    m, n, k = 300, 2112, 7168
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=21))
+    wq, ws = wq.to(gpu), ws.to(gpu)
+    cases = []
+    for seed in (22, 23):
+        xq, xs = sglang_per_token_group_quant_fp8(O.gen_activation(m, k, seed=seed).to(gpu), 128, column_major_scales=True)
+        alone = fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+        assert "splitk_reduce_kernel" in lib.sglq_debug_last_gemm_kernel().decode()
+        cases.append((xq, xs, alone))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)]
+    pointers = set()
+    got = [[], []]
+    for rep in range(20):
+        for i, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                pointers.add(_lib.workspace(gpu)[0])
+                xq, xs, _ = cases[i]
+                got[i].append(fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+    torch.cuda.synchronize()
+    assert len(pointers) == 2
+    for i in range(2):
+        for y in got[i]:
+            assert torch.equal(y, cases[i][2])
