@@ -55,6 +55,7 @@ struct GemmArgs {
   int splits;
   int64_t b_expert_stride, sb_expert_stride;  // grouped GEMM: bytes / floats between experts' weights / weight scales
   int num_experts;
+  int stream_out;  // the output is larger than the last-level cache: store it with the non-temporal hint
 };
 
 // Grouped GEMM tile plan in the workspace (int32): [0] = number of row tiles, then from [4] on
@@ -412,7 +413,9 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
         const int ml = wave * RPW + it * 2 + (lane >> 5);
         const uint32_t m_rel = (uint32_t)((ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1)));
         const uint32_t voff = (c * 8 < BN) ? m_rel * row_bytes + (uint32_t)c * 16u : OOB;
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 0);
+        // (aux bit 1 = nt: a line that will not be read again before it leaves the caches)
+        if (p.stream_out) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 2);
+        else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 0);
       }
     } else {
 #pragma unroll
@@ -2423,6 +2426,10 @@ static void fill_common(GemmArgs& p, const void* a, int64_t lda, const void* b, 
   p.K = (int)K;
   p.a_bytes = (uint32_t)((M - 1) * lda + K);
   p.b_bytes = (uint32_t)((N - 1) * ldb + K);
+  // 256 MB of last-level cache: an output well beyond it is written past the caches (8192 x 32768 x 512,
+  // 537 MB: 236 -> 199 us); one that fits is better left there for the kernel that reads it next
+  // (4096 x 32768 x 512, 268 MB: 97 -> 108 us with the hint)
+  p.stream_out = 2 * M * N > (int64_t)384 << 20;
 }
 
 static int finish(const char* name) {

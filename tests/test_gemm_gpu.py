@@ -339,6 +339,32 @@ def check_every_kind(gpu, m, n, k):
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL)
 
 
+def test_output_beyond_the_last_level_cache(gpu):
+    """An output of more than 384 MiB is stored with the non-temporal hint.  The same rows
+    computed as two launches of half the rows each (plain stores, the same 256-row tiles) must
+    give the same bits, and a row sample matches the oracle."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("fp8_blockwise, output above 384 MiB")
+    m, n, k = 8192, 24832, 512
+    assert 2 * m * n > 384 << 20 >= m * n
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((m, k), generator=g, device=gpu).to(torch.bfloat16)
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=5))
+    wqg, wsg = wq.to(gpu), ws.to(gpu)
+    xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    out = fp8_blockwise_scaled_mm(xq, wqg.t(), xs, wsg.t(), torch.bfloat16)
+    h = m // 2
+    for lo in (0, h):
+        part = fp8_blockwise_scaled_mm(xq[lo:lo + h], wqg.t(), xs[lo:lo + h].t().contiguous().t(), wsg.t(), torch.bfloat16)
+        assert torch.equal(out[lo:lo + h], part)
+        del part
+    rows = sample_rows(m, 12)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows.to(gpu)].cpu(), wq.t(), xs[rows.to(gpu)].cpu(), ws.t(), torch.float32)
+    torch.testing.assert_close(out[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("mnk", [(1, 128, 128), (7, 2112, 7168), (16, 7168, 2048), (17, 264, 1024), (33, 4096, 512),
                                  (64, 1536, 4096), (48, 136, 16384)])
 def test_decode_kernel_split_k(gpu, splits, mnk):
