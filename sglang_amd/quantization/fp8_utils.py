@@ -87,3 +87,127 @@ def apply_fp8_linear(
     assert weight_scale.numel() == weight.shape[1], "cutlass w8a8 fp8 sgl-kernel only supports per-channel scale"
     output = fp8_scaled_mm(qinput, weight, x_scale, weight_scale, out_dtype=input.dtype, bias=bias)
     return output.view(*output_shape)
+
+
+# ---------------------------------------------------------------------------------------------
+# The names the reference's linear methods import for this path (fp8_utils.py:79-147,182-258).
+
+cutlass_w8a8_block_fp8_linear_with_fallback = w8a8_block_fp8_linear
+
+
+def deepgemm_w8a8_block_fp8_linear_with_fallback(
+    input: torch.Tensor,
+    weight: torch.Tensor,
+    block_size: List[int],
+    weight_scale: torch.Tensor,
+    input_scale: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """The call sequence of deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:215-258):
+    the activation scales are column-major with the row count padded to a multiple of four
+    (`scale_tma_aligned=True`), fp32 (the packed UE8M0 form is the reference's Blackwell-only
+    variant); the GEMM is this library's block-scaled kernel, which takes the scales' strides as
+    they are.  Outputs other than bfloat16 and weights whose N is not a multiple of 64 take the
+    row-major path, as in the reference."""
+    assert input_scale is None
+    if not (input.dtype == torch.bfloat16 and weight.shape[0] % 64 == 0 and weight.shape[1] % 128 == 0):
+        return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True, scale_tma_aligned=True)
+    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
+    if bias is not None:
+        output += bias
+    return output.to(dtype=input.dtype).view(*output_shape)
+
+
+def cutlass_fp8_supported() -> bool:
+    """True where fp8_scaled_mm can run (fp8_utils.py:79-88 asks for an SM89+ CUDA build): here,
+    where the HIP library loads and a GPU is present."""
+    from .. import _lib
+
+    try:
+        _lib.load()
+    except Exception:
+        return False
+    return torch.cuda.is_available()
+
+
+def cutlass_block_fp8_supported() -> bool:
+    """True where fp8_blockwise_scaled_mm can run (fp8_utils.py:115-128).  The reference also
+    wants SGLANG_SUPPORT_CUTLASS_BLOCK_FP8 set; this library has no slower path to prefer."""
+    return cutlass_fp8_supported()
+
+
+def dispatch_w8a8_block_fp8_linear():
+    """The block-FP8 linear the layers call (fp8_utils.py:137-147)."""
+    return cutlass_w8a8_block_fp8_linear_with_fallback
+
+
+# ---------------------------------------------------------------------------------------------
+# Weight preparation at load time (plain torch on whatever device the weights are on; not timed).
+
+
+def input_to_float8(x: torch.Tensor, dtype: torch.dtype = torch.float8_e4m3fn):
+    """Per-tensor quantization in torch (fp8_utils.py:339-355): amax clamped at 1e-12,
+    q = clamp(x * (fp_max / amax)) rounded to `dtype`; returns q and 1 / (fp_max / amax)."""
+    fp_max = torch.finfo(dtype).max
+    lo, hi = x.aminmax()
+    amax = torch.maximum(lo.abs(), hi.abs()).float().clamp(min=1e-12)
+    scale = fp_max / amax
+    q = (x.float() * scale).clamp(min=-fp_max, max=fp_max).to(dtype).contiguous()
+    return q, scale.float().reciprocal()
+
+
+def _expand_block_scales(x_s: torch.Tensor, block_size: List[int], n: int, k: int) -> torch.Tensor:
+    return x_s.repeat_interleave(block_size[0], dim=-2).repeat_interleave(block_size[1], dim=-1)[..., :n, :k]
+
+
+def block_quant_dequant(x_q_block: torch.Tensor, x_s: torch.Tensor, block_size: List[int], dtype: torch.dtype) -> torch.Tensor:
+    """Block-quantized weight [..., n, k] with scales [..., ceil(n/bn), ceil(k/bk)] back to `dtype`
+    (fp8_utils.py:401-421)."""
+    *_, n, k = x_q_block.shape
+    return (x_q_block.to(torch.float32) * _expand_block_scales(x_s, block_size, n, k)).to(dtype)
+
+
+def _tensor_quant_fp8(x: torch.Tensor, dtype: torch.dtype):
+    # the reference quantizes with its CUDA operator where it has one and in torch elsewhere
+    # (fp8_utils.py:392-396); the operator here is scaled_fp8_quant on GPU tensors
+    if x.is_cuda:
+        from .fp8_kernel import scaled_fp8_quant
+
+        return scaled_fp8_quant(x)
+    return input_to_float8(x, dtype=dtype)
+
+
+def block_quant_to_tensor_quant(x_q_block: torch.Tensor, x_s: torch.Tensor, block_size: List[int]):
+    """Block-wise FP8 quantization re-quantized with one scale for the tensor (fp8_utils.py:358-398)."""
+    n, k = x_q_block.shape
+    assert x_s.shape[0] == (n + block_size[0] - 1) // block_size[0]
+    assert x_s.shape[1] == (k + block_size[1] - 1) // block_size[1]
+    return _tensor_quant_fp8(block_quant_dequant(x_q_block, x_s, block_size, torch.float32), x_q_block.dtype)
+
+
+def channel_quant_to_tensor_quant(x_q_channel: torch.Tensor, x_s: torch.Tensor):
+    """Per-channel FP8 quantization re-quantized with one scale for the tensor (fp8_utils.py:489-499)."""
+    return _tensor_quant_fp8(x_q_channel.to(torch.float32) * x_s, x_q_channel.dtype)
+
+
+def ceil_to_ue8m0(x: torch.Tensor) -> torch.Tensor:
+    """The next power of two at or above abs(x) (fp8_utils.py:485-486)."""
+    return torch.pow(2.0, torch.ceil(torch.log2(x.abs())))
+
+
+def per_block_cast_to_fp8(x: torch.Tensor):
+    """128 x 128 block quantization of a 2-D weight with power-of-two scales (fp8_utils.py:468-481):
+    block amax clamped at 1e-4, scale = ceil_to_ue8m0(amax / 448), q = x * (1 / scale)."""
+    assert x.dim() == 2
+    m, n = x.shape
+    mp, np_ = (m + 127) // 128 * 128, (n + 127) // 128 * 128
+    padded = torch.zeros((mp, np_), dtype=x.dtype, device=x.device)
+    padded[:m, :n] = x
+    blocks = padded.view(mp // 128, 128, np_ // 128, 128)
+    amax = blocks.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    sf = ceil_to_ue8m0(amax / 448.0)
+    q = (blocks * (1.0 / sf)).to(torch.float8_e4m3fn)
+    return q.view(mp, np_)[:m, :n].contiguous(), sf.view(mp // 128, np_ // 128)

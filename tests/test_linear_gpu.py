@@ -125,3 +125,60 @@ def test_triton_path_block_fp8_linear(gpu):
         assert torch.equal(out.view(torch.int16), other.view(torch.int16))
     with pytest.raises(NotImplementedError):
         triton_w8a8_block_fp8_linear(x.to(gpu), wq.to(gpu), [64, 64], ws.to(gpu))
+
+
+@pytest.mark.parametrize("m", [5, 130])
+def test_deepgemm_path_block_fp8_linear(gpu, m):
+    """deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:215-258): column-major activation
+    scales with the row count padded to a multiple of four.  Same kernels and sums as the plain
+    column-major path, so the results are equal bit for bit; fp16 inputs and an N that is not a
+    multiple of 64 take the row-major path, which gives the same bits as well."""
+    from sglang_amd.quantization import fp8_utils as F
+
+    print("deepgemm-path block fp8 linear", m, flush=True)
+    n, k = 1536, 2048
+    x = O.gen_activation(m, k, seed=6, outliers=True)
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=7))
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(8)) * 0.1).to(torch.bfloat16)
+    xq, xs = O.per_token_group_quant_fp8(x, 128)
+    mm = O.fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.float32)
+    for b in (None, bias.to(gpu)):
+        out = F.deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), wq.to(gpu), [128, 128], ws.to(gpu), bias=b)
+        want = mm + bias.float() if b is not None else mm
+        tol = 1e-2 + 1e-2 * want.abs() + mm.abs() * 2.0**-8
+        err = (out.cpu().float() - want).abs()
+        assert out.dtype == torch.bfloat16 and bool((err <= tol).all()), f"max excess {(err - tol).max().item()}"
+        other = F.cutlass_w8a8_block_fp8_linear_with_fallback(x.to(gpu), wq.to(gpu), [128, 128], ws.to(gpu), bias=b)
+        assert torch.equal(out.view(torch.int16), other.view(torch.int16))
+    # fall-backs: fp16 activations; N = 1504 (a multiple of 4 and of 32, not of 64)
+    half = F.deepgemm_w8a8_block_fp8_linear_with_fallback(x.half().to(gpu), wq.to(gpu), [128, 128], ws.to(gpu))
+    assert half.dtype == torch.float16
+    assert torch.equal(half, F.triton_w8a8_block_fp8_linear(x.half().to(gpu), wq.to(gpu), [128, 128], ws.to(gpu)))
+    narrow = F.deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), wq[:1504].contiguous().to(gpu), [128, 128], ws.to(gpu))
+    assert torch.equal(narrow, out_rows(F, x.to(gpu), wq[:1504].contiguous().to(gpu), ws.to(gpu)))
+    assert F.cutlass_fp8_supported() and F.cutlass_block_fp8_supported()
+    assert F.dispatch_w8a8_block_fp8_linear() is F.cutlass_w8a8_block_fp8_linear_with_fallback
+
+
+def out_rows(F, x, wq, ws):
+    return F.triton_w8a8_block_fp8_linear(x, wq, [128, 128], ws)
+
+
+def test_tensor_requant_of_block_weights_on_the_device(gpu):
+    """block_quant_to_tensor_quant / channel_quant_to_tensor_quant on GPU tensors quantize with
+    scaled_fp8_quant (the reference's CUDA branch, fp8_utils.py:392-396): scale = amax / 448 of
+    the dequantized weight and codes that match the oracle's per-tensor quantization of it."""
+    from sglang_amd.quantization import fp8_utils as F
+
+    print("tensor requant", flush=True)
+    wq, ws = O.block_quant_weight(O.gen_weight(300, 520, seed=9))
+    deq = F.block_quant_dequant(wq, ws, [128, 128], torch.float32)
+    q, s = F.block_quant_to_tensor_quant(wq.to(gpu), ws.to(gpu), [128, 128])
+    ref_q, ref_s = O.per_tensor_quant_fp8(deq)
+    assert torch.equal(s.cpu().view(-1), ref_s.view(-1))
+    assert torch.equal(q.cpu().view(torch.uint8), ref_q.view(torch.uint8))
+    ch = torch.rand(300, 1) * 0.01 + 0.001
+    q2, s2 = F.channel_quant_to_tensor_quant(wq.to(gpu), ch.to(gpu))
+    ref_q2, ref_s2 = O.per_tensor_quant_fp8(wq.float() * ch)
+    assert torch.equal(s2.cpu().view(-1), ref_s2.view(-1))
+    assert torch.equal(q2.cpu().view(torch.uint8), ref_q2.view(torch.uint8))
