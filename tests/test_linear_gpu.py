@@ -182,3 +182,48 @@ def test_tensor_requant_of_block_weights_on_the_device(gpu):
     ref_q2, ref_s2 = O.per_tensor_quant_fp8(wq.float() * ch)
     assert torch.equal(s2.cpu().view(-1), ref_s2.view(-1))
     assert torch.equal(q2.cpu().view(torch.uint8), ref_q2.view(torch.uint8))
+
+
+def test_fp8_linear_from_a_16_bit_checkpoint(gpu):
+    """fp8.py:362-378 then apply_fp8_linear: per-channel weight quantization at load time, the
+    transposed view, dynamic per-token activations.  Against the oracle's sequence on the same
+    codes, and loosely against the unquantized product (FP8 keeps 3 mantissa bits)."""
+    from sglang_amd.quantization.fp8 import process_weights_after_loading
+    from sglang_amd.quantization.fp8_utils import apply_fp8_linear
+
+    print("fp8 linear, 16-bit checkpoint", flush=True)
+    m, n, k = 48, 1024, 2048
+    x = O.gen_activation(m, k, seed=11)
+    w = O.gen_weight(n, k, seed=12).to(torch.bfloat16)
+    wt, ws, in_scale = process_weights_after_loading(w.to(gpu), is_checkpoint_fp8_serialized=False)
+    assert wt.shape == (k, n) and wt.stride(0) == 1 and ws.shape == (n, 1) and in_scale is None
+    out = apply_fp8_linear(x.to(gpu), wt, ws)
+    xq, xs = O.per_token_quant_fp8(x)
+    ref = O.fp8_scaled_mm(xq, wt.cpu(), xs, ws.cpu(), torch.float32, None)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=1e-2, atol=1e-2)
+    exact = x.float() @ w.float().t()
+    assert ((out.cpu().float() - exact).norm() / exact.norm()).item() < 0.06
+
+
+def test_requantize_fused_shards_with_max_scale(gpu):
+    """utils.py:95-121 on the device: every shard ends up on the largest scale; a shard that
+    already has it keeps its codes."""
+    from sglang_amd.quantization.utils import requantize_with_max_scale
+
+    print("requantize fused shards", flush=True)
+    g = torch.Generator().manual_seed(13)
+    codes = (torch.randn((96, 256), generator=g) * 40).clamp(-448, 448).to(torch.float8_e4m3fn)
+    scales = torch.tensor([0.5, 2.0, 1.0])
+    w = codes.clone().to(gpu)
+    max_scale, w2 = requantize_with_max_scale(w, scales.to(gpu), [32, 32, 32])
+    assert max_scale.item() == 2.0 and w2.data_ptr() == w.data_ptr()
+    assert torch.equal(w2[32:64].cpu().view(torch.uint8), codes[32:64].view(torch.uint8))
+    for i, s in ((0, 0.5), (2, 1.0)):
+        want = (codes[32 * i:32 * i + 32].float() * s).half().float()
+        q, _ = O.per_tensor_quant_fp8(want, torch.tensor([2.0]))
+        assert torch.equal(w2[32 * i:32 * i + 32].cpu().view(torch.uint8), q.view(torch.uint8))
+    # a fused checkpoint: the last scale was never loaded, the weight is left alone
+    untouched = codes.clone().to(gpu)
+    init = torch.tensor([1.5, torch.finfo(torch.float8_e4m3fn).min, torch.finfo(torch.float8_e4m3fn).min])
+    m2, w3 = requantize_with_max_scale(untouched, init.to(gpu), [32, 32, 32])
+    assert m2.item() == 1.5 and torch.equal(w3.cpu().view(torch.uint8), codes.view(torch.uint8))

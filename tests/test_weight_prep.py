@@ -102,3 +102,41 @@ def test_dispatch_names():
     # no GPU here (or no library): the predicates say so instead of raising
     assert F.cutlass_fp8_supported() in (True, False)
     assert F.cutlass_block_fp8_supported() == F.cutlass_fp8_supported()
+
+
+def test_convert_to_channelwise_and_dequantize():
+    from sglang_amd.quantization import utils as U
+
+    s = torch.tensor([0.5, 0.25, 2.0])
+    got = U.convert_to_channelwise(s, [2, 1, 3])
+    assert got.shape == (6, 1) and got.dtype == torch.float32
+    assert got.view(-1).tolist() == [0.5, 0.5, 0.25, 2.0, 2.0, 2.0]
+    scalar = U.convert_to_channelwise(torch.tensor(0.125), [2, 2])
+    assert scalar.shape == (4, 1) and scalar.view(-1).tolist() == [0.125] * 4
+    assert U.all_close_1d(torch.tensor([1.0, 1.0, 1.0])) and not U.all_close_1d(torch.tensor([1.0, 1.5]))
+    codes = e4m3_codes((4, 8), seed=7)
+    assert torch.equal(U.per_tensor_dequantize(codes.to(FP8), 0.5), (codes * 0.5).half())
+
+
+def test_fp8_process_weights_after_loading():
+    from sglang_amd.quantization import fp8 as P
+
+    # 16-bit checkpoint: channel c holds codes * 2^-c with a 448 in it: scale 2^-c, the codes back
+    codes = e4m3_codes((3, 64), seed=8)
+    codes[:, 0] = 448.0
+    w = (codes * torch.tensor([[1.0], [0.5], [0.25]])).to(torch.bfloat16)
+    wt, scale, in_scale = P.process_weights_after_loading(w, is_checkpoint_fp8_serialized=False)
+    assert wt.shape == (64, 3) and wt.stride(0) == 1 and in_scale is None
+    assert scale.shape == (3, 1) and scale.view(-1).tolist() == [1.0, 0.5, 0.25]
+    assert torch.equal(wt.t().float(), codes)
+    # an all-zero channel: eps keeps the division defined
+    q0, s0 = P.quantize_weight_per_channel(torch.zeros(1, 16))
+    assert s0.item() == (torch.tensor(1e-10) / 448).item() and torch.equal(q0.float(), torch.zeros(1, 16))
+    # FP8 checkpoint, two fused shards, static activations
+    q = codes.to(FP8)
+    wt2, scale2, in2 = P.process_weights_after_loading(q, torch.tensor([0.5, 2.0]), [1, 2], input_scale=torch.tensor([0.1, 0.3]),
+                                                       static_activations=True)
+    assert wt2.shape == (64, 3) and scale2.view(-1).tolist() == [0.5, 2.0, 2.0] and abs(in2.item() - 0.3) < 1e-7
+    # block quantization: nothing to do
+    ws = torch.ones(1, 1)
+    assert P.process_weights_after_loading(q, ws, block_quant=True) == (q, ws, None)
