@@ -2,7 +2,9 @@
 sizes and writes the table that tuned_configs.load_tuned_configs reads: the counterpart of the
 reference's benchmark/kernels/quantization/tuning_block_wise_kernel.py for its Triton kernel.
 
-    python -m sglang_amd.quantization.tune_block_fp8 --N 4096 --K 7168 [--M 1 8 64 ...] [--out DIR]
+    python -m sglang_amd.quantization.tune_block_fp8 --N 4096 --K 7168 [--M 1 8 64 ...] [--out DIR] [--dtype int8_w8a8]
+
+(--dtype int8_w8a8 tunes the block-scaled INT8 GEMM, w8a8_block_int8_matmul, instead.)
 
 Every candidate (kernel code, split-K factor) is timed from HIP-graph replays with the weights
 rotated through more than the last-level cache; an entry is written only where a candidate beats
@@ -39,9 +41,12 @@ def candidates(m: int, n: int, k: int):
     return out
 
 
-def tune(n: int, k: int, ms, iters: int, margin: float, dev):
+def tune(n: int, k: int, ms, iters: int, margin: float, dev, dtype: str = "fp8_w8a8"):
     from sglang_amd import _lib
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    int8 = dtype == "int8_w8a8"
 
     lib = _lib.load()
     lib.sglq_tuned_clear()
@@ -53,16 +58,25 @@ def tune(n: int, k: int, ms, iters: int, margin: float, dev):
         torch.cuda.synchronize()
     del spin
     g = torch.Generator(device=dev).manual_seed(n + k)
-    w = (torch.randn((n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
+    if int8:
+        w = torch.randint(-127, 128, (n, k), generator=g, device=dev, dtype=torch.int32).to(torch.int8)
+    else:
+        w = (torch.randn((n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
     ws = torch.rand(((n + 127) // 128, (k + 127) // 128), generator=g, device=dev) * 1e-2 + 1e-3
     copies = max(1, min(8, int(600e6 // (n * k))))
     wq = [w] + [w.clone() for _ in range(copies - 1)]
     table = {}
     for m in ms:
-        a = (torch.randn((m, k), generator=g, device=dev) * 2).to(torch.float8_e4m3fn)
-        sa = (torch.rand((k // 128, m), generator=g, device=dev) * 1e-2 + 1e-3).t()  # column-major [m, k / 128]
+        if int8:
+            a = torch.randint(-127, 128, (m, k), generator=g, device=dev, dtype=torch.int32).to(torch.int8)
+            sa = torch.rand((m, k // 128), generator=g, device=dev) * 1e-2 + 1e-3  # row-major, as the INT8 quantizer writes it
+        else:
+            a = (torch.randn((m, k), generator=g, device=dev) * 2).to(torch.float8_e4m3fn)
+            sa = (torch.rand((k // 128, m), generator=g, device=dev) * 1e-2 + 1e-3).t()  # column-major [m, k / 128]
 
         def run(j):
+            if int8:
+                return w8a8_block_int8_matmul(a, wq[j], sa, ws, [128, 128], torch.bfloat16)
             return fp8_blockwise_scaled_mm(a, wq[j].t(), sa, ws.t(), torch.bfloat16)
 
         def time_it():
@@ -129,10 +143,11 @@ def main():
     ap.add_argument("--iters", type=int, default=8)
     ap.add_argument("--margin", type=float, default=0.04)
     ap.add_argument("--out", type=str, default=None, help="directory for the table (default: the package's configs/)")
+    ap.add_argument("--dtype", choices=["fp8_w8a8", "int8_w8a8"], default="fp8_w8a8", help="block-scaled FP8 or block-scaled INT8 GEMM")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
-    table = tune(args.N, args.K, args.M, args.iters, args.margin, dev)
-    path = save_config(args.N, args.K, table, args.out)
+    table = tune(args.N, args.K, args.M, args.iters, args.margin, dev, args.dtype)
+    path = save_config(args.N, args.K, table, args.out, dtype=args.dtype)
     print("wrote", path)
 
 

@@ -552,43 +552,59 @@ def test_tuned_table_selects_the_kernel(gpu):
 
 
 def test_shipped_tuned_tables_give_oracle_results(gpu):
-    """Every selection in the tables shipped under sglang_amd/quantization/configs/ is run once at its
-    own (M, N, K) with the tables loaded as a user has them, and checked against the oracle on the
-    first and last 256 output columns."""
+    """Every selection in the tables shipped under sglang_amd/quantization/configs/ (block FP8 and
+    block INT8) is run once at its own (M, N, K) with the tables loaded as a user has them, and
+    checked against the oracle on the first and last 256 output columns."""
     import json
 
     from sglang_amd import _lib
     from sglang_amd.quantization import tuned_configs as T
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
-    lib = _lib.load()
+    _lib.load()
     assert T.load_tuned_configs() >= 0
     cases = []
     for path in sorted(T.CONFIG_DIR.iterdir()):
         parsed = T.parse_file_name(path.name)
-        if parsed is None or parsed[3] != "fp8_w8a8":
+        if parsed is None or parsed[3] not in T.KIND_OF_DTYPE:
             continue
         table = {int(key): val for key, val in json.loads(path.read_text()).items()}
-        cases += [(m, parsed[0], parsed[1], v["tile"], v["splits"]) for m, v in table.items() if v["tile"] or v["splits"]]
+        cases += [(parsed[3], m, parsed[0], parsed[1], v["tile"], v["splits"]) for m, v in table.items() if v["tile"] or v["splits"]]
     say("tuned selections shipped:", len(cases))
+    assert {c[0] for c in cases} == {"fp8_w8a8", "int8_w8a8"}
     gg = torch.Generator(device=gpu).manual_seed(3)
+
+    def codes(shape, int8):
+        if int8:
+            return torch.randint(-127, 128, shape, generator=gg, device=gpu, dtype=torch.int32).to(torch.int8)
+        return (torch.randn(shape, generator=gg, device=gpu) * 2).to(FP8)
+
     weights = {}
-    for m, n, k, tile, splits in cases:
-        say("tuned entry", m, n, k, tile, splits)
-        if (n, k) not in weights:
+    for dtype, m, n, k, tile, splits in cases:
+        say("tuned entry", dtype, m, n, k, tile, splits)
+        int8 = dtype == "int8_w8a8"
+        if (dtype, n, k) not in weights:
             weights.clear()  # one weight at a time on the device
-            w = (torch.randn((n, k), generator=gg, device=gpu) * 0.5).to(FP8)
             ws = torch.rand(((n + 127) // 128, k // 128), generator=gg, device=gpu) * 1e-2 + 1e-3
-            weights[(n, k)] = (w, ws)
-        w, ws = weights[(n, k)]
+            weights[(dtype, n, k)] = (codes((n, k), int8), ws)
+        w, ws = weights[(dtype, n, k)]
         rows = min(m, 48)
-        a = (torch.randn((m, k), generator=gg, device=gpu) * 2).to(FP8)
+        a = codes((m, k), int8)
         sa = (torch.rand((k // 128, m), generator=gg, device=gpu) * 1e-2 + 1e-3).t()
-        out = fp8_blockwise_scaled_mm(a, w.t(), sa, ws.t(), torch.bfloat16)
+        if int8:
+            sa = sa.contiguous()
+            out = w8a8_block_int8_matmul(a, w, sa, ws, [128, 128], torch.bfloat16)
+        else:
+            out = fp8_blockwise_scaled_mm(a, w.t(), sa, ws.t(), torch.bfloat16)
         for cols in (slice(0, 256), slice(n - 256, n)):
+            if cols.start % 128:
+                continue
             nb = slice(cols.start // 128, (cols.stop + 127) // 128)
-            ref = O.fp8_blockwise_scaled_mm(a[:rows].cpu(), w[cols].cpu().t(), sa[:rows].cpu().contiguous(),
-                                            ws[nb].cpu().t()[:, : 2], torch.float32, acc_dtype=torch.float64) \
-                if cols.start % 128 == 0 else None
-            if ref is not None:
-                torch.testing.assert_close(out[:rows, cols].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+            if int8:
+                ref = O.w8a8_block_int8_matmul(a[:rows].cpu(), w[cols].cpu(), sa[:rows].cpu(), ws[nb].cpu(), torch.float32,
+                                               acc_dtype=torch.float64)
+            else:
+                ref = O.fp8_blockwise_scaled_mm(a[:rows].cpu(), w[cols].cpu().t(), sa[:rows].cpu().contiguous(),
+                                                ws[nb].cpu().t()[:, : 2], torch.float32, acc_dtype=torch.float64)
+            torch.testing.assert_close(out[:rows, cols].cpu().float(), ref, rtol=RTOL, atol=ATOL)
