@@ -42,7 +42,7 @@ int sglq_abi_version(void);
  * output_s  fp32; element (row, g) lives at output_s[row*s_stride_row + g*s_stride_col],
  *           which covers the reference's row-major, column-major and padded
  *           column-major scale buffers (per_token_group_quant_8bit.cu:54-64,153-156)
- * group_size in {16, 32, 64, 128}; hidden % group_size == 0. */
+ * group_size in {8, 16, 32, 64, 128}; hidden % group_size == 0. */
 int sglq_per_token_group_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,
                                    int64_t num_tokens, int64_t hidden, int group_size,
                                    int64_t s_stride_row, int64_t s_stride_col, float eps, float fp8_min,

@@ -670,13 +670,13 @@ static int group_quant_entry(const char* name, const void* input, int in_dtype, 
                                                sc, eps, qmin, qmax, st);                                      \
     return check_launch(name);                                                                                \
   }
-#define SGLQ_GQ_DT(DT) SGLQ_GQ_CASE(DT, 128) SGLQ_GQ_CASE(DT, 64) SGLQ_GQ_CASE(DT, 32) SGLQ_GQ_CASE(DT, 16)
+#define SGLQ_GQ_DT(DT) SGLQ_GQ_CASE(DT, 128) SGLQ_GQ_CASE(DT, 64) SGLQ_GQ_CASE(DT, 32) SGLQ_GQ_CASE(DT, 16) SGLQ_GQ_CASE(DT, 8)
   SGLQ_GQ_DT(SGLQ_BF16)
   SGLQ_GQ_DT(SGLQ_FP16)
   SGLQ_GQ_DT(SGLQ_FP32)
 #undef SGLQ_GQ_DT
 #undef SGLQ_GQ_CASE
-  set_error("%s: unsupported in_dtype %d / group_size %d (group sizes built: 16, 32, 64, 128)", name, in_dtype,
+  set_error("%s: unsupported in_dtype %d / group_size %d (group sizes built: 8, 16, 32, 64, 128)", name, in_dtype,
             group_size);
   return SGLQ_EUNSUPPORTED;
 }

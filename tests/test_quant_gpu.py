@@ -42,7 +42,7 @@ def test_group_quant_fp8_bit_exact(gpu, dtype, shape):
         assert_bits_equal(q, q_ref, f"codes cm={cm} tma={tma}")
 
 
-@pytest.mark.parametrize("group", [16, 32, 64, 128])
+@pytest.mark.parametrize("group", [8, 16, 32, 64, 128])
 def test_group_quant_fp8_group_sizes(gpu, group):
     say("group_quant group", group)
     x = O.gen_activation(129, 1024, seed=group, outliers=True)
@@ -106,6 +106,35 @@ def test_group_quant_int8_bit_exact(gpu):
     sgl_per_token_group_quant_int8(xg, q, s, 128, 1e-10, -128.0, 127.0)
     assert_bits_equal(s, s_ref, "scales")
     assert_bits_equal(q, q_ref, "codes")
+
+
+@pytest.mark.parametrize("to_int8", [False, True], ids=["fp8", "int8"])
+@pytest.mark.parametrize("group", [8, 16, 32, 64, 128])
+@pytest.mark.parametrize("shape", [(127, 256), (512, 1024), (128, 4096)])
+def test_group_quant_grid_of_the_reference_test(gpu, shape, group, to_int8):
+    """The grid of sgl-kernel/tests/test_per_token_group_quant_8bit.py:266-279 (token counts and
+    hidden sizes thinned): every group size, both code types, row-major scales and the two
+    column-major buffers of create_per_token_group_quant_fp8_output_scale written by the op itself."""
+    from sglang_amd.quantization.fp8_kernel import create_per_token_group_quant_fp8_output_scale
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8, sgl_per_token_group_quant_int8
+
+    say("group_quant grid", shape, group, to_int8)
+    m, k = shape
+    x = O.gen_activation(m, k, seed=m + k + group, outliers=True)
+    lo, hi = (-128.0, 127.0) if to_int8 else (-448.0, 448.0)
+    q_dtype = torch.int8 if to_int8 else torch.float8_e4m3fn
+    q_ref, s_ref = O.per_token_group_quant_8bit(x, group, 1e-10, lo, hi, q_dtype)
+    xg = x.to(gpu)
+    for cm, tma in ((False, False), (True, False), (True, True)):
+        q = torch.empty_like(xg, dtype=q_dtype)
+        s = create_per_token_group_quant_fp8_output_scale(xg.shape, gpu, group, column_major_scales=cm, scale_tma_aligned=tma,
+                                                          scale_ue8m0=False)
+        if to_int8:
+            sgl_per_token_group_quant_int8(xg, q, s, group, 1e-10, lo, hi)
+        else:
+            sgl_per_token_group_quant_fp8(xg, q, s, group, 1e-10, lo, hi, False)
+        assert_bits_equal(s, s_ref, f"scales cm={cm} tma={tma}")
+        assert_bits_equal(q, q_ref, f"codes cm={cm} tma={tma}")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
