@@ -120,6 +120,24 @@ def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(3, 14080, 512), (127, 512, 14080), (5, 8192, 16384), (1024, 14080, 4096), (4096, 14080, 14080)])
+def test_fp8_blockwise_scaled_mm_sizes_of_the_reference_test(gpu, mnk, out_dtype):
+    """Corner points of the grid of sgl-kernel/tests/test_fp8_blockwise_gemm.py:84-87 (M from 1 to 4096,
+    N and K up to 14080 = 110 x 128 and 16384), against the oracle on a sample of rows."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("fp8_blockwise, reference grid", mnk, out_dtype)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = sample_rows(m, 24)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), out_dtype)
+    assert out.dtype == out_dtype and tuple(out.shape) == (m, n)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(1, 128, 128), (5, 2112, 1536), (17, 7168, 2048), (127, 512, 7168), (128, 4096, 256),
                                  (300, 2048, 1024), (512, 1544, 1024), (1024, 640, 2048)])
 def test_fp8_blockwise_scaled_mm_fused_bias(gpu, tile, mnk, out_dtype):
@@ -272,6 +290,40 @@ def test_fp8_scaled_mm(gpu, tile, mnk, with_bias):
     ref = O.fp8_scaled_mm(xq[rows], wq.t(), xs[rows], ws, torch.float32, bias, acc_dtype=torch.float64)
     out = fp8_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs.to(gpu), ws.to(gpu), torch.bfloat16,
                         None if bias is None else bias.to(gpu))
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("mnk", [(1, 16, 512), (8192, 16, 16384), (64, 16384, 512), (4096, 128, 8192), (32, 8192, 16384), (512, 1024, 1024)])
+def test_scaled_mm_sizes_of_the_reference_tests(gpu, mnk, with_bias, out_dtype):
+    """Corner points of the grids of sgl-kernel/tests/test_int8_gemm.py:33-37 and test_fp8_gemm.py:39-43
+    (M 1 ... 8192, N 16 ... 16384, K 512 ... 16384, bias or not, both output types): INT32
+    accumulators exactly, both epilogues against the oracle on a sample of rows."""
+    from sglang_amd.sgl_kernel import fp8_scaled_mm, int8_mm_i32, int8_scaled_mm
+
+    say("scaled_mm, reference grids", mnk, with_bias, out_dtype)
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(m + n + k)
+    bias = (torch.randn(n, generator=g) * 0.1).to(out_dtype) if with_bias else None
+    bias_g = None if bias is None else bias.to(gpu)
+    rows = sample_rows(m, 24)
+    x = O.gen_activation(m, k, seed=m + k)
+    # INT8
+    wt, s_b, _ = O.gen_int8_weight(k, n, seed=n + k)
+    xq, xs = O.per_token_quant_int8(x)
+    wg = wt.t().contiguous().to(gpu).t()
+    assert torch.equal(int8_mm_i32(xq.to(gpu), wg).cpu()[rows], O.int8_mm_i32(xq[rows], wt))
+    out = int8_scaled_mm(xq.to(gpu), wg, xs.to(gpu), s_b.to(gpu), out_dtype, bias_g)
+    ref = O.int8_scaled_mm(xq[rows], wt, xs[rows], s_b, torch.float32, bias)
+    assert out.dtype == out_dtype
+    torch.testing.assert_close(out.cpu()[rows].float(), ref.float(), rtol=RTOL, atol=ATOL)
+    # FP8 per token / per channel
+    fq, fs = O.per_token_quant_fp8(x)
+    wq, ws = O.per_tensor_quant_weight(O.gen_weight(n, k, seed=n))
+    out = fp8_scaled_mm(fq.to(gpu), wq.to(gpu).t(), fs.to(gpu), ws.to(gpu), out_dtype, bias_g)
+    ref = O.fp8_scaled_mm(fq[rows], wq.t(), fs[rows], ws, torch.float32, bias, acc_dtype=torch.float64)
+    assert out.dtype == out_dtype
     torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
 
 
