@@ -2334,6 +2334,8 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
                            (plain_scales && p.M <= 128 && weight_bytes < (64 << 20)) ||
                            (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20)) ||
                            (p.M <= 256 && weight_bytes < (16 << 20)) ||  // (256 x 7168 x 2048 block-FP8: 21.2 -> 15.5 us)
+                           // (160 x 8192 x 2048: 17.9 -> 14.6 us; on N = 32768 the row tiles' second reads of the weights miss the L2)
+                           (p.M <= 256 && weight_bytes <= (16 << 20) && p.K <= 2048 && p.N <= 16384) ||
                            (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
@@ -2367,7 +2369,9 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // Measured against the 128 x 128 kernel: 256 x 7168 x 16384 64 -> 44 us, 1024 x 7168 x 2048
   // 26 -> 20 us, 2048 x 4096 x 7168 74 -> 58 us, 2048 x 2112 x 7168 64 -> 48 us; below 256 rows
   // it only wins on large weights (256 x 24576 x 1536 22 -> 17 us, but 256 x 2112 x 7168 19 -> 21 us).
-  const bool mid = p.M > 256 || (p.M > 128 && weight_bytes >= (24 << 20)) || (p.M > 64 && weight_bytes >= (48 << 20));
+  // ... and on wide ones (160 x 12288 x 1536: 22.3 -> 13.7 us, 256 x 32768 x 512: 13.3 -> 11.2 us)
+  const bool mid = p.M > 256 || (p.M > 128 && weight_bytes >= (24 << 20)) || (p.M > 64 && weight_bytes >= (48 << 20)) ||
+                   (p.M > 128 && weight_bytes >= (16 << 20) && p.N >= 12288);
   if ((p.K & 127) == 0 && p.K >= 384 && (t_tile == 130 || (t_tile == 0 && g_use_dma && mid))) {
     launch_pipe128<KIND, OUT_DT>(p, ws_bytes, st);
     return;
