@@ -2336,6 +2336,10 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
                            (p.M <= 256 && weight_bytes < (16 << 20)) ||  // (256 x 7168 x 2048 block-FP8: 21.2 -> 15.5 us)
                            // (160 x 8192 x 2048: 17.9 -> 14.6 us; on N = 32768 the row tiles' second reads of the weights miss the L2)
                            (p.M <= 256 && weight_bytes <= (16 << 20) && p.K <= 2048 && p.N <= 16384) ||
+                           // narrow and deep (160 x 1024 x 16384: 25.0 -> 19.2 us, 160 x 2048 x 8192: 20.8 -> 18.0 us)
+                           (weight_bytes <= (16 << 20) && (p.N <= 1024 ? p.M <= 256 : p.N <= 2048 && p.M <= 192)) ||
+                           // small weights, deep K (512 x 1024 x 4096: 22.4 -> 16.9 us, 512 x 512 x 7168: 19.4 -> 15.6 us)
+                           (p.M <= 512 && weight_bytes <= (6 << 20) && p.K >= 4096) ||
                            (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
