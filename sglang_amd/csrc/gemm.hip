@@ -2332,7 +2332,9 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const bool plain_scales = !is_block(KIND);
   const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) ||
                            (plain_scales && p.M <= 128 && weight_bytes < (64 << 20)) ||
-                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20)) ||
+                           // (not on wide weights, whose many row tiles re-read them past the L2: 512 x 32768 x 512
+                           // 25.4 us here, 16.9 us on the 256-row kernel; 512 x 16384 x 1024 19.2 against 14.3 us)
+                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20) && (p.N <= 8192 || (p.M <= 256 && p.N <= 16384))) ||
                            (p.M <= 256 && weight_bytes < (16 << 20)) ||  // (256 x 7168 x 2048 block-FP8: 21.2 -> 15.5 us)
                            // (160 x 8192 x 2048: 17.9 -> 14.6 us; on N = 32768 the row tiles' second reads of the weights miss the L2)
                            (p.M <= 256 && weight_bytes <= (16 << 20) && p.K <= 2048 && p.N <= 16384) ||
