@@ -111,7 +111,11 @@ int sglq_per_token_quant_int8(const void* input, int in_dtype, void* output_q, f
  *   sfa fp32 [M, ceil(K/128)]  at sfa[m*sfa_stride_m + kb*sfa_stride_k]
  *   sfb fp32 [ceil(K/128), ceil(N/128)] at sfb[kb*sfb_stride_k + nb*sfb_stride_n]
  *   out [M, N] row stride ldo, out_dtype in {BF16, FP16}
- * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, a and b 16-byte aligned.
+ * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, a and b 16-byte aligned; N % 8 == 0,
+ * ldo % 8 == 0 and out 16-byte aligned (output rows are written in 16-byte pieces; the
+ * reference's own checks, fp8_blockwise_gemm_kernel.cu:383, int8_gemm_kernel.cu:679,
+ * fp8_gemm_kernel.cu:1108).  The same holds for every GEMM entry point below
+ * (sglq_int8_mm_i32: N % 4 == 0, ldo % 4 == 0).
  *
  * workspace (all four GEMM entry points): optional device scratch of
  * workspace_bytes bytes, 16-byte aligned, owned by the caller and not shared
@@ -270,7 +274,8 @@ int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, c
  * split-K factor `splits` (0 = by shape) instead of the built-in heuristics.  The first matching
  * entry wins; a kernel that does not apply to a shape falls through to the next one that does, so
  * no entry can make a call fail.  Results do not depend on the table beyond the summation order
- * that each kernel has anyway.  Fill the table before GEMMs are launched from other threads. */
+ * that each kernel has anyway.  The table is guarded by a reader/writer lock: entries may be
+ * added or cleared while other threads launch GEMMs. */
 #define SGLQ_KIND_FP8_BLOCK 0  /* sglq_fp8_blockwise_scaled_mm(_bias) */
 #define SGLQ_KIND_FP8_ROWCOL 1 /* sglq_fp8_scaled_mm */
 #define SGLQ_KIND_I8_ROWCOL 2  /* sglq_int8_scaled_mm */
@@ -279,7 +284,11 @@ int sglq_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, c
 int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits);
 int sglq_tuned_clear(void);
 
-/* Test hook without a reference counterpart: non-zero (default) makes the GEMMs
+/* The sglq_debug_* hooks below are for tests and measurements, are not part of the operator
+ * ABI, and act on the calling thread only (thread-local state): a thread that forces a kernel
+ * cannot change what GEMM calls on other threads launch.
+ *
+ * Test hook without a reference counterpart: non-zero (default) makes the GEMMs
  * copy global memory straight into LDS with buffer loads, zero stages the same
  * bytes through registers.  Both must give identical results. */
 void sglq_debug_set_direct_lds(int on);

@@ -19,6 +19,9 @@
 // Global -> LDS copies use buffer loads that write LDS directly (each wavefront
 // instruction fills 1 KiB = 8 rows); rows past M/N and chunks past K read as zero
 // through the buffer range check.
+#include <atomic>
+#include <mutex>
+#include <shared_mutex>
 #include <type_traits>
 
 #include "sglq_common.h"
@@ -254,7 +257,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + j * 16 + g * 4;
-      if (n >= p.N) continue;  // N % 4 == 0 is checked on the host: a run of 4 is in or out as a whole
+      if (n >= p.N) continue;  // N % 8 == 0 (% 4 for 32-bit outputs) is checked on the host: a run of 4 is in or out as a whole
       finish4<KIND, OUT_DT, BLOCK_BIAS>(p, m, n, acc[i][j], sam);
     }
   }
@@ -424,11 +427,7 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
         const int m = m0 + (ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1));
         if (m < p.M && c * 8 < BN) {
           char* row = out + ((int64_t)m * p.ldo + n) * 2;
-          if (n + 8 <= p.N) {
-            *reinterpret_cast<v4i*>(row) = v[it];
-          } else if (n + 4 <= p.N) {  // N is a multiple of 4: a half chunk is the only possible remainder
-            *reinterpret_cast<v2u*>(row) = v2u{(uint32_t)v[it][0], (uint32_t)v[it][1]};
-          }
+          if (n + 8 <= p.N) *reinterpret_cast<v4i*>(row) = v[it];  // (N is a multiple of 8: a chunk is in or out as a whole)
         }
       }
     }
@@ -810,7 +809,6 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 
   // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
   const int total = p.tiles_m * p.tiles_n;
-  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   int tile = blockIdx.x;
   int tm, tn;
   tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
@@ -851,12 +849,8 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
     if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
     } else {
-      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
-      if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, cm0, cn0, wm, wn, r16, g, lane,
-                                               wave);
-      else
-        epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, cm0 + wm * TM, cn0 + wn * TN, r16, g);
+      // (rows of 16-bit outputs are 16-byte aligned: checked on the host)
+      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, cm0, cn0, wm, wn, r16, g, lane, wave);
     }
     if (!has_next) break;
     tile = next_tile;
@@ -1131,7 +1125,6 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   const int tiles_m = MODE == PIPE_GROUPED ? plan[0] : p.tiles_m;
   const int tiles = tiles_m * p.tiles_n;
   const int total = tiles * splits;
-  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   auto unit_origin = [&](int u, int& um0, int& un0, int& ukb0, int& uexpert, int& um_end) {
     const int split = MODE == PIPE_SPLITK ? u / tiles : 0;
     int tm, tn;
@@ -1218,18 +1211,11 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     } else if constexpr (MODE == PIPE_GROUPED) {
       GemmArgs q = p;
       q.M = m_end;  // rows past the expert's last one belong to other experts
-      if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, false, BM / 2>(q, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
-                                                          wave);
-      else
-        epilogue<KIND, OUT_DT, MI, NI, 0>(q, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, false, BM / 2>(q, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane, wave);
     } else {
-      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
-      if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS, BM / 2>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn,
-                                                                     r16, g, lane, wave);
-      else
-        epilogue<KIND, OUT_DT, MI, NI, (MODE == PIPE_BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+      // (rows of 16-bit outputs are 16-byte aligned: checked on the host)
+      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, MODE == PIPE_BIAS, BM / 2>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16,
+                                                                             g, lane, wave);
     }
     if (!has_next) break;
     unit = next_unit;
@@ -1484,7 +1470,6 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 
   // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
   const int total = p.tiles_m * p.tiles_n;
-  const bool aligned_out = ((p.ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   int tile = blockIdx.x;
   int tm, tn;
   tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
@@ -1555,12 +1540,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
-      // 16-byte stores need 16-byte aligned rows; otherwise fall back to the 8-byte runs
-      if (aligned_out)
-        epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane,
-                                                   wave);
-      else
-        epilogue<KIND, OUT_DT, MI, NI, (BIAS) ? 1 : 0>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
+      // (rows of 16-bit outputs are 16-byte aligned: checked on the host)
+      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane, wave);
     }
     if (!has_next) break;
     tile = next_tile;
@@ -1916,25 +1897,32 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
-static bool g_use_dma = true;
+// The test hooks (sglq_debug_*) are per calling thread: a test that forces a kernel cannot
+// change what another thread's GEMM calls launch.
+static thread_local bool g_use_dma = true;
 
-// Compute units of the current device (cached; a multiple of 8 keeps the persistent
-// kernel's tile walk on one XCD per block).
+// Compute units of the current device, rounded down to a multiple of 8 (keeps the persistent
+// kernels' tile walk on one XCD per block).  The only process-wide state besides the tuned
+// table: an immutable property, cached per device ordinal (a racing first call stores the same value).
+constexpr int MAX_DEVICES = 64;
 static int num_cus() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached = n >= 8 ? (n / 8) * 8 : n;
+  static std::atomic<int> cached[MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) dev = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    n = n >= 8 ? (n / 8) * 8 : n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached;
+  return n;
 }
 
-static int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
+static thread_local int g_force_splits = 0;  // test hook: > 0 fixes the split-K factor where split-K applies
 // The selection in force for the call being launched on this thread: the test hooks, else a
 // matching entry of the tuned table, else 0 = the built-in heuristics.
 static thread_local int t_tile = 0, t_splits = 0;
-static int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile, 130 = 128 rows pipelined (0 = from the average group)
+static thread_local int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile, 130 = 128 rows pipelined (0 = from the average group)
 static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
 
 template <int KIND, int OUT_DT>
@@ -2032,7 +2020,7 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 // 256 = the plain 256 x 256 kernel, 258 = the pipelined one (K >= 384, else the plain one),
 // 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258),
 // 130 = the pipelined kernel with 128-row tiles (K >= 384, else the 128 x 128 kernel)
-static int g_force_tile = 0;
+static thread_local int g_force_tile = 0;
 
 static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws_bytes, int& splits);
 
@@ -2291,8 +2279,9 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
 // Tuned kernel selections per problem, the counterpart of the reference's per-(N, K) JSON
 // tables for its Triton kernels (python/sglang/srt/layers/quantization/fp8_kernel.py:738-776,
 // layers/quantization/configs/): an entry names the kernel (a code of sglq_debug_force_tile)
-// and the split-K factor for kind, N, K and a range of M.  Filled once at start-up through
-// sglq_tuned_add (not while GEMMs are being launched from other threads); read-only afterwards.
+// and the split-K factor for kind, N, K and a range of M.  Normally filled once at start-up through
+// sglq_tuned_add; a reader/writer lock makes later additions safe against GEMM calls on other
+// threads (an uncontended shared lock costs tens of nanoseconds per GEMM call).
 struct TunedEntry {
   int kind;
   int64_t n, k, m_lo, m_hi;
@@ -2301,23 +2290,30 @@ struct TunedEntry {
 constexpr int MAX_TUNED = 1024;
 static TunedEntry g_tuned[MAX_TUNED];
 static int g_num_tuned = 0;
+static std::shared_mutex g_tuned_lock;
 
-static const TunedEntry* tuned_lookup(int kind, int64_t m, int64_t n, int64_t k) {
+static bool tuned_lookup(int kind, int64_t m, int64_t n, int64_t k, int& tile, int& splits) {
+  std::shared_lock<std::shared_mutex> guard(g_tuned_lock);
   for (int i = 0; i < g_num_tuned; ++i) {
     const TunedEntry& e = g_tuned[i];
-    if (e.kind == kind && e.n == n && e.k == k && m >= e.m_lo && m <= e.m_hi) return &e;
+    if (e.kind == kind && e.n == n && e.k == k && m >= e.m_lo && m <= e.m_hi) {
+      tile = e.tile;
+      splits = e.splits;
+      return true;
+    }
   }
-  return nullptr;
+  return false;
 }
 
 template <int KIND, int OUT_DT>
 static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   t_tile = g_force_tile;
   t_splits = g_force_splits;
-  if (t_tile == 0 && t_splits == 0 && g_num_tuned > 0) {
-    if (const TunedEntry* e = tuned_lookup(KIND, p.M, p.N, p.K)) {
-      t_tile = e->tile;
-      t_splits = e->splits;
+  if (t_tile == 0 && t_splits == 0) {
+    int tile = 0, splits = 0;
+    if (tuned_lookup(KIND, p.M, p.N, p.K, tile, splits)) {
+      t_tile = tile;
+      t_splits = splits;
     }
   }
   if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (t_tile == 0 || t_tile == 16 || t_tile == 32) &&
@@ -2412,8 +2408,13 @@ static int gemm_common_checks(const char* name, const void* a, int64_t lda, cons
     set_error("%s: mat_a and mat_b must be 16-byte aligned", name);
     return SGLQ_EINVAL;
   }
-  if (N % 4 != 0 || ldo % 4 != 0 || ldo < N || (reinterpret_cast<uintptr_t>(out) & (4 * out_elem_bytes - 1))) {
-    set_error("%s: N and ldo must be multiples of 4 and out aligned to 4 elements", name);
+  // Output rows are written in 16-byte pieces: N and ldo multiples of 16 bytes' worth of elements,
+  // the base 16-byte aligned (the reference asks the same of its outputs: int8_gemm_kernel.cu:679,
+  // fp8_gemm_kernel.cu:1108, fp8_blockwise_gemm_kernel.cu:383).
+  const int64_t per16 = 16 / out_elem_bytes;
+  if (N % per16 != 0 || ldo % per16 != 0 || ldo < N || (reinterpret_cast<uintptr_t>(out) & 15)) {
+    set_error("%s: N (%lld) and ldo (%lld) must be multiples of %lld and out 16-byte aligned", name, (long long)N,
+              (long long)ldo, (long long)per16);
     return SGLQ_EINVAL;
   }
   const int64_t a_bytes = (M - 1) * lda + K, b_bytes = (N - 1) * ldb + K;
@@ -2463,6 +2464,7 @@ extern "C" void sglq_debug_set_direct_lds(int on) { g_use_dma = on != 0; }
 extern "C" void sglq_debug_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void sglq_debug_force_splits(int splits) { g_force_splits = splits; }
 extern "C" int sglq_tuned_clear(void) {
+  std::unique_lock<std::shared_mutex> guard(g_tuned_lock);
   g_num_tuned = 0;
   return SGLQ_OK;
 }
@@ -2474,6 +2476,7 @@ extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int6
     set_error("tuned_add: kind 0..4, positive N and K, 0 <= m_lo <= m_hi, a known kernel code and 0 <= splits <= 64 expected");
     return SGLQ_EINVAL;
   }
+  std::unique_lock<std::shared_mutex> guard(g_tuned_lock);
   if (g_num_tuned >= MAX_TUNED) {
     set_error("tuned_add: the table holds %d entries", MAX_TUNED);
     return SGLQ_EUNSUPPORTED;

@@ -48,3 +48,83 @@ def process_weights_after_loading(
     scale = convert_to_channelwise(weight_scale, logical_widths)
     in_scale = input_scale.max() if (static_activations and input_scale is not None) else None
     return weight.t(), scale, in_scale
+
+
+class Fp8Config:
+    """The fields of Fp8Config (fp8.py:96-190) that the linear method reads."""
+
+    def __init__(
+        self,
+        is_checkpoint_fp8_serialized: bool = False,
+        activation_scheme: str = "dynamic",
+        weight_block_size: Optional[List[int]] = None,
+    ):
+        if activation_scheme not in ("static", "dynamic"):
+            raise ValueError(f"Unsupported activation scheme {activation_scheme}")
+        if weight_block_size is not None:
+            if not is_checkpoint_fp8_serialized:
+                raise ValueError("block-wise quantization needs an FP8 checkpoint")
+            if len(weight_block_size) != 2:
+                raise ValueError(f"weight_block_size must have two entries, got {len(weight_block_size)}")
+            if activation_scheme != "dynamic":
+                raise ValueError("block-wise quantization takes dynamic activation scales only")
+        self.is_checkpoint_fp8_serialized = is_checkpoint_fp8_serialized
+        self.activation_scheme = activation_scheme
+        self.weight_block_size = weight_block_size
+
+
+class Fp8LinearMethod:
+    """process_weights_after_loading and apply of Fp8LinearMethod (fp8.py:204-223,333-488) for
+    the branches that end in this library's GEMMs, on any object with `weight` and, per branch,
+    `weight_scale_inv` (block quantization), `weight_scale` + `logical_widths` (FP8 checkpoint)
+    and `input_scale` (static activations)."""
+
+    def __init__(self, quant_config: Fp8Config):
+        from .fp8_utils import cutlass_fp8_supported, dispatch_w8a8_block_fp8_linear
+
+        self.quant_config = quant_config
+        self.cutlass_fp8_supported = cutlass_fp8_supported()
+        self.block_quant = quant_config.weight_block_size is not None
+        self.w8a8_block_fp8_linear = dispatch_w8a8_block_fp8_linear()
+
+    def process_weights_after_loading(self, layer) -> None:
+        cfg = self.quant_config
+        static = cfg.activation_scheme == "static"
+        if self.block_quant:
+            layer.weight = torch.nn.Parameter(layer.weight.data, requires_grad=False)
+            layer.weight_scale_inv = torch.nn.Parameter(layer.weight_scale_inv.data, requires_grad=False)
+            return
+        weight, weight_scale, input_scale = process_weights_after_loading(
+            layer.weight.data,
+            getattr(layer, "weight_scale", None),
+            getattr(layer, "logical_widths", None),
+            getattr(layer, "input_scale", None),
+            block_quant=False,
+            is_checkpoint_fp8_serialized=cfg.is_checkpoint_fp8_serialized,
+            static_activations=static,
+        )
+        layer.weight = torch.nn.Parameter(weight, requires_grad=False)
+        layer.weight_scale = torch.nn.Parameter(weight_scale, requires_grad=False)
+        layer.input_scale = torch.nn.Parameter(input_scale, requires_grad=False) if input_scale is not None else None
+
+    def apply(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        from .fp8_utils import apply_fp8_linear
+
+        if self.block_quant:
+            return self.w8a8_block_fp8_linear(
+                input=x,
+                weight=layer.weight,
+                block_size=self.quant_config.weight_block_size,
+                weight_scale=layer.weight_scale_inv,
+                input_scale=None,
+                bias=bias,
+            )
+        return apply_fp8_linear(
+            input=x,
+            weight=layer.weight,
+            weight_scale=layer.weight_scale,
+            input_scale=layer.input_scale,
+            bias=bias,
+            cutlass_fp8_supported=self.cutlass_fp8_supported,
+            use_per_token_if_dynamic=False,
+        )

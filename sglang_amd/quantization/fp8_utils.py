@@ -9,7 +9,13 @@ import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from ..sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
-from .fp8_kernel import per_token_group_quant_fp8, sglang_per_token_quant_fp8, static_quant_fp8, w8a8_block_fp8_matmul
+from .fp8_kernel import (
+    per_token_group_quant_fp8,
+    scaled_fp8_quant,
+    sglang_per_token_quant_fp8,
+    static_quant_fp8,
+    w8a8_block_fp8_matmul,
+)
 
 
 def w8a8_block_fp8_linear(
@@ -69,22 +75,50 @@ def apply_fp8_linear(
     weight: torch.Tensor,
     weight_scale: torch.Tensor,
     input_scale: Optional[torch.Tensor] = None,
+    input_scale_ub: Optional[torch.Tensor] = None,
     bias: Optional[torch.Tensor] = None,
+    cutlass_fp8_supported: bool = True,
+    use_per_token_if_dynamic: bool = False,
+    pad_output: Optional[bool] = None,
+    compressed_tensor_quant: bool = False,
 ) -> torch.Tensor:
-    """Per-token activation / per-channel weight FP8 linear: the dynamic branch of
-    apply_fp8_linear that ends in fp8_scaled_mm (fp8_utils.py:693,720-733).
+    """FP8 linear with per-token or per-tensor activation scales and per-channel or per-tensor
+    weight scales: apply_fp8_linear (fp8_utils.py:539-778), same parameters in the same order,
+    every branch ending in this library's fp8_scaled_mm.
 
-    weight is the [K, N] transposed view, weight_scale one fp32 per output channel."""
+    weight is the [K, N] transposed view of the stored [N, K] codes; weight_scale has one fp32
+    per output channel ([N, 1] or [N]) or a single element.
+
+    * default branch (:684-733): a static `input_scale` quantizes through static_quant_fp8 with
+      the scale repeated per token; otherwise the activations are quantized per token.
+    * `compressed_tensor_quant` (:567-596): scaled_fp8_quant(input, input_scale,
+      use_per_token_if_dynamic=...), i.e. static per-tensor, dynamic per-tensor or dynamic
+      per-token activation scales.
+    * A per-tensor activation scale is repeated per token and a per-tensor weight scale per
+      channel before the GEMM, which takes [M] and [N] scales; the reference sends those cases
+      to torch._scaled_mm (:644-655,735-748), whose result is the same product.
+    * `input_scale_ub` is accepted and unused, as in the reference's body.  `pad_output` only
+      pads rows for torch._scaled_mm there and has no effect here.  `cutlass_fp8_supported`
+      chooses between the sgl_kernel GEMM and torch._scaled_mm in the reference; this library has
+      one GEMM and uses it for either value."""
+    del input_scale_ub, pad_output, cutlass_fp8_supported
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[1]]
-    if input_scale is not None:
+    if compressed_tensor_quant:
+        qinput, x_scale = scaled_fp8_quant(input_2d.contiguous(), input_scale, use_per_token_if_dynamic=use_per_token_if_dynamic)
+    elif input_scale is not None:
         # static per-tensor activation scale, broadcast to one scale per token because the GEMM
         # takes per-token scales (fp8_utils.py:684-689)
         assert input_scale.numel() == 1
         qinput, x_scale = static_quant_fp8(input_2d.contiguous(), input_scale, repeat_scale=True)
     else:
-        qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
-    assert weight_scale.numel() == weight.shape[1], "cutlass w8a8 fp8 sgl-kernel only supports per-channel scale"
+        qinput, x_scale = sglang_per_token_quant_fp8(input_2d.contiguous())
+    m, n = qinput.shape[0], weight.shape[1]
+    if x_scale.numel() == 1 and m != 1:
+        x_scale = x_scale.reshape(1, 1).expand(m, 1).contiguous()
+    if weight_scale.numel() == 1 and n != 1:
+        weight_scale = weight_scale.to(torch.float32).reshape(1, 1).expand(n, 1).contiguous()
+    assert weight_scale.numel() == n, "fp8_scaled_mm takes one weight scale per output channel (or a single one)"
     output = fp8_scaled_mm(qinput, weight, x_scale, weight_scale, out_dtype=input.dtype, bias=bias)
     return output.view(*output_shape)
 

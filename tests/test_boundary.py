@@ -206,6 +206,11 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 4, 2, 12, 8, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 2, 4, 2, 8, 8, None) == 2 and b"Half or BFloat16" in lib.sglq_last_error()
     assert lib.sglq_apply_shuffle_mul_sum(p, p, p, None, 0, 0, 2, 8, 8, None) == 0
+    # output rows are written in 16-byte pieces: N and ldo multiples of 8 (4 for int32), base 16-byte aligned
+    assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 12, 0, 4, 12, 32, None, 0, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
+    assert lib.sglq_fp8_scaled_mm(p, 32, p, 32, p, p, None, p, 20, 0, 4, 16, 32, None, 0, None) == 1 and b"multiples of 8" in lib.sglq_last_error()
+    assert lib.sglq_fp8_blockwise_scaled_mm(p, 128, p, 128, p, 1, 4, p, 1, 1, p + 8, 8, 0, 4, 8, 128, None, 0, None) == 1 and b"16-byte aligned" in lib.sglq_last_error()
+    assert lib.sglq_int8_mm_i32(p, 32, p, 32, p, 6, 4, 6, 32, None, 0, None) == 1 and b"multiples of 4" in lib.sglq_last_error()
     # empty problems are a no-op
     assert lib.sglq_int8_scaled_mm(p, 32, p, 32, p, p, None, p, 8, 0, 0, 8, 32, None, 0, None) == 0
 

@@ -227,3 +227,111 @@ def test_requantize_fused_shards_with_max_scale(gpu):
     init = torch.tensor([1.5, torch.finfo(torch.float8_e4m3fn).min, torch.finfo(torch.float8_e4m3fn).min])
     m2, w3 = requantize_with_max_scale(untouched, init.to(gpu), [32, 32, 32])
     assert m2.item() == 1.5 and torch.equal(w3.cpu().view(torch.uint8), codes.view(torch.uint8))
+
+
+def _fp8_linear_case(m, n, k, seed):
+    x = O.gen_activation(m, k, seed=seed)
+    wq, ws = O.per_tensor_quant_weight(O.gen_weight(n, k, seed=seed + 1))
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(seed + 2)) * 0.1).to(torch.bfloat16)
+    return x, wq, ws, bias
+
+
+def test_apply_fp8_linear_called_as_fp8_linear_method_calls_it(gpu):
+    """The keyword list of Fp8LinearMethod.apply (fp8.py:480-488), dynamic activations."""
+    from sglang_amd.quantization.fp8_utils import apply_fp8_linear
+
+    print("fp8 linear, keyword list of fp8.py", flush=True)
+    x, wq, ws, bias = _fp8_linear_case(33, 1024, 2048, 40)
+    xq, xs = O.per_token_quant_fp8(x)
+    ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16, bias)
+    out = apply_fp8_linear(input=x.to(gpu), weight=wq.to(gpu).t(), weight_scale=ws.to(gpu), input_scale=None,
+                           bias=bias.to(gpu), cutlass_fp8_supported=True, use_per_token_if_dynamic=False)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_linear_method_objects_on_a_layer(gpu):
+    """W8A8Fp8LinearMethod, W8A8Int8LinearMethod and Fp8LinearMethod (block quantization) driven the
+    way a linear layer drives them: process_weights_after_loading(layer), then apply(layer, x, bias)
+    (linear.py:231,406,1295)."""
+    import types
+
+    from sglang_amd.quantization.fp8 import Fp8Config, Fp8LinearMethod
+    from sglang_amd.quantization.w8a8_fp8 import W8A8Fp8Config, W8A8Fp8LinearMethod
+    from sglang_amd.quantization.w8a8_int8 import W8A8Int8LinearMethod
+
+    print("linear methods on a layer", flush=True)
+    P = lambda t: torch.nn.Parameter(t.to(gpu), requires_grad=False)
+    # W8A8 FP8 from a 16-bit checkpoint
+    m, n, k = 24, 512, 1024
+    x = O.gen_activation(m, k, seed=50)
+    w = O.gen_weight(n, k, seed=51).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(52)) * 0.1).to(torch.bfloat16)
+    layer = types.SimpleNamespace(weight=P(w), weight_scale=None)
+    method = W8A8Fp8LinearMethod(W8A8Fp8Config(is_checkpoint_fp8_serialized=False))
+    method.process_weights_after_loading(layer)
+    wq_ref, ws_ref = O.per_token_group_quant_fp8(w, k)
+    assert torch.equal(layer.weight.t().contiguous().cpu().view(torch.uint8), wq_ref.view(torch.uint8))
+    assert torch.equal(layer.weight_scale.cpu(), ws_ref)
+    out = method.apply(layer, x.to(gpu).view(2, 12, k), bias.to(gpu))
+    xq, xs = O.per_token_quant_fp8(x)
+    ref = O.fp8_scaled_mm(xq, wq_ref.t(), xs, ws_ref, torch.bfloat16, bias)
+    assert tuple(out.shape) == (2, 12, n)
+    torch.testing.assert_close(out.cpu().view(m, n).float(), ref.float(), rtol=1e-2, atol=1e-2)
+    # W8A8 INT8
+    wt, s_b, bias8 = O.gen_int8_weight(1024, 768, seed=53)
+    layer = types.SimpleNamespace(weight=P(wt.t().contiguous()), weight_scale=P(s_b.reshape(-1, 1)))
+    method = W8A8Int8LinearMethod()
+    method.process_weights_after_loading(layer)
+    out = method.apply(layer, x.to(gpu), bias8.to(gpu))
+    aq, as_ = O.per_token_quant_int8(x)
+    ref = O.int8_scaled_mm(aq, wt, as_, s_b, torch.bfloat16, bias8)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    # block FP8
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=54))
+    layer = types.SimpleNamespace(weight=P(wq), weight_scale_inv=P(ws))
+    method = Fp8LinearMethod(Fp8Config(is_checkpoint_fp8_serialized=True, weight_block_size=[128, 128]))
+    method.process_weights_after_loading(layer)
+    out = method.apply(layer, x.to(gpu), None)
+    gq, gs = O.per_token_group_quant_fp8(x, 128)
+    ref = O.fp8_blockwise_scaled_mm(gq, wq.t(), gs, ws.t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("per_token", [True, False])
+@pytest.mark.parametrize("static", [False, True])
+def test_apply_fp8_linear_compressed_tensor_branch(gpu, per_token, static):
+    """compressed_tensor_quant=True (fp8_utils.py:567-596; caller
+    compressed_tensors_w8a8_fp8.py:152-160): scaled_fp8_quant decides the activation scale's
+    granularity; a per-tensor scale is repeated per token for the GEMM."""
+    from sglang_amd.quantization.fp8_utils import apply_fp8_linear
+
+    print(f"fp8 linear, compressed-tensors branch per_token={per_token} static={static}", flush=True)
+    m = 20
+    x, wq, ws, bias = _fp8_linear_case(m, 768, 1024, 60)
+    in_scale = torch.tensor([0.015], dtype=torch.float32) if static else None
+    if static:
+        xq, xs = O.per_tensor_quant_fp8(x, in_scale)
+        xs = xs.reshape(1, 1).expand(m, 1).contiguous()
+    elif per_token:
+        xq, xs = O.per_token_quant_fp8(x)
+    else:
+        xq, xs = O.per_tensor_quant_fp8(x)
+        xs = xs.reshape(1, 1).expand(m, 1).contiguous()
+    ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16, bias)
+    out = apply_fp8_linear(input=x.to(gpu), weight=wq.to(gpu).t(), weight_scale=ws.to(gpu),
+                           input_scale=in_scale.to(gpu) if static else None, bias=bias.to(gpu),
+                           use_per_token_if_dynamic=per_token, compressed_tensor_quant=True)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_apply_fp8_linear_per_tensor_weight_scale(gpu):
+    """A single weight scale (the reference's torch._scaled_mm case, fp8_utils.py:735-748) is
+    repeated per channel."""
+    from sglang_amd.quantization.fp8_utils import apply_fp8_linear
+
+    print("fp8 linear, one weight scale", flush=True)
+    x, wq, ws, bias = _fp8_linear_case(17, 512, 1024, 70)
+    xq, xs = O.per_token_quant_fp8(x)
+    ref = O.fp8_scaled_mm(xq, wq.t(), xs, ws, torch.bfloat16, bias)
+    out = apply_fp8_linear(x.to(gpu), wq.to(gpu).t(), ws[:1].reshape(1).to(gpu), bias=bias.to(gpu), cutlass_fp8_supported=False)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
