@@ -142,6 +142,26 @@ int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b,
                                       int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                       int64_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference.  sglq_fp8_blockwise_scaled_mm for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it) and therefore have no workspace to pass: the split-K partial sums go through a
+ * fixed device array of SGLQ_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held
+ * until the process ends) and the call allocates nothing.  Same arguments, checks and results
+ * as sglq_fp8_blockwise_scaled_mm called with a workspace of that size.  Problems with
+ * M * N > SGLQ_NOALLOC_MAX_OUTPUTS are rejected with SGLQ_EINVAL.  All calls on one GPU share
+ * that GPU's array: calls that overlap on one GPU (two streams, two threads) race on the
+ * partial sums and must be serialised by the caller; calls in sequence on one stream are safe
+ * (the array needs no clearing between calls).  The array's address is resolved per device on
+ * the first call there, or by sglq_init() with that device current: call either once before
+ * capturing a graph. */
+#define SGLQ_NOALLOC_SCRATCH_BYTES (32ll << 20)
+#define SGLQ_NOALLOC_MAX_OUTPUTS (SGLQ_NOALLOC_SCRATCH_BYTES / 8)
+int sglq_init(void);
+int sglq_fp8_blockwise_scaled_mm_noalloc(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                         int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                         int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                         int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.fp8_blockwise_scaled_grouped_mm
  * (sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:587-754; schema
  * common_extension.cc:192-197; callers python/sglang/srt/layers/moe/cutlass_moe.py:170-213):

@@ -32,6 +32,9 @@ SIGNATURES = {
     "sglq_static_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                      c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
+    "sglq_fp8_blockwise_scaled_mm_noalloc": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                             c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
+    "sglq_init": [],
     "sglq_fp8_blockwise_scaled_mm_bias": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                           c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_grouped_mm": [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p,

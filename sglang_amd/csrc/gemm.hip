@@ -2738,3 +2738,68 @@ extern "C" int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64
   launch_kind<KIND_I8_RAW, SGLQ_BF16>(p, workspace_bytes, static_cast<hipStream_t>(stream));
   return finish(name);
 }
+
+// ---------------------------------------------------------------------------
+// The block-scaled FP8 GEMM for callers that cannot allocate device memory (code under HIP
+// graph capture, serving loops, harnesses that forbid it): the split-K partial sums pass through
+// a fixed array in device memory instead of a caller workspace.  Every GPU the library runs on
+// holds its own copy of the array, at its own address, until the process ends.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[SGLQ_NOALLOC_SCRATCH_BYTES];
+
+// In host code `scratch` is a stand-in for the symbol, not a device address: the address of the
+// current device's copy comes from hipGetSymbolAddress, once per device.
+static std::mutex g_scratch_lock;
+static void* g_scratch_ptr[sglq::MAX_DEVICES];
+
+static int scratch_of_current_device(const char* name, void** ptr_out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("%s: hipGetDevice failed: %s", name, hipGetErrorString(e));
+    return SGLQ_ELAUNCH;
+  }
+  if (dev < 0 || dev >= sglq::MAX_DEVICES) {
+    set_error("%s: device ordinal %d is beyond the %d this library keeps scratch addresses for", name, dev, sglq::MAX_DEVICES);
+    return SGLQ_EUNSUPPORTED;
+  }
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", name, dev, hipGetErrorString(e));
+      return SGLQ_ELAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *ptr_out = g_scratch_ptr[dev];
+  return SGLQ_OK;
+}
+
+extern "C" int sglq_init(void) {
+  void* ptr = nullptr;
+  return scratch_of_current_device("sglq_init", &ptr);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_mm_noalloc(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                                    const float* sfa, int64_t sfa_stride_m, int64_t sfa_stride_k,
+                                                    const float* sfb, int64_t sfb_stride_k, int64_t sfb_stride_n,
+                                                    void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N,
+                                                    int64_t K, void* stream) {
+  const char* name = "fp8_blockwise_scaled_mm_noalloc";
+  // two fp32 partial sums per output must fit, so that split-K (the reason for the scratch) can apply
+  if (M > 0 && N > 0 && M * N > SGLQ_NOALLOC_MAX_OUTPUTS) {
+    set_error("%s: M * N = %lld exceeds the %lld outputs that the %lld-byte device scratch serves; use "
+              "sglq_fp8_blockwise_scaled_mm with a caller-owned workspace",
+              name, (long long)(M * N), (long long)SGLQ_NOALLOC_MAX_OUTPUTS, (long long)SGLQ_NOALLOC_SCRATCH_BYTES);
+    return SGLQ_EINVAL;
+  }
+  void* ws = nullptr;
+  const int rc = scratch_of_current_device(name, &ws);
+  if (rc) return rc;
+  // The partial sums of a split are written in full before the reduction reads them, so nothing
+  // in the scratch has to start at zero and no clearing pass is needed.
+  return blockwise_entry<KIND_FP8_BLOCK>(name, a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb, sfb_stride_k, sfb_stride_n,
+                                         nullptr, out, ldo, out_dtype, M, N, K, ws, SGLQ_NOALLOC_SCRATCH_BYTES, stream);
+}

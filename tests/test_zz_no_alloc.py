@@ -1,0 +1,71 @@
+"""The entry point that allocates nothing, sglq_fp8_blockwise_scaled_mm_noalloc, against
+sglq_fp8_blockwise_scaled_mm called with a caller workspace of the same size: the outputs must be
+identical bit for bit (same kernels, same split-K factors), on calls in a row that share the
+library's device scratch, the later ones smaller than the first."""
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SCRATCH_BYTES = 32 << 20  # SGLQ_NOALLOC_SCRATCH_BYTES in include/sglq.h
+
+
+def _case(m, n, k, seed, dev):
+    x = O.gen_activation(m, k, seed=seed)
+    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=seed + 1))
+    xq, xs = O.per_token_group_quant_fp8(x, 128)
+    return xq, xs, wq, ws, xq.to(dev), xs.to(dev), wq.to(dev), ws.to(dev)
+
+
+def _call(lib, name, a, b, sa, sb, out, m, n, k, extra):
+    fn = getattr(lib, name)
+    # weight [N, K] row-major = the column-major [K, N] operand; row-major activation scales;
+    # weight scales [N/128, K/128] as stored: strides (k, n) = (1, K/128)
+    return fn(a.data_ptr(), k, b.data_ptr(), k, sa.data_ptr(), sa.stride(0), sa.stride(1), sb.data_ptr(), sb.stride(1), sb.stride(0),
+              out.data_ptr(), n, 0, m, n, k, *extra, torch.cuda.current_stream().cuda_stream)
+
+
+def test_noalloc_entry_point_matches_the_workspace_entry_point(gpu):
+    from sglang_amd import _lib
+
+    lib = _lib.load()
+    assert lib.sglq_init() == 0, lib.sglq_last_error()
+    workspace = torch.empty(SCRATCH_BYTES, dtype=torch.uint8, device=gpu)
+    # split-K decode kernel (4 splits), then the pipelined kernel with K split over work units,
+    # then a smaller split-K problem whose partial sums land on the first calls' leftovers
+    shapes = [(64, 7168, 16384), (512, 4096, 7168), (40, 512, 4096), (64, 7168, 16384), (8, 2112, 7168)]
+    for i, (m, n, k) in enumerate(shapes):
+        print(f"noalloc case {i}: {m} x {n} x {k}", flush=True)
+        xq, xs, wq, ws, dxq, dxs, dwq, dws = _case(m, n, k, 9000 + 10 * i, gpu)
+        want = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+        got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=gpu)
+        rc = _call(lib, "sglq_fp8_blockwise_scaled_mm", dxq, dwq, dxs, dws, want, m, n, k, (workspace.data_ptr(), workspace.numel()))
+        assert rc == 0, lib.sglq_last_error()
+        kernel = lib.sglq_debug_last_gemm_kernel().decode()
+        rc = _call(lib, "sglq_fp8_blockwise_scaled_mm_noalloc", dxq, dwq, dxs, dws, got, m, n, k, ())
+        assert rc == 0, lib.sglq_last_error()
+        assert lib.sglq_debug_last_gemm_kernel().decode() == kernel
+        if i < 4:
+            assert "splitk" in kernel, kernel  # these shapes are here because they use the scratch
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"case {i} ({kernel}) differs from the workspace entry point"
+        rows = sorted(set([0, m - 1, m // 2, (m * 3) // 7]))
+        ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32)
+        torch.testing.assert_close(got[rows].cpu().float(), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_noalloc_entry_point_rejects_what_the_scratch_cannot_serve(gpu):
+    from sglang_amd import _lib
+
+    lib = _lib.load()
+    t = torch.zeros(4096, dtype=torch.uint8, device=gpu)
+    p = t.data_ptr()
+    # M * N above SGLQ_NOALLOC_MAX_OUTPUTS = 4 Mi: refused before anything is launched
+    rc = lib.sglq_fp8_blockwise_scaled_mm_noalloc(p, 128, p, 128, p, 1, 1, p, 1, 1, p, 4096, 0, 4096, 4096, 128, None)
+    assert rc == 1 and b"exceeds" in lib.sglq_last_error() and b"workspace" in lib.sglq_last_error()
+    # the other checks are the workspace entry point's
+    rc = lib.sglq_fp8_blockwise_scaled_mm_noalloc(p, 128, p, 128, p, 1, 1, p, 1, 1, p, 12, 0, 4, 12, 128, None)
+    assert rc == 1 and b"multiples of 8" in lib.sglq_last_error()
+    assert lib.sglq_fp8_blockwise_scaled_mm_noalloc(p, 128, p, 128, p, 1, 1, p, 1, 1, p, 8, 0, 0, 8, 128, None) == 0
