@@ -1,8 +1,9 @@
-"""Build recipe for libsglq.so (hipcc, gfx950 only).
+"""Build recipe for libsglq.so and libsglq_bench.so (hipcc, gfx950 only).
 
-``python -m sglang_amd.build`` compiles every HIP source under ``csrc/`` into
-``sglang_amd/libsglq.so``.  The shared object has a plain C ABI (``include/sglq.h``)
-and does not link against torch.
+``python -m sglang_amd.build`` compiles the operator sources under ``csrc/`` into
+``sglang_amd/libsglq.so`` (plain C ABI, ``include/sglq.h``; does not link against torch) and
+the measurement kernels (``csrc/bench_kernels.hip``: MFMA ceiling loop, clock probe, streaming
+passes) into ``sglang_amd/libsglq_bench.so``, which only ``bench.py`` loads.
 """
 
 from __future__ import annotations
@@ -16,7 +17,9 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libsglq.so"
+BENCH_LIB_PATH = PKG_DIR / "libsglq_bench.so"
 SOURCES = ["common.hip", "quant.hip", "moe.hip", "gemm.hip"]
+BENCH_SOURCES = ["bench_kernels.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -43,9 +46,10 @@ def build(verbose: bool = False, jobs: int = 4) -> Path:
     obj_dir.mkdir(exist_ok=True)
     procs = []
     objs = []
-    for src in SOURCES:
+    bench_objs = []
+    for src in SOURCES + BENCH_SOURCES:
         obj = obj_dir / (src + ".o")
-        objs.append(str(obj))
+        (bench_objs if src in BENCH_SOURCES else objs).append(str(obj))
         cmd = [hipcc, *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -59,6 +63,12 @@ def build(verbose: bool = False, jobs: int = 4) -> Path:
     out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if out.returncode != 0:
         raise RuntimeError("link failed:\n" + out.stdout)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", str(BENCH_LIB_PATH), *bench_objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        raise RuntimeError("link of the measurement kernels failed:\n" + out.stdout)
     return LIB_PATH
 
 

@@ -1,0 +1,218 @@
+// Measurement kernels for gfx950 (built into libsglq_bench.so, not into the operator library):
+//   * a register-only MFMA loop, the ceiling that the matrix pipe sustains on real operand
+//     bytes at the clock the chip settles to under that load,
+//   * a clock probe (shader-clock and constant-rate counters per XCD), from which a harness
+//     derives the average shader clock over a timed region,
+//   * a plain copy and a read-only / write-only pass of known size, the yardsticks for the
+//     FETCH_SIZE / WRITE_SIZE profiler counters and for the memory system's streaming rate.
+// C ABI, raw pointers, nothing allocated; every kernel runs a bounded loop.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+namespace {
+
+// Variants of the MFMA loop.  One iteration is the K step of a 128 x 64 wave tile:
+// 32 x v_mfma_f32_16x16x128_f8f6f4 or 16 x v_mfma_f32_32x32x64_f8f6f4 = 2 097 152 flop per wave.
+constexpr int ACCUMULATE_16 = 0;  // 16x16x128, accumulating in place (per-row/per-column kinds)
+constexpr int FOLD_16 = 1;        // 16x16x128 from a zero accumulator, result folded in with 4 FMAs (block-scaled kind)
+constexpr int ACCUMULATE_32 = 2;  // 32x32x64, accumulating in place
+constexpr int FOLD_32 = 3;        // 32x32x64 in pairs (one 128-byte K block), the pair's result folded in with 16 FMAs
+
+struct ClockSample {
+  uint64_t shader_cycles, realtime_ticks;
+};
+
+__device__ __forceinline__ ClockSample read_clocks() {
+  ClockSample s;
+  s.shader_cycles = __builtin_readcyclecounter();      // s_memtime: counts at the shader clock
+  s.realtime_ticks = __builtin_amdgcn_s_memrealtime(); // constant-rate reference counter
+  return s;
+}
+
+template <int VARIANT>
+__global__ __launch_bounds__(512) void mfma_ceiling_kernel(const v8i* __restrict__ operands, int iters, float* __restrict__ sink,
+                                                           uint64_t* __restrict__ clocks) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // six operand registers' worth of bytes per lane, distinct per wave (6 x 512 x 32 B = 96 KiB are read)
+  v8i a[2], b[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) a[i] = operands[(i * 8 + wave) * 64 + lane];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b[j] = operands[((2 + j) * 8 + wave) * 64 + lane];
+  const float scale = 1.0f + 1e-6f * (float)lane;
+
+  ClockSample t0 = read_clocks();
+  if constexpr (VARIANT == ACCUMULATE_16 || VARIANT == FOLD_16) {
+    v4f acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+      // the operands are opaque to the compiler in every iteration: nothing is hoisted
+      asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+      v4f prev = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        asm volatile("" : "+v"(a[i & 1]));  // a new activation fragment as far as the compiler knows
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if constexpr (VARIANT == ACCUMULATE_16) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], a[i & 1], acc[i][j], 0, 0, 0, 0, 0, 0);
+          } else {
+            const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], a[i & 1], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            const int idx = i * 4 + j;
+            if (idx > 0) {  // fold the previous result while this MFMA runs
+              const int pi = (idx - 1) / 4, pj = (idx - 1) % 4;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[pi][pj][e] = __builtin_fmaf(prev[e], scale, acc[pi][pj][e]);
+            }
+            prev = part;
+          }
+        }
+      }
+      if constexpr (VARIANT == FOLD_16) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[7][3][e] = __builtin_fmaf(prev[e], scale, acc[7][3][e]);
+      }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    sink[blockIdx.x * 512 + threadIdx.x] = s;
+  } else {
+    v16f acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+      asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+      v16f prev;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) prev[e] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        asm volatile("" : "+v"(a[0]), "+v"(a[1]));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if constexpr (VARIANT == ACCUMULATE_32) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[j], a[i & 1], acc[i][j], 0, 0, 0, 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[2 + j], a[(i + 1) & 1], acc[i][j], 0, 0, 0, 0, 0, 0);
+          } else {
+            v16f zero;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) zero[e] = 0.f;
+            v16f part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[j], a[i & 1], zero, 0, 0, 0, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[2 + j], a[(i + 1) & 1], part, 0, 0, 0, 0, 0, 0);
+            const int idx = i * 2 + j;
+            if (idx > 0) {
+              const int pi = (idx - 1) / 2, pj = (idx - 1) % 2;
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[pi][pj][e] = __builtin_fmaf(prev[e], scale, acc[pi][pj][e]);
+            }
+            prev = part;
+          }
+        }
+      }
+      if constexpr (VARIANT == FOLD_32) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[3][1][e] = __builtin_fmaf(prev[e], scale, acc[3][1][e]);
+      }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+    sink[blockIdx.x * 512 + threadIdx.x] = s;
+  }
+  ClockSample t1 = read_clocks();
+  if (threadIdx.x == 0) {
+    clocks[2 * blockIdx.x] = t1.shader_cycles - t0.shader_cycles;
+    clocks[2 * blockIdx.x + 1] = t1.realtime_ticks - t0.realtime_ticks;
+  }
+}
+
+// One sample of both counters per XCD: slot = the XCC id of the CU the block runs on.
+// Blocks on the same XCD write nearly identical values; the last writer stays.
+__global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t* __restrict__ out) {
+  if (threadIdx.x != 0) return;
+  const ClockSample s = read_clocks();
+  // HW_REG_XCC_ID (hardware register 20), bits 3:0
+  const uint32_t xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & 15u;
+  out[2 * xcc] = s.shader_cycles;
+  out[2 * xcc + 1] = s.realtime_ticks;
+}
+
+// mode 0: dst = src; 1: read src only (one value per block written at the end); 2: write dst only
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, int64_t n16, int* __restrict__ sink) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  v4i keep = {0, 0, 0, 0};
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) {
+    if constexpr (MODE == 0) dst[i] = src[i];
+    if constexpr (MODE == 1) {
+      const v4i v = src[i];
+      keep[0] ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+    }
+    if constexpr (MODE == 2) dst[i] = v4i{(int)i, 1, 2, 3};
+  }
+  if constexpr (MODE == 1) {
+    if (keep[0] == 0x5a5a5a5a) sink[blockIdx.x] = keep[0];  // practically never: keeps the loads alive
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// variant 0..3 (see above); operands: 96 KiB of e4m3 bytes (no NaN codes); sink: blocks * 512 floats;
+// clocks: blocks * 2 uint64 (shader cycles, constant-rate ticks of each block).  8 waves per block,
+// one block per CU when blocks = the CU count.  Returns the HIP error code of the launch.
+int sglqb_mfma_ceiling(int variant, int iters, const void* operands, float* sink, uint64_t* clocks, int blocks, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const v8i* ops = static_cast<const v8i*>(operands);
+  if (blocks <= 0 || iters < 0 || !operands || !sink || !clocks) return -1;
+  switch (variant) {
+    case ACCUMULATE_16: mfma_ceiling_kernel<ACCUMULATE_16><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
+    case FOLD_16: mfma_ceiling_kernel<FOLD_16><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
+    case ACCUMULATE_32: mfma_ceiling_kernel<ACCUMULATE_32><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
+    case FOLD_32: mfma_ceiling_kernel<FOLD_32><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}
+
+// out: 16 x 2 uint64 (per XCC id: shader cycles, constant-rate ticks), zero-filled by the caller.
+int sglqb_clock_probe(uint64_t* out, int blocks, void* stream) {
+  if (!out || blocks <= 0) return -1;
+  clock_probe_kernel<<<blocks, 64, 0, static_cast<hipStream_t>(stream)>>>(out);
+  return (int)hipGetLastError();
+}
+
+// mode 0 copy, 1 read only, 2 write only over `bytes` (a multiple of 16); sink: `blocks` ints.
+int sglqb_stream(int mode, const void* src, void* dst, int64_t bytes, int* sink, int blocks, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (bytes < 0 || bytes % 16 != 0 || blocks <= 0) return -1;
+  const v4i* s = static_cast<const v4i*>(src);
+  v4i* d = static_cast<v4i*>(dst);
+  if (mode == 0) stream_kernel<0><<<blocks, 256, 0, st>>>(s, d, bytes / 16, sink);
+  else if (mode == 1) stream_kernel<1><<<blocks, 256, 0, st>>>(s, d, bytes / 16, sink);
+  else if (mode == 2) stream_kernel<2><<<blocks, 256, 0, st>>>(s, d, bytes / 16, sink);
+  else return -1;
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"
