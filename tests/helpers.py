@@ -74,6 +74,27 @@ def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
 FP8 = torch.float8_e4m3fn
 
 
+def rows_per_tile(m: int, cap: int = 48, seed: int = 0) -> torch.Tensor:
+    """Rows on which a large GEMM is compared with the oracle, chosen so that every row tile of
+    every kernel is read: the first, the last and one random row of each 64-row tile up to
+    M = 1024 and of each 256-row tile (the persistent kernels' tile height, which also covers
+    their second-round tiles and the hand-over between consecutive tiles of a block) above,
+    plus one row for each of the 16 positions inside an MFMA fragment and the rows 1 and M - 2.
+    Up to `cap` rows all rows are taken."""
+    if m <= cap:
+        return torch.arange(m)
+    g = torch.Generator().manual_seed(1000003 * seed + m)
+    tile = 64 if m <= 1024 else 256
+    rows = [0, 1, m - 2, m - 1]
+    for t0 in range(0, m, tile):
+        t1 = min(m, t0 + tile)
+        rows += [t0, t1 - 1, t0 + int(torch.randint(0, t1 - t0, (1,), generator=g))]
+    for pos in range(16):  # every lane row of a 16-row fragment, each in a random fragment
+        frag = int(torch.randint(0, m // 16, (1,), generator=g))
+        rows.append(frag * 16 + pos)
+    return torch.tensor(sorted(set(r for r in rows if 0 <= r < m)))
+
+
 def moe_case(num_experts, rows_per_expert, n, k, seed, dtype=torch.bfloat16):
     """Inputs built the way the reference's grouped-GEMM test builds them
     (sgl-kernel/tests/test_fp8_blockwise_moe.py:39-63,119-190): N(0,1) activations quantized per

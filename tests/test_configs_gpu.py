@@ -2,11 +2,13 @@
 checked against the oracle: codes and scales bit-exact, INT32 accumulators exact,
 bf16 outputs within rtol/atol 1e-2.  Activations are generated on the CPU with
 the configuration's seed and the same bytes go to both sides; for large M the
-oracle is evaluated on a row sample (every row is independent of the others)."""
+oracle is evaluated on rows of every row tile (first, last and a random row of each tile plus
+every position inside an MFMA fragment: about 110 rows at M = 8192), and the whole output is
+compared with the generic 128 x 128 kernel's, which the same oracle rows validate."""
 import pytest
 import torch
 
-from helpers import assert_bits_equal
+from helpers import assert_bits_equal, rows_per_tile
 from oracle import w8a8_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -27,11 +29,28 @@ def block_weight(n, k, seed):
     return _weights[key]
 
 
-def rows_of(m, cap=16):
-    if m <= cap:
-        return torch.arange(m)
-    g = torch.Generator().manual_seed(m)
-    return torch.cat([torch.randperm(m, generator=g)[: cap - 2], torch.tensor([0, m - 1])]).unique()
+def rows_of(m):
+    return rows_per_tile(m, cap=16)
+
+
+def whole_output_check(fn, out, m, what):
+    """Every element of a large output against the same GEMM on the generic 128 x 128 kernel
+    (forced through the test hook), whose result the oracle rows validate as well: a wrong tile,
+    scale or K block anywhere in the output of the selected kernel shows up here."""
+    from sglang_amd import _lib
+
+    if m < 512:
+        return
+    lib = _lib.load()
+    selected = lib.sglq_debug_last_gemm_kernel().decode()
+    lib.sglq_debug_force_tile(128)
+    try:
+        generic = fn()
+        assert lib.sglq_debug_last_gemm_kernel().decode().startswith("gemm_kernel")
+    finally:
+        lib.sglq_debug_force_tile(0)
+    torch.testing.assert_close(out.float(), generic.float(), rtol=RTOL, atol=ATOL, msg=lambda s: f"{what} ({selected}) vs generic kernel: {s}")
+    return generic
 
 
 def run_block_case(gpu, m, n, k, seed, outliers=False):
@@ -47,9 +66,13 @@ def run_block_case(gpu, m, n, k, seed, outliers=False):
     assert_bits_equal(xq[rows.to(gpu)], xq_ref, "FP8 codes")
     assert_bits_equal(xs[rows.to(gpu)].contiguous(), xs_ref, "group scales")
     wq_g = wq.to(gpu)
-    out = fp8_blockwise_scaled_mm(xq, wq_g.t(), xs, ws.to(gpu).t(), torch.bfloat16)
+    ws_g = ws.to(gpu)
+    out = fp8_blockwise_scaled_mm(xq, wq_g.t(), xs, ws_g.t(), torch.bfloat16)
     ref = O.fp8_blockwise_scaled_mm(xq_ref, wq.t(), xs_ref, ws.t(), torch.float32)
     torch.testing.assert_close(out[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+    generic = whole_output_check(lambda: fp8_blockwise_scaled_mm(xq, wq_g.t(), xs, ws_g.t(), torch.bfloat16), out, m, f"block {m}x{n}x{k}")
+    if generic is not None:
+        torch.testing.assert_close(generic[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
 
 
 def test_config0(gpu):
@@ -83,10 +106,13 @@ def _config3_case(gpu, m, n, k, wq, ws):
     xq, xs = sglang_per_token_quant_fp8(x.to(gpu))
     assert_bits_equal(xq[rows.to(gpu)], xq_ref, "FP8 codes")
     assert_bits_equal(xs[rows.to(gpu)], xs_ref, "token scales")
+    wq_g, ws_g = wq.to(gpu), ws.to(gpu)
     for b in (None, bias):
-        out = fp8_scaled_mm(xq, wq.to(gpu).t(), xs, ws.to(gpu), torch.bfloat16, None if b is None else b.to(gpu))
+        bg = None if b is None else b.to(gpu)
+        out = fp8_scaled_mm(xq, wq_g.t(), xs, ws_g, torch.bfloat16, bg)
         ref = O.fp8_scaled_mm(xq_ref, wq.t(), xs_ref, ws, torch.float32, b)
         torch.testing.assert_close(out[rows.to(gpu)].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+        whole_output_check(lambda: fp8_scaled_mm(xq, wq_g.t(), xs, ws_g, torch.bfloat16, bg), out, m, f"per-channel {m}x{n}x{k}")
 
 
 @pytest.mark.parametrize("nk", LLAMA70B_NK)

@@ -4,6 +4,7 @@ path's contract states for floating-point outputs)."""
 import pytest
 import torch
 
+from helpers import rows_per_tile
 from oracle import w8a8_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -21,11 +22,8 @@ def rand_i8(shape, seed, lo=-128, hi=128):
 
 
 def sample_rows(m, cap=48):
-    if m <= cap:
-        return torch.arange(m)
-    g = torch.Generator().manual_seed(m)
-    idx = torch.randperm(m, generator=g)[: cap - 4]
-    return torch.cat([idx, torch.tensor([0, 1, m - 2, m - 1])]).unique()
+    """Rows of every row tile (see helpers.rows_per_tile)."""
+    return rows_per_tile(m, cap)
 
 
 @pytest.fixture(params=[1, 0], ids=["direct_lds", "via_regs"])
