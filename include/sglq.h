@@ -142,6 +142,25 @@ int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b,
                                       int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                       int64_t workspace_bytes, void* stream);
 
+/* The call pair of cutlass_w8a8_block_fp8_linear_with_fallback
+ * (python/sglang/srt/layers/quantization/fp8_utils.py:204-211: per_token_group_quant_fp8 with
+ * groups of 128, fp8_blockwise_scaled_mm, `output += bias`) as one entry point, the fused form
+ * that the reference's CPU backend has for its INT8 path (sgl-kernel/csrc/cpu/gemm_int8.cpp:422-489):
+ *   x    [M, K] contiguous activations, in_dtype in {BF16, FP16, FP32}, 16-byte aligned, K % 128 == 0
+ *   b, sfb, bias (may be NULL), out: as sglq_fp8_blockwise_scaled_mm_bias
+ *   eps  lower bound of a group's abs-max (the callers' 1e-10)
+ * For M <= 8 (16-bit activations) on the shapes that the decode kernel without split-K takes, one
+ * kernel quantizes each K block's activations in LDS right before multiplying them: no
+ * quantization launch, no round trip of codes and scales through memory, no workspace.  Other
+ * shapes run the quantization kernel and the GEMM one after the other; their codes and
+ * column-major scales need M * K + 4 * M * K / 128 bytes (each rounded up to 256) at the head of
+ * the 16-byte aligned workspace, the rest serves the GEMM's split-K as usual.  The output is
+ * bit-identical to sglq_per_token_group_quant_fp8 followed by sglq_fp8_blockwise_scaled_mm(_bias). */
+int sglq_w8a8_block_fp8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* sfb,
+                               int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out, int64_t ldo,
+                               int out_dtype, int64_t M, int64_t N, int64_t K, float eps, void* workspace,
+                               int64_t workspace_bytes, void* stream);
+
 /* No counterpart in the reference.  sglq_fp8_blockwise_scaled_mm for callers that cannot
  * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
  * forbid it) and therefore have no workspace to pass: the split-K partial sums go through a

@@ -35,6 +35,8 @@ SIGNATURES = {
     "sglq_fp8_blockwise_scaled_mm_noalloc": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                              c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
     "sglq_init": [],
+    "sglq_w8a8_block_fp8_linear": [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int,
+                                   c_int64, c_int64, c_int64, c_float, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_bias": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                           c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_grouped_mm": [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p,

@@ -24,6 +24,7 @@
 #include <shared_mutex>
 #include <type_traits>
 
+#include "quant_device.h"
 #include "sglq_common.h"
 
 namespace sglq {
@@ -59,6 +60,7 @@ struct GemmArgs {
   int64_t b_expert_stride, sb_expert_stride;  // grouped GEMM: bytes / floats between experts' weights / weight scales
   int num_experts;
   int stream_out;  // the output is larger than the last-level cache: store it with the non-temporal hint
+  float quant_eps;  // fused quantization (gemm_stream_quant_kernel): lower bound of a group's abs-max
 };
 
 // Grouped GEMM tile plan in the workspace (int32): [0] = number of row tiles, then from [4] on
@@ -1874,6 +1876,211 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// gemm_stream_kernel for M <= 8 with the activation quantization folded in: p.a holds the
+// 16-bit activations (row stride p.lda BYTES) instead of FP8 codes and group scales.  A wave
+// streams, next to the weight rows of its K blocks, the 8 x 128 activations of the same K
+// blocks (8 rows x 256 bytes) through its ring, and turns them into the codes and the scale of
+// per-token-group quantization with groups of 128 = one K block right before the block's MFMAs:
+//   * lane l takes 16 elements (32 bytes) of row l / 8; the row's eight lanes are adjacent, so
+//     the group's abs-max is three DPP steps, as in group_quant_kernel;
+//   * scale and codes come from the same device functions as that kernel (quant_device.h):
+//     bit-identical codes and scales;
+//   * the 16 codes of a lane are one 16-byte chunk of the MFMA operand tile: they go to a
+//     wave-private 8 x 128-byte tile in LDS in the swizzled layout of the MFMA operand reads, and
+//     the operand is read back from there (the lanes of fragment rows 8..15, whose results are
+//     never stored, read rows 0..7 again); the row's scale reaches the MFMA lanes of that row
+//     with one cross-lane read.
+// LDS accesses of one wave execute in order, so the tile needs no barrier.  Weight rows, K
+// split over the waves and the order of every sum are those of gemm_stream_kernel<KIND, 1, NIB>:
+// the output equals quantize-then-multiply through that kernel bit for bit, without the
+// quantization launch and without the codes' round trip through memory.
+// ---------------------------------------------------------------------------
+template <int NIB, int OUT_DT, int IN_DT, int ROWS>
+__global__ __launch_bounds__(256) void gemm_stream_quant_kernel(const GemmArgs p) {
+  constexpr int KIND = KIND_FP8_BLOCK;
+  constexpr int BN = NIB * 16, XR = 8;
+  constexpr int WC = BN / 8, XC = XR * 256 / 1024;  // one-KiB copies per stage: weights, activations
+  constexpr int CPW = WC + XC + 1;                  // ... and the weight scale
+  constexpr int W_BYTES = BN * 128, X_BYTES = XR * 256, S_BYTES = 256;
+  constexpr int STAGE_BYTES = W_BYTES + X_BYTES + S_BYTES;
+  constexpr int NSTAGE = SGLQ_STREAM_NSTAGE;
+  constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+  constexpr int TILE_BYTES = 8 * 128;  // the quantized activations of the current K block
+  // ROWS (1, 2, 4 or 8, at least M): rows that take part in the quantization.  A row's 128 elements are
+  // spread over 64 / ROWS adjacent lanes, so that a wave spends 2 ROWS elements' worth of arithmetic
+  // per lane and K block instead of 16 whatever M is.
+  constexpr int LPR = 64 / ROWS, EPL = 128 / LPR, WPL = EPL / 2;  // lanes per row, elements and 32-bit words per lane
+  static_assert(ROWS == 1 || ROWS == 2 || ROWS == 4 || ROWS == 8, "rows per wave");
+  static_assert((NSTAGE - 1) * CPW <= 63, "vmcnt holds 6 bits");
+  static_assert(NIB * 1024 <= RING_BYTES, "the partial sums are exchanged through a wave's ring");
+
+  __shared__ __attribute__((aligned(1024))) char smem[4 * (RING_BYTES + TILE_BYTES)];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4, l8 = lane >> 3;
+  const int n0 = blockIdx.x * BN;
+  const int nkb = p.K >> 7;
+  const int nsteps = (nkb - wave + 3) >> 2;  // K blocks wave, wave + 4, ...
+
+  const v4u rx = make_rsrc_sgpr(p.a, p.a_bytes);
+  const v4u rb = make_rsrc_sgpr(p.b, p.b_bytes);
+
+  // weights: as gemm_stream_kernel (copy gj brings rows 8 gj .. 8 gj + 7, lane l row l / 8, chunk (l % 8) ^ swz(row))
+  const int c16_even = (((lane & 7) ^ l8) & 7) * 16, c16_odd = (((lane & 7) ^ l8 ^ 1) & 7) * 16;
+  const uint32_t offw_even = (uint32_t)(n0 + l8) * p.ldb + c16_even, offw_odd = (uint32_t)(n0 + l8) * p.ldb + c16_odd;
+  const uint32_t step_w = 8u * p.ldb;
+  // activations: copy j brings rows 4 j .. 4 j + 3 of the K block, lane l 16 bytes (8 elements) of row
+  // 4 j + l / 16; rows past M are out of range and read as zero
+  const uint32_t x_piece = (uint32_t)(lane & 15) * 16u;
+  uint32_t offx[XC];
+#pragma unroll
+  for (int j = 0; j < XC; ++j) {
+    const int row = 4 * j + (lane >> 4);
+    offx[j] = row < p.M ? (uint32_t)row * p.lda + x_piece : OOB;
+  }
+  const int nblocks = (p.N + 127) >> 7;
+  const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
+  const v4u rsb = make_rsrc_sgpr(p.sb, (uint32_t)(sfb_elems * 4));
+  int nb = n0 >> 7;  // BN divides 128: one scale block per block of rows
+  if (nb >= nblocks) nb = nblocks - 1;
+  const uint32_t off_sb = lane == 0 ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
+  const int sfb_step = (int)(p.sb_stride_k * 4);
+
+  const uint32_t ring = lds_addr(smem) + (uint32_t)wave * RING_BYTES;
+  auto issue_group = [&](int t) {  // all copies of this wave's t-th K block into slot t % NSTAGE
+    const uint32_t st = ring + (uint32_t)(t % NSTAGE) * STAGE_BYTES;
+    const uint32_t kb = (uint32_t)(wave + 4 * t);
+    const uint32_t kill = t < nsteps ? 0u : OOB;  // past the end: out of range, the K offset is not bounds-checked
+    const uint32_t k0 = t < nsteps ? kb * 128u : 0u;
+#pragma unroll
+    for (int j = 0; j < WC; ++j)
+      lds_copy16(rb, st + j * 1024, (((j & 1) ? offw_odd : offw_even) + j * step_w) | kill, k0);
+#pragma unroll
+    for (int j = 0; j < XC; ++j) lds_copy16(rx, st + W_BYTES + j * 1024, offx[j] | kill, k0 * 2u);
+    lds_copy4(rsb, st + W_BYTES + X_BYTES, off_sb | kill, t < nsteps ? kb * (uint32_t)sfb_step : 0u);
+  };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  v4f acc[NIB];
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  char* my_ring = smem + wave * RING_BYTES;
+  char* my_tile = smem + 4 * RING_BYTES + wave * TILE_BYTES;
+  // operand read of the tile: row r16 % ROWS (swz(row) = row for rows 0..7)
+  const int t_row = r16 & (ROWS - 1);
+  const int tile_off0 = t_row * 128 + (((2 * g) ^ t_row) * 16), tile_off1 = tile_off0 ^ 16;
+  // quantization lanes: row l / LPR, elements EPL (l % LPR) .. + EPL - 1 of the K block; its codes are EPL
+  // bytes of the row's 16-byte chunk EPL (l % LPR) / 16, which sits at chunk position chunk ^ swz(row) = chunk ^ row
+  const int q_row = lane / LPR, q_first = (lane % LPR) * EPL;
+  const int q_src = q_row * 256 + q_first * 2;
+  const int q_dst = q_row * 128 + ((((q_first >> 4) ^ q_row) & 7) * 16) + (q_first & 15);
+  // byte index of a lane that holds the scale of fragment row r16 (rows past ROWS repeat the rows below, like the codes)
+  const int scale_from = ((r16 & (ROWS - 1)) * LPR) * 4;
+
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t) issue_group(t);
+
+  for (int t = 0; t < nsteps; ++t) {
+    issue_group(t + NSTAGE - 1);
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * CPW) : "memory");
+
+    const char* st = my_ring + (t % NSTAGE) * STAGE_BYTES;
+    // ---- per-token-group quantization of this K block's ROWS x 128 activations
+    uint32_t w[WPL];
+    {
+      const char* src = st + W_BYTES + q_src;
+      if constexpr (WPL == 8) {
+        const v4u lo = *reinterpret_cast<const v4u*>(src), hi = *reinterpret_cast<const v4u*>(src + 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = lo[i], w[4 + i] = hi[i];
+      } else if constexpr (WPL == 4) {
+        const v4u lo = *reinterpret_cast<const v4u*>(src);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = lo[i];
+      } else if constexpr (WPL == 2) {
+        const v2u lo = *reinterpret_cast<const v2u*>(src);
+        w[0] = lo.x, w[1] = lo.y;
+      } else {
+        w[0] = *reinterpret_cast<const uint32_t*>(src);
+      }
+    }
+    // |x| of a 16-bit float orders like its low 15 bits taken as an integer (bfloat16 and half alike)
+    v2us m16 = {0, 0};
+#pragma unroll
+    for (int i = 0; i < WPL; ++i) m16 = __builtin_elementwise_max(m16, __builtin_bit_cast(v2us, w[i] & 0x7fff7fffu));
+    uint32_t hmax = m16.x > m16.y ? m16.x : m16.y;
+    if constexpr (LPR == 8) hmax = group_umax<8>(hmax);
+    else if constexpr (LPR == 16) hmax = group_umax<16>(hmax);
+    else if constexpr (LPR == 32) hmax = umax(group_umax<16>(hmax), (uint32_t)__shfl_xor((int)group_umax<16>(hmax), 16));
+    else hmax = wave_umax(hmax);
+    const float amax_x = to_f32_16<IN_DT>((uint16_t)hmax);
+    const float amax = u2f(umax(f2u(amax_x), f2u(p.quant_eps)));
+    const float y_s = div_by(amax, 448.0f, 1.0f / 448.0f);
+    const float rcp = 1.0f / y_s;
+    uint32_t codes[(EPL + 3) / 4];
+#pragma unroll
+    for (int i = 0; i < WPL; ++i) {
+      const float lo = quantize_elem<false>(to_f32_16<IN_DT>((uint16_t)(w[i] & 0xffffu)), y_s, rcp, -448.0f, 448.0f);
+      const float hi = quantize_elem<false>(to_f32_16<IN_DT>((uint16_t)(w[i] >> 16)), y_s, rcp, -448.0f, 448.0f);
+      if (i & 1) codes[i >> 1] = cvt_pk_e4m3<true>(lo, hi, codes[i >> 1]);
+      else codes[i >> 1] = cvt_pk_e4m3<false>(lo, hi, 0);
+    }
+    if constexpr (EPL == 16) *reinterpret_cast<v4u*>(my_tile + q_dst) = v4u{codes[0], codes[1], codes[2], codes[3]};
+    else if constexpr (EPL == 8) *reinterpret_cast<v2u*>(my_tile + q_dst) = v2u{codes[0], codes[1]};
+    else if constexpr (EPL == 4) *reinterpret_cast<uint32_t*>(my_tile + q_dst) = codes[0];
+    else *reinterpret_cast<uint16_t*>(my_tile + q_dst) = (uint16_t)codes[0];
+    // (executed by every lane: a cross-lane read only sees lanes that take part in it)
+    const float sfa = u2f((uint32_t)__builtin_amdgcn_ds_bpermute(scale_from, (int)f2u(y_s)));
+
+    v8i wf[NIB];
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) wf[j] = read_frag(st + j * 16 * 128);
+    const float sfb = *reinterpret_cast<const float*>(st + W_BYTES + X_BYTES);
+    const v4i alo = *reinterpret_cast<const v4i*>(my_tile + tile_off0), ahi = *reinterpret_cast<const v4i*>(my_tile + tile_off1);
+    const v8i af = v8i{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+    const float sc = sfa * sfb;
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) {
+      const v4f part = block_mfma<KIND>(wf[j], af);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[j][e] = __builtin_fmaf(part[e], sc, acc[j][e]);
+    }
+  }
+
+  // as gemm_stream_kernel: waves 1..3 leave their partial sums in their own ring, wave 0 adds them in wave order
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  if (wave != 0) {
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) *reinterpret_cast<v4f*>(my_ring + j * 1024 + lane * 16) = acc[j];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+#pragma unroll
+      for (int j = 0; j < NIB; ++j) {
+        const v4f t = *reinterpret_cast<const v4f*>(smem + w * RING_BYTES + j * 1024 + lane * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[j][e] += t[e];
+      }
+    v4f out_acc[1][NIB];
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) out_acc[0][j] = acc[j];
+    epilogue<KIND, OUT_DT, 1, NIB>(p, out_acc, 0, n0, r16, g);
+  }
+}
+
 // Sum the split-K partials in split order and apply the epilogue; one thread per
 // run of four consecutive n.
 template <int KIND, int OUT_DT>
@@ -2218,9 +2425,10 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 }
 
 // Decode path without split-K: blocks of 16 or 32 weight rows over the whole of K (M <= 32; M <= 64 on small weights).
-template <int KIND, int OUT_DT>
-static bool launch_stream(GemmArgs& p, hipStream_t st) {
-  if (p.M > 64 || p.K < 512) return false;
+// stream_rows: weight rows per block in units of 16 (1 or 2) that this kernel takes the problem with, 0 = it does not.
+template <int KIND>
+static int stream_rows(const GemmArgs& p) {
+  if (p.M > 64 || p.K < 512) return 0;
   // Rows of weight per block (16 or 32; 0 = leave the shape to the split-K kernel), from a sweep over
   // N = 1024 ... 57344, K = 512 ... 28672 and M = 1 ... 64 with the weights rotated through more than the
   // last-level cache.  Against the split-K kernel this one saves the second launch and the partial sums,
@@ -2258,6 +2466,12 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
     if (p.N < 1024) nib = 0;
   }
   if (p.M > 32 && nib == 2) nib = 0;  // (64 activation rows are built with 16-row blocks only)
+  return nib;
+}
+
+template <int KIND, int OUT_DT>
+static bool launch_stream(GemmArgs& p, hipStream_t st) {
+  const int nib = stream_rows<KIND>(p);
   if (nib == 0) return false;
   p.splits = 1;
   p.tiles_m = 1;
@@ -2305,17 +2519,29 @@ static bool tuned_lookup(int kind, int64_t m, int64_t n, int64_t k, int& tile, i
   return false;
 }
 
-template <int KIND, int OUT_DT>
-static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+// The selection in force for this call: the calling thread's test hooks, else a tuned entry.
+static void pick_selection(int kind, const GemmArgs& p) {
   t_tile = g_force_tile;
   t_splits = g_force_splits;
   if (t_tile == 0 && t_splits == 0) {
     int tile = 0, splits = 0;
-    if (tuned_lookup(KIND, p.M, p.N, p.K, tile, splits)) {
+    if (tuned_lookup(kind, p.M, p.N, p.K, tile, splits)) {
       t_tile = tile;
       t_splits = splits;
     }
   }
+}
+
+// Whether the decode kernel without split-K takes this problem (and with how many weight rows per block).
+template <int KIND>
+static int stream_choice(const GemmArgs& p) {
+  if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (t_tile == 0 || t_tile == 16 || t_tile == 32)) return stream_rows<KIND>(p);
+  return 0;
+}
+
+template <int KIND, int OUT_DT>
+static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  pick_selection(KIND, p);
   if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (t_tile == 0 || t_tile == 16 || t_tile == 32) &&
       launch_stream<KIND, OUT_DT>(p, st))
     return;
@@ -2737,6 +2963,109 @@ extern "C" int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64
   p.ws = workspace;
   launch_kind<KIND_I8_RAW, SGLQ_BF16>(p, workspace_bytes, static_cast<hipStream_t>(stream));
   return finish(name);
+}
+
+// ---------------------------------------------------------------------------
+// Quantize-and-multiply in one call: per-token-group FP8 quantization (groups of 128) of 16-bit
+// activations followed by the block-scaled FP8 GEMM, the pair of calls of
+// cutlass_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:204-209).  For up to 8 rows on the
+// shapes that the full-K decode kernel takes, one launch does both (gemm_stream_quant_kernel);
+// otherwise the two kernels run one after the other with the codes and scales in the workspace.
+// Either way the output is bit-identical to the two operators called in turn.
+// ---------------------------------------------------------------------------
+template <int OUT_DT>
+static void launch_stream_quant(GemmArgs& p, int nib, int in_dtype, hipStream_t st) {
+  p.splits = 1;
+  p.tiles_m = 1;
+  p.tiles_n = (p.N + 16 * nib - 1) / (16 * nib);
+  const dim3 grid((uint32_t)p.tiles_n), block(256);
+  g_last_kernel = nib == 1 ? "gemm_stream_quant_kernel<16 rows>" : "gemm_stream_quant_kernel<32 rows>";
+  auto launch = [&](auto nib_tag, auto in_tag) {
+    constexpr int NIB = decltype(nib_tag)::value, IN_DT = decltype(in_tag)::value;
+    if (p.M <= 1) gemm_stream_quant_kernel<NIB, OUT_DT, IN_DT, 1><<<grid, block, 0, st>>>(p);
+    else if (p.M <= 2) gemm_stream_quant_kernel<NIB, OUT_DT, IN_DT, 2><<<grid, block, 0, st>>>(p);
+    else if (p.M <= 4) gemm_stream_quant_kernel<NIB, OUT_DT, IN_DT, 4><<<grid, block, 0, st>>>(p);
+    else gemm_stream_quant_kernel<NIB, OUT_DT, IN_DT, 8><<<grid, block, 0, st>>>(p);
+  };
+  using one = std::integral_constant<int, 1>;
+  using two = std::integral_constant<int, 2>;
+  using bf16 = std::integral_constant<int, SGLQ_BF16>;
+  using fp16 = std::integral_constant<int, SGLQ_FP16>;
+  if (in_dtype == SGLQ_BF16) {
+    if (nib == 1) launch(one{}, bf16{});
+    else launch(two{}, bf16{});
+  } else {
+    if (nib == 1) launch(one{}, fp16{});
+    else launch(two{}, fp16{});
+  }
+}
+
+extern "C" int sglq_w8a8_block_fp8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* sfb,
+                                          int64_t sfb_stride_k, int64_t sfb_stride_n, const void* bias, void* out,
+                                          int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K, float eps,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* name = "w8a8_block_fp8_linear";
+  if (in_dtype != SGLQ_BF16 && in_dtype != SGLQ_FP16 && in_dtype != SGLQ_FP32) {
+    set_error("%s: activations must be BFloat16, Half or Float", name);
+    return SGLQ_EUNSUPPORTED;
+  }
+  if (K > 0 && K % 128 != 0) {
+    set_error("%s: K (%lld) must be a multiple of the quantization group, 128", name, (long long)K);
+    return SGLQ_EINVAL;
+  }
+  // (x stands in for the codes: same row count, contiguous rows of K elements)
+  int rc = gemm_common_checks(name, x, K, b, ldb, out, ldo, M, N, K, 2);
+  if (rc < 0) return SGLQ_OK;
+  if (rc) return rc;
+  if (!sfb) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (out_dtype != SGLQ_BF16 && out_dtype != SGLQ_FP16) {
+    set_error("%s: out_dtype must be Half or BFloat16", name);
+    return SGLQ_EINVAL;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M <= 8 && in_dtype != SGLQ_FP32 && M * K * 2 < (1ll << 31)) {
+    GemmArgs p;
+    fill_common(p, x, K, b, ldb, out, ldo, M, N, K);
+    p.sb = sfb;
+    p.bias = bias;
+    p.sb_stride_k = sfb_stride_k;
+    p.sb_stride_n = sfb_stride_n;
+    pick_selection(KIND_FP8_BLOCK, p);
+    const int nib = stream_choice<KIND_FP8_BLOCK>(p);
+    // Measured against the two launches (graph-timed, weights rotated past the last-level cache, DeepSeek-V3 and
+    // Llama-70B shapes): the single kernel wins for M <= 4 where its blocks fill one to two and a half rounds of the
+    // CUs (1 x 7168 x 16384: 27.8 -> 26.3 us, 4 x 4096 x 7168: 9.0 -> 8.2 us, 4 x 8192 x 8192: 17.1 -> 15.4 us); with
+    // fewer blocks the quantization's latency is exposed (1 x 2112 x 7168: 7.5 -> 8.2 us), with many more its
+    // arithmetic, repeated by every block, costs more than the launch it saves (4 x 57344 x 8192: 83.9 -> 86.7 us),
+    // and from 5 rows on it loses nearly everywhere (8 x 4096 x 7168: 9.2 -> 10.1 us).  A forced 16- or 32-row
+    // block (test hook) takes the single kernel for any M <= 8.
+    const int blocks = nib > 0 ? (int)((N + 16 * nib - 1) / (16 * nib)) : 0;
+    const bool pays = g_force_tile != 0 || (M <= 4 && blocks >= num_cus() && 2 * blocks <= 5 * num_cus());
+    if (nib > 0 && pays) {
+      p.lda = (uint32_t)(K * 2);  // row stride of the 16-bit activations in bytes
+      p.a_bytes = (uint32_t)(M * K * 2);
+      p.quant_eps = eps;
+      if (out_dtype == SGLQ_BF16) launch_stream_quant<SGLQ_BF16>(p, nib, in_dtype, st);
+      else launch_stream_quant<SGLQ_FP16>(p, nib, in_dtype, st);
+      return finish(name);
+    }
+  }
+  // two launches: codes [M, K] and column-major scales [M, K / 128] at the head of the workspace
+  const int64_t code_bytes = (M * K + 255) / 256 * 256, scale_bytes = (M * (K / 128) * 4 + 255) / 256 * 256;
+  if (!workspace || workspace_bytes < code_bytes + scale_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15)) {
+    set_error("%s: a 16-byte aligned workspace of at least %lld bytes is needed for the quantized activations of this shape (%lld given)",
+              name, (long long)(code_bytes + scale_bytes), (long long)workspace_bytes);
+    return SGLQ_EINVAL;
+  }
+  char* ws = static_cast<char*>(workspace);
+  float* scales = reinterpret_cast<float*>(ws + code_bytes);
+  rc = sglq_per_token_group_quant_fp8(x, in_dtype, ws, scales, M, K, 128, 1, M, eps, -448.0f, 448.0f, stream);
+  if (rc) return rc;
+  return blockwise_entry<KIND_FP8_BLOCK>(name, ws, K, b, ldb, scales, 1, M, sfb, sfb_stride_k, sfb_stride_n, bias, out, ldo, out_dtype,
+                                         M, N, K, ws + code_bytes + scale_bytes, workspace_bytes - code_bytes - scale_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------

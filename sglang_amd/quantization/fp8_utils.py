@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
-from ..sgl_kernel.gemm import fp8_blockwise_scaled_mm_bias
+from ..sgl_kernel.gemm import block_fp8_linear, fp8_blockwise_scaled_mm_bias
 from .fp8_kernel import (
     per_token_group_quant_fp8,
     scaled_fp8_quant,
@@ -16,6 +16,11 @@ from .fp8_kernel import (
     static_quant_fp8,
     w8a8_block_fp8_matmul,
 )
+
+
+# Rows up to which w8a8_block_fp8_linear hands quantization and GEMM to one operator: the single
+# fused decode kernel is chosen for up to 4 rows (measured; beyond that two launches are faster).
+FUSED_QUANT_MAX_ROWS = 4
 
 
 def w8a8_block_fp8_linear(
@@ -36,6 +41,12 @@ def w8a8_block_fp8_linear(
     assert list(block_size) == [128, 128], "only 128x128 weight blocks are built"
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[0]]
+    fusable_bias = bias is None or (bias.dtype == input_2d.dtype and bias.is_contiguous() and bias.numel() == weight.shape[0])
+    if (input_2d.shape[0] <= FUSED_QUANT_MAX_ROWS and fusable_bias and input_2d.dtype in (torch.bfloat16, torch.float16)
+            and input_2d.is_contiguous() and weight.shape[1] % 128 == 0 and weight.is_contiguous()):
+        # decode-sized batches: quantization and GEMM (and bias) as one operator, a single kernel on the
+        # shapes of the decode kernel without split-K; bit-identical to the calls below
+        return block_fp8_linear(input_2d, weight.T, weight_scale.T, bias).view(*output_shape)
     q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
     if bias is not None and bias.dtype == input_2d.dtype and bias.is_contiguous() and bias.numel() == weight.shape[0]:
         # the GEMM and `output += bias` (fp8_utils.py:207-211) in one kernel, same two roundings

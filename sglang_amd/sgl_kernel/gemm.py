@@ -208,6 +208,39 @@ def fp8_blockwise_scaled_mm_bias(mat_a, mat_b, scales_a, scales_b, out_dtype, bi
     return out
 
 
+def block_fp8_linear(input_2d, mat_b, scales_b, bias=None, eps=1e-10):
+    """per_token_group_quant_fp8(input_2d, 128) followed by fp8_blockwise_scaled_mm and the caller's
+    bias add (fp8_utils.py:204-211) as one operator; for up to 8 rows on the shapes of the decode
+    kernel without split-K it is a single launch.  input_2d [M, K] contiguous, 16- or 32-bit float;
+    mat_b [K, N] column-major e4m3fn; scales_b [K/128, N/128] fp32; the output has input_2d's dtype
+    (bfloat16 or half).  Bit-identical to the operators called in turn."""
+    _check(input_2d.is_cuda and mat_b.is_cuda and scales_b.is_cuda, "tensors must be CUDA tensors")
+    _check(input_2d.dim() == 2 and input_2d.is_contiguous(), "input must be a contiguous 2D tensor")
+    _check(mat_b.dim() == 2 and mat_b.stride(0) == 1 and mat_b.dtype == FP8, "mat_b must be a column major Float8_e4m3fn tensor")
+    _check(input_2d.dtype in (torch.bfloat16, torch.float16), "input must be BFloat16 or Half (the output takes its dtype)")
+    m, k = input_2d.shape
+    n = mat_b.size(1)
+    _check(mat_b.size(0) == k, "input and mat_b shapes cannot be multiplied")
+    _check(k % 128 == 0, "K must be a multiple of the quantization group, 128")
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    _check(scales_b.dtype == torch.float32 and scales_b.dim() == 2 and scales_b.shape == (k // 128, (n + 127) // 128),
+           "scales_b must be a Float32 [K/128, ceil(N/128)] tensor")
+    out_dtype = input_2d.dtype
+    if bias is not None:
+        _check(bias.is_cuda and bias.is_contiguous() and bias.numel() == n and bias.dtype == out_dtype,
+               "bias must be a contiguous CUDA tensor of N elements in the output dtype")
+    out = torch.empty((m, n), dtype=out_dtype, device=input_2d.device)
+    if m == 0 or n == 0:
+        return out
+    rc = _lib.load().sglq_w8a8_block_fp8_linear(
+        input_2d.data_ptr(), DTYPE_CODE[input_2d.dtype], mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_b.data_ptr(), scales_b.stride(0), scales_b.stride(1), None if bias is None else bias.data_ptr(),
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, eps, *_lib.workspace(input_2d.device),
+        _lib.stream_ptr(input_2d.device))
+    _lib.check(rc, "w8a8_block_fp8_linear")
+    return out
+
+
 def _group_quant_impl(fn_name, q_dtype, input, output_q, output_s, group_size, eps, qmin, qmax):
     check_group_quant(input, output_q, output_s, group_size, q_dtype)
     if input.numel() == 0:
