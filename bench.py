@@ -7,12 +7,15 @@ DeepSeek-V3 linear shapes at a prefill chunk of M = 4096, through the public
 operator API.  Inputs are synthetic and resident in HBM before timing starts.
 
 Prints ONE JSON line: whole-step block-FP8 GEMM throughput, the roofline of the
-dominant kernel (the GEMM, timed with events on the launch stream), the
-quantization kernel's HBM figure, and a CPU baseline (the torch restatement of
-the same path, timed on a bounded row sample on the host cores).
+dominant kernel (the GEMM, timed with events on the launch stream; next to the
+published peak the MFMA pipe's measured ceiling under a register-only loop and the
+shader clock the run saw), the quantization kernel's HBM figure inside the step,
+a `configs` block with every configuration of the baseline (graph-timed per shape),
+and a CPU baseline (the torch restatement of the same path on the host cores).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
     python bench.py --sweep sweep.jsonl                # every configuration, one line per shape
+    python bench.py --ceiling                          # only the MFMA pipe's sustained rate
 """
 import argparse
 import json
@@ -72,6 +75,104 @@ def make_activation(m, k, seed, dev):
 
     g = torch.Generator(device=dev).manual_seed(seed)
     return torch.randn((m, k), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+
+class BenchKernels:
+    """ctypes binding of sglang_amd/libsglq_bench.so (csrc/bench_kernels.hip): the register-only MFMA
+    loop, the clock probe and the streaming passes.  Measurement helpers only; the operators never load it."""
+
+    VARIANTS = {0: "16x16x128 accumulate in place", 1: "16x16x128 from zero + fold FMAs (block-scaled kind)",
+                2: "32x32x64 accumulate in place", 3: "32x32x64 pairs from zero + fold FMAs"}
+
+    def __init__(self, dev):
+        import ctypes
+
+        import torch
+
+        path = ROOT / "sglang_amd" / "libsglq_bench.so"
+        if not path.exists():
+            raise RuntimeError(f"{path} is missing: build it first (python -m sglang_amd.build)")
+        c = ctypes
+        self.lib = c.CDLL(str(path))
+        self.lib.sglqb_mfma_ceiling.argtypes = [c.c_int, c.c_int, c.c_void_p, c.c_void_p, c.c_void_p, c.c_int, c.c_void_p]
+        self.lib.sglqb_clock_probe.argtypes = [c.c_void_p, c.c_int, c.c_void_p]
+        self.lib.sglqb_stream.argtypes = [c.c_int, c.c_void_p, c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_void_p]
+        self.dev = dev
+        self.cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        self.torch = torch
+
+    def _stream(self):
+        return self.torch.cuda.current_stream(self.dev).cuda_stream
+
+    def clock_sample(self):
+        """(shader cycles, 100 MHz ticks) per XCD at this point of the current stream, as a device tensor [16, 2]."""
+        out = self.torch.zeros((16, 2), dtype=self.torch.int64, device=self.dev)
+        rc = self.lib.sglqb_clock_probe(out.data_ptr(), 8 * self.cus, self._stream())
+        assert rc == 0, rc
+        return out
+
+    @staticmethod
+    def clock_mhz(before, after):
+        """Average shader clock between two samples: shader cycles per tick of the 100 MHz reference counter,
+        averaged over the XCDs that reported both times."""
+        b, a = before.cpu().double(), after.cpu().double()
+        ok = (b[:, 1] > 0) & (a[:, 1] > b[:, 1])
+        if not bool(ok.any()):
+            return 0.0
+        return float((((a[:, 0] - b[:, 0]) / (a[:, 1] - b[:, 1]))[ok]).mean() * 100.0)
+
+    def operands(self, kind="random"):
+        torch = self.torch
+        g = torch.Generator(device=self.dev).manual_seed(1)
+        if kind == "random":  # N(0,1) rounded to e4m3: what quantized activations and weights look like
+            t = torch.randn(96 * 1024, generator=g, device=self.dev).to(torch.float8_e4m3fn)
+        else:                 # 0, 1, 2: few bits toggle
+            t = torch.randint(0, 3, (96 * 1024,), generator=g, device=self.dev).float().to(torch.float8_e4m3fn)
+        return t.view(torch.uint8)
+
+    def mfma_ceiling(self, variant, operands, iters=20000):
+        """PFLOP/s and shader clock of the register-only MFMA loop: 8 waves per CU, one block per CU."""
+        torch = self.torch
+        sink = torch.empty(self.cus * 512, dtype=torch.float32, device=self.dev)
+        clocks = torch.zeros(self.cus * 2, dtype=torch.int64, device=self.dev)
+        run = lambda: self.lib.sglqb_mfma_ceiling(variant, iters, operands.data_ptr(), sink.data_ptr(), clocks.data_ptr(),
+                                                  self.cus, self._stream())
+        for _ in range(2):
+            assert run() == 0
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        assert run() == 0
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e)
+        c = clocks.cpu().view(self.cus, 2).double()
+        flops = 2097152.0 * 8 * self.cus * iters
+        mhz = float((c[:, 0] / c[:, 1]).mean() * 100.0)
+        tflops = flops / ms / 1e9
+        # MFMA-pipe utilisation at that clock: 4 SIMDs x 65536 flop per 32 cycles = 8192 flop per CU and cycle
+        util = tflops * 1e12 / (self.cus * 8192.0 * mhz * 1e6)
+        return {"variant": self.VARIANTS[variant], "TFLOPs": round(tflops, 1), "clock_mhz": round(mhz, 0),
+                "mfma_pipe_utilisation": round(util, 3), "ms": round(ms, 2)}
+
+
+def run_ceiling(args):
+    """bench.py --ceiling: the MFMA pipe's sustained rate under a register-only loop (no memory traffic), for the
+    instruction mixes of the two GEMM families and two kinds of operand bytes.  One JSON line."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    bk = BenchKernels(dev)
+    out = {"what": "register-only MFMA loop, 8 waves per CU, 20000 K steps of a 128 x 64 wave tile per wave",
+           "published_peak_TFLOPs": PEAK_FP8_TFLOPS, "cus": bk.cus, "runs": []}
+    for kind in ("random", "small_integers"):
+        ops = bk.operands(kind)
+        for v in range(4):
+            r = bk.mfma_ceiling(v, ops)
+            r["operands"] = kind
+            r["frac_of_published_peak"] = round(r["TFLOPs"] / PEAK_FP8_TFLOPS, 3)
+            out["runs"].append(r)
+    print(json.dumps(out), flush=True)
 
 
 class Timer:
@@ -177,11 +278,17 @@ def run_headline(args):
         step()
     torch.cuda.synchronize()
     wall_graph = None
+    bk = BenchKernels(dev)
+    clk0 = bk.clock_sample()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    clk1 = bk.clock_sample()
+    torch.cuda.synchronize()
+    step_clock_mhz = bk.clock_mhz(clk0, clk1)
     if args.graph:
         # the same K steps replayed as one HIP graph, for comparison (measured: no faster than the launches above)
         graph = torch.cuda.CUDAGraph()
@@ -226,8 +333,23 @@ def run_headline(args):
     torch.cuda.synchronize()
     quant_big_gbs = round(group_quant_bytes(m, layers[big][1]) / (iso.total_ms() / iso.count()) / 1e6, 1)
     del xs_iso
-    # the dominant kernel: the GEMM launch that takes the largest share of the step
+    # the clock while the dominant GEMM launch alone repeats (settled), and the MFMA pipe's ceiling right after
     dom = max(range(len(layers)), key=lambda i: tg[i].total_ms())
+    n_d, k_d, x_d, wq_d, ws_d = layers[dom]
+    xq_d, xs_d = sglang_per_token_group_quant_fp8(x_d, 128, column_major_scales=True)
+    for _ in range(20):
+        fp8_blockwise_scaled_mm(xq_d, wq_d.t(), xs_d, ws_d.t(), torch.bfloat16)
+    c0 = bk.clock_sample()
+    for _ in range(20):
+        fp8_blockwise_scaled_mm(xq_d, wq_d.t(), xs_d, ws_d.t(), torch.bfloat16)
+    c1 = bk.clock_sample()
+    torch.cuda.synchronize()
+    dom_clock_mhz = bk.clock_mhz(c0, c1)
+    ops_rand = bk.operands("random")
+    ceil_fold = bk.mfma_ceiling(1, ops_rand, iters=10000)
+    ceil_acc = bk.mfma_ceiling(0, ops_rand, iters=10000)
+    # the dominant kernel: the GEMM launch that takes the largest share of the step
+    props = torch.cuda.get_device_properties(dev)
     dom_n, dom_k = layers[dom][0], layers[dom][1]
     dom_ms = tg[dom].total_ms() / tg[dom].count()
     dom_flops = 2.0 * m * dom_n * dom_k
@@ -240,7 +362,6 @@ def run_headline(args):
         traffic_all = tj.get("gemm_hbm_bytes_per_launch_avg")
     gemm_tflops = flops_step / (gemm_ms * 1e-3) / 1e12
     quant_gbs = qbytes_step / (quant_ms * 1e-3) / 1e9
-    props = torch.cuda.get_device_properties(dev)
 
     out = {
         "metric": "block-FP8 GEMM TFLOPS (% of FP8 MFMA peak); quant kernel GB/s (% of HBM)",
@@ -270,6 +391,20 @@ def run_headline(args):
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(dom_tflops / PEAK_FP8_TFLOPS, 4),
+            "practical_peak": {
+                "value": ceil_fold["TFLOPs"],
+                "unit": "TFLOP/s",
+                "what": "register-only loop of this kernel's MFMA mix (v_mfma_f32_16x16x128_f8f6f4 from a zero accumulator + 4 fold "
+                        "FMAs, 8 waves per CU) on N(0,1) e4m3 operands, no memory traffic, measured in this run: what the matrix "
+                        "pipe sustains at the clock the chip settles to under that load",
+                "clock_mhz": ceil_fold["clock_mhz"],
+                "mfma_pipe_utilisation": ceil_fold["mfma_pipe_utilisation"],
+                "frac_of_it": round(dom_tflops / ceil_fold["TFLOPs"], 4),
+                "accumulate_in_place_TFLOPs": ceil_acc["TFLOPs"],
+                "accumulate_in_place_clock_mhz": ceil_acc["clock_mhz"],
+            },
+            "clock_mhz": round(dom_clock_mhz, 0),
+            "mfma_pipe_utilisation": round(dom_tflops * 1e12 / (props.multi_processor_count * 8192.0 * max(dom_clock_mhz, 1.0) * 1e6), 3),
             "traffic": traffic,
             "avg_launch_ms": round(dom_ms, 4),
             "flops_per_launch": dom_flops,
@@ -285,20 +420,29 @@ def run_headline(args):
             "kernel": "sgl_per_token_group_quant_fp8 (group_quant_kernel)",
             "bound": "hbm",
             "launch": f"A[4096,{layers[big][1]}] bf16 -> e4m3fn + fp32 scales (largest of the step)",
-            "achieved": quant_big_gbs,
+            "achieved": quant_in_step_gbs,
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
-            "frac": round(quant_big_gbs / PEAK_HBM_GBS, 4),
+            "frac": round(quant_in_step_gbs / PEAK_HBM_GBS, 4),
             "bytes_per_launch": group_quant_bytes(m, layers[big][1]),
-            "measured": "10 back-to-back launches on 2 alternating inputs, events on the launch stream",
-            "same_launch_inside_the_step_GBs": quant_in_step_gbs,
+            "measured": "inside the timed step (right after the preceding GEMM, whose output write-back shares HBM with it), "
+                        "events on the launch stream",
+            "same_launch_isolated_GBs": quant_big_gbs,
+            "same_launch_isolated_frac": round(quant_big_gbs / PEAK_HBM_GBS, 4),
+            "isolated_measured": "10 back-to-back launches on 2 alternating inputs",
             "all_launches_inside_the_step_GBs": round(quant_gbs, 1),
+            "all_launches_inside_the_step_frac": round(quant_gbs / PEAK_HBM_GBS, 4),
         },
         "graph_ms_per_step": None if wall_graph is None else round(wall_graph * 1e3 / args.steps, 4),
         "per_shape": per_shape,
         "device": {"name": props.name, "cus": props.multi_processor_count,
-                   "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
+                   "clock_mhz": round(step_clock_mhz, 0),
+                   "clock_is": "average shader clock over the timed steps: shader-cycle counter against the 100 MHz reference "
+                               "counter, sampled per XCD on the launch stream before and after them",
+                   "nominal_clock_mhz": getattr(props, "clock_rate", 0) // 1000},
     }
+    if not args.no_configs:
+        out["configs"] = config_summary(args)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_rows)
     print(json.dumps(out), flush=True)
@@ -338,7 +482,37 @@ def time_kernel(fn, iters, rotate=1):
     return best
 
 
-def run_sweep(args):
+def config_summary(args):
+    """Every configuration of the baseline, graph-timed as --sweep does, condensed for the one JSON line:
+    per (config, shape) the quantization and GEMM device times and the fraction of the roofline that bounds
+    the GEMM there (HBM for the decode-sized M, MFMA for the prefill-sized ones)."""
+    rows = []
+    run_sweep(args, collect=rows, cfg2_ms=(64, 8192), only={"0", "1", "2", "3", "4"})
+    out = {}
+    for r in rows:
+        cfg = f"cfg{r['cfg']}"
+        if r.get("op") == "total":
+            out.setdefault(cfg, {}).setdefault("totals", []).append({"M": r["M"], "total_us": r["total_us"], "TFLOPs": r["TFLOPs"],
+                                                                      "frac_mfma": round(r["TFLOPs"] / PEAK_FP8_TFLOPS, 4)})
+            continue
+        m = r["M"]
+        hbm_bound = m <= 128
+        e = {"M": m, "N": r["N"], "K": r["K"], "quant_us": r["quant_us"], "gemm_us": r["gemm_us"],
+             "bound": "hbm" if hbm_bound else "mfma",
+             "frac": r["gemm_frac_hbm"] if hbm_bound else r["gemm_frac_mfma"]}
+        e["rate"] = f"{r['gemm_GBs']} GB/s" if hbm_bound else f"{r.get('gemm_TFLOPs', r.get('gemm_TOPs'))} T(FL)OP/s"
+        if "quant_GBs" in r:
+            e["quant_frac_hbm"] = round(r["quant_GBs"] / PEAK_HBM_GBS, 4)
+        out.setdefault(cfg, {}).setdefault("shapes", []).append(e)
+    for cfg, d in out.items():
+        sh = d.get("shapes", [])
+        if sh:
+            d["linear_us_sum"] = round(sum(x["quant_us"] + x["gemm_us"] for x in sh), 1)
+    out["timing"] = "device time per call from a HIP graph of 20 calls, inputs and weights rotated past the last-level cache"
+    return out
+
+
+def run_sweep(args, collect=None, cfg2_ms=None, only=None):
     import torch
 
     from sglang_amd import _lib
@@ -355,11 +529,16 @@ def run_sweep(args):
         torch.mm(spin, spin)
         torch.cuda.synchronize()
     del spin
-    out_path = Path(args.sweep)
-    out_path.parent.mkdir(parents=True, exist_ok=True)
-    f = open(out_path, "w")
+    f = None
+    if collect is None:
+        out_path = Path(args.sweep)
+        out_path.parent.mkdir(parents=True, exist_ok=True)
+        f = open(out_path, "w")
 
     def emit(**kw):
+        if collect is not None:
+            collect.append(kw)
+            return
         f.write(json.dumps(kw) + "\n")
         f.flush()
         print(json.dumps(kw), flush=True)
@@ -386,7 +565,8 @@ def run_sweep(args):
              gemm_frac_hbm=round(block_gemm_bytes(m, n, k) / tg / 1e6 / PEAK_HBM_GBS, 4))
         return tq, tg
 
-    only = None if not args.sweep_only else set(args.sweep_only.split(","))
+    if only is None:
+        only = None if not args.sweep_only else set(args.sweep_only.split(","))
 
     def want(cfg):
         return only is None or str(cfg) in only
@@ -415,7 +595,7 @@ def run_sweep(args):
     del w8s
     # cfg 2
     for i, (n, k) in enumerate(DSV3_NK if want(2) else ()):
-        for m in (1, 8, 64, 512, 4096, 8192):
+        for m in cfg2_ms or (1, 8, 64, 512, 4096, 8192):
             block_case(2, "dsv3", m, n, k, 2000 + i)
     # cfg 3
     for i, (n, k) in enumerate(LLAMA8B_NK if want(3) else ()):
@@ -540,7 +720,8 @@ def run_sweep(args):
                  layer_us=round(layer * 1e3, 1), layer_TFLOPs=round(fl / layer / 1e9, 2),
                  steps_us={s: round(v * 1e3, 1) for s, v in t.items()}, steps_sum_us=round(sum(v for s, v in t.items() if s not in SEPARATE) * 1e3, 1),
                  steps_GBs={s: round(b / t[s] / 1e6, 1) for s, b in moved.items()})
-    f.close()
+    if f is not None:
+        f.close()
 
 
 def main():
@@ -552,6 +733,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (reference point for the rocprofv3 byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the `configs` block (every baseline configuration, graph-timed)")
+    ap.add_argument("--ceiling", action="store_true", help="only measure the MFMA pipe's sustained rate (register-only loop) and exit")
     ap.add_argument("--graph", action="store_true", help="also time the K steps replayed as one HIP graph (graph_ms_per_step)")
     ap.add_argument("--prewarm-ms", type=float, default=150.0, help="untimed steps for this long before the warm-up steps")
     ap.add_argument("--sweep", type=str, default=None, help="write per-shape lines for every configuration to this file")
@@ -564,7 +747,9 @@ def main():
               "a tensor-parallel deployment shards N or K per rank and all-reduces outside it). Run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
-    if args.sweep:
+    if args.ceiling:
+        run_ceiling(args)
+    elif args.sweep:
         run_sweep(args)
     else:
         run_headline(args)
