@@ -105,21 +105,22 @@ class BenchKernels:
         return self.torch.cuda.current_stream(self.dev).cuda_stream
 
     def clock_sample(self):
-        """(shader cycles, 100 MHz ticks) per XCD at this point of the current stream, as a device tensor [16, 2]."""
-        out = self.torch.zeros((16, 2), dtype=self.torch.int64, device=self.dev)
-        rc = self.lib.sglqb_clock_probe(out.data_ptr(), 8 * self.cus, self._stream())
+        """(shader cycles, 100 MHz ticks) per compute unit at this point of the current stream, as a device
+        tensor [4096, 2] (slots of CUs that no block of the probe landed on stay zero)."""
+        out = self.torch.zeros((4096, 2), dtype=self.torch.int64, device=self.dev)
+        rc = self.lib.sglqb_clock_probe(out.data_ptr(), 32 * self.cus, self._stream())
         assert rc == 0, rc
         return out
 
     @staticmethod
     def clock_mhz(before, after):
         """Average shader clock between two samples: shader cycles per tick of the 100 MHz reference counter,
-        averaged over the XCDs that reported both times."""
+        the median over the compute units that reported both times."""
         b, a = before.cpu().double(), after.cpu().double()
         ok = (b[:, 1] > 0) & (a[:, 1] > b[:, 1])
         if not bool(ok.any()):
             return 0.0
-        return float((((a[:, 0] - b[:, 0]) / (a[:, 1] - b[:, 1]))[ok]).mean() * 100.0)
+        return float((((a[:, 0] - b[:, 0]) / (a[:, 1] - b[:, 1]))[ok]).median() * 100.0)
 
     def operands(self, kind="random"):
         torch = self.torch
@@ -154,6 +155,56 @@ class BenchKernels:
         util = tflops * 1e12 / (self.cus * 8192.0 * mhz * 1e6)
         return {"variant": self.VARIANTS[variant], "TFLOPs": round(tflops, 1), "clock_mhz": round(mhz, 0),
                 "mfma_pipe_utilisation": round(util, 3), "ms": round(ms, 2)}
+
+
+def calibrate_copy(dev):
+    """One plain copy kernel of known size (stream_kernel<0> of libsglq_bench.so: reads 256 MiB, writes 256 MiB),
+    the yardstick for what the profiler's FETCH_SIZE / WRITE_SIZE counters report per byte."""
+    import torch
+
+    bk = BenchKernels(dev)
+    src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(8 * bk.cus, dtype=torch.int32, device=dev)
+    rc = bk.lib.sglqb_stream(0, src.data_ptr(), dst.data_ptr(), src.numel(), sink.data_ptr(), 8 * bk.cus, bk._stream())
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+
+
+def run_launches(args):
+    """bench.py --launches "M,N,K;M,N,K;...": each listed block-FP8 linear (group quantization, then the GEMM) as
+    plain launches, `--launch-reps` times each after one untimed call, in the order given: the program to put under
+    `rocprofv3 --pmc ...`, whose per-dispatch rows then map to the shapes by order.  Prints one JSON line with
+    the kernel each shape selected and its event-timed duration."""
+    import torch
+
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        calibrate_copy(dev)
+    rows = []
+    for i, spec in enumerate(args.launches.split(";")):
+        m, n, k = (int(v) for v in spec.split(","))
+        wq, ws = make_block_weight(n, k, 7000 + i, dev)
+        x = make_activation(m, k, 7100 + i, dev)
+        xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+        fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+        torch.cuda.synchronize()
+        t = Timer()
+        for _ in range(args.launch_reps):
+            xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+            t.time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+        torch.cuda.synchronize()
+        us = t.total_ms() / t.count() * 1e3
+        rows.append({"M": m, "N": n, "K": k, "kernel": lib.sglq_debug_last_gemm_kernel().decode(), "gemm_us": round(us, 2),
+                     "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "GBs": round(block_gemm_bytes(m, n, k) / us / 1e3, 1),
+                     "algorithmic_bytes": block_gemm_bytes(m, n, k)})
+        del wq, x, xq
+    print(json.dumps({"launches": rows, "reps": args.launch_reps}), flush=True)
 
 
 def run_ceiling(args):
@@ -259,11 +310,7 @@ def run_headline(args):
                 kernel_of[li] = _lib.load().sglq_debug_last_gemm_kernel().decode()
 
     if args.calibrate_copy:
-        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        torch.add(src, 1.0, out=dst)  # a plain elementwise kernel: reads 256 MiB, writes 256 MiB
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(dev)
 
     # The chip needs about 60 steps (60 ms) of this load before its step time settles (962 us per step over
     # steps 10-20, 933 over 20-30, 890-900 from step 60 on; measured): run untimed steps for 150 ms first, so
@@ -438,7 +485,7 @@ def run_headline(args):
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": round(step_clock_mhz, 0),
                    "clock_is": "average shader clock over the timed steps: shader-cycle counter against the 100 MHz reference "
-                               "counter, sampled per XCD on the launch stream before and after them",
+                               "counter, sampled per compute unit on the launch stream before and after them (median over the CUs)",
                    "nominal_clock_mhz": getattr(props, "clock_rate", 0) // 1000},
     }
     if not args.no_configs:
@@ -731,9 +778,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-rows", type=int, default=4096, help="activation rows in the CPU-baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 256 MiB device copy (reference point for the rocprofv3 byte counters)")
+                    help="also run one plain 256 MiB copy kernel first (reference point for the rocprofv3 byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-configs", action="store_true", help="skip the `configs` block (every baseline configuration, graph-timed)")
+    ap.add_argument("--launches", type=str, default=None,
+                    help='"M,N,K;M,N,K;...": run these block-FP8 linears as plain launches in this order and exit (for profiler counter runs)')
+    ap.add_argument("--launch-reps", type=int, default=5)
     ap.add_argument("--ceiling", action="store_true", help="only measure the MFMA pipe's sustained rate (register-only loop) and exit")
     ap.add_argument("--graph", action="store_true", help="also time the K steps replayed as one HIP graph (graph_ms_per_step)")
     ap.add_argument("--prewarm-ms", type=float, default=150.0, help="untimed steps for this long before the warm-up steps")
@@ -747,7 +797,9 @@ def main():
               "a tensor-parallel deployment shards N or K per rank and all-reduces outside it). Run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
-    if args.ceiling:
+    if args.launches:
+        run_launches(args)
+    elif args.ceiling:
         run_ceiling(args)
     elif args.sweep:
         run_sweep(args)

@@ -1,7 +1,7 @@
 // Measurement kernels for gfx950 (built into libsglq_bench.so, not into the operator library):
 //   * a register-only MFMA loop, the ceiling that the matrix pipe sustains on real operand
 //     bytes at the clock the chip settles to under that load,
-//   * a clock probe (shader-clock and constant-rate counters per XCD), from which a harness
+//   * a clock probe (shader-clock and constant-rate counters per compute unit), from which a harness
 //     derives the average shader clock over a timed region,
 //   * a plain copy and a read-only / write-only pass of known size, the yardsticks for the
 //     FETCH_SIZE / WRITE_SIZE profiler counters and for the memory system's streaming rate.
@@ -145,15 +145,19 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(const v8i* __restrict
   }
 }
 
-// One sample of both counters per XCD: slot = the XCC id of the CU the block runs on.
-// Blocks on the same XCD write nearly identical values; the last writer stays.
+// One sample of both counters per compute unit: slot = (XCC id, shader engine, shader array, CU) of the
+// CU the block runs on (4096 slots).  The shader-cycle counters of different CUs are not aligned with each
+// other, so only differences between two samples of the same slot mean anything.  Blocks on the same CU write
+// nearly identical values; the last writer stays.
 __global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t* __restrict__ out) {
   if (threadIdx.x != 0) return;
   const ClockSample s = read_clocks();
-  // HW_REG_XCC_ID (hardware register 20), bits 3:0
+  // HW_REG_XCC_ID (hardware register 20) bits 3:0; HW_REG_HW_ID (register 4): CU id bits 11:8, SH id bit 12, SE id bits 15:13
   const uint32_t xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & 15u;
-  out[2 * xcc] = s.shader_cycles;
-  out[2 * xcc + 1] = s.realtime_ticks;
+  const uint32_t cu = __builtin_amdgcn_s_getreg(4 | (8 << 6) | ((8 - 1) << 11)) & 255u;
+  const uint32_t slot = (xcc << 8) | cu;
+  out[2 * slot] = s.shader_cycles;
+  out[2 * slot + 1] = s.realtime_ticks;
 }
 
 // mode 0: dst = src; 1: read src only (one value per block written at the end); 2: write dst only
@@ -195,7 +199,7 @@ int sglqb_mfma_ceiling(int variant, int iters, const void* operands, float* sink
   return (int)hipGetLastError();
 }
 
-// out: 16 x 2 uint64 (per XCC id: shader cycles, constant-rate ticks), zero-filled by the caller.
+// out: 4096 x 2 uint64 (per CU slot: shader cycles, constant-rate ticks), zero-filled by the caller.
 int sglqb_clock_probe(uint64_t* out, int blocks, void* stream) {
   if (!out || blocks <= 0) return -1;
   clock_probe_kernel<<<blocks, 64, 0, static_cast<hipStream_t>(stream)>>>(out);

@@ -71,6 +71,11 @@ constexpr int PLAN_HEADER = 4, PLAN_ENTRY = 4;
 // and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
 constexpr int waitcnt_vm_lgkm0(int vm) { return (vm & 0xf) | (((vm >> 4) & 3) << 14) | (7 << 4); }
 // ... and one that waits for LDS / scalar-memory operations only
+// Tile rows per band of the tile walk (tile_of_block).  8 was measured against 4 and 16 with the
+// profiler's FETCH_SIZE counter on the 256-row kernels: see tile_of_block.
+#ifndef SGLQ_GROUP_M
+#define SGLQ_GROUP_M 8
+#endif
 #ifndef SGLQ_STREAM_NSTAGE
 #define SGLQ_STREAM_NSTAGE 3
 #endif
@@ -163,7 +168,7 @@ SGLQ_DEV void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn)
   const int q = total >> 3, rem = total & 7;
   const int xcd = pid & 7, idx = pid >> 3;
   int tile = xcd * q + (xcd < rem ? xcd : rem) + idx;
-  constexpr int GROUP_M = 8;
+  constexpr int GROUP_M = SGLQ_GROUP_M;
   const int width = GROUP_M * tiles_n;
   const int group = tile / width;
   const int first_m = group * GROUP_M;
