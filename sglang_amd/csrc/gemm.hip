@@ -71,10 +71,14 @@ constexpr int PLAN_HEADER = 4, PLAN_ENTRY = 4;
 // and all LDS / scalar-memory operations are done (vmcnt is split over bits 3:0 and 15:14).
 constexpr int waitcnt_vm_lgkm0(int vm) { return (vm & 0xf) | (((vm >> 4) & 3) << 14) | (7 << 4); }
 // ... and one that waits for LDS / scalar-memory operations only
-// Tile rows per band of the tile walk (tile_of_block).  8 was measured against 4 and 16 with the
-// profiler's FETCH_SIZE counter on the 256-row kernels: see tile_of_block.
+// Tile rows per band of the tile walk (tile_of_block).  Measured with the profiler's FETCH_SIZE counter (bytes
+// that miss the XCDs' L2s) on the 256-row kernels at M = 4096: bands of 4 rows fetch 6 % less than bands of 8
+// on 7168 x 16384 (224-wide tiles) and 20 % less on 2112 x 7168 (192-wide tiles), the same on 24576 x 1536 and
+// 4096 x 7168 (with 32 tiles in flight per XCD, 4 x 8 and 8 x 4 touch the same number of rows when the tile is
+// square); bands of 16 fetch 40-70 % more.  Launch times move by less than 2 % between 4 and 8 and by +2-3 %
+// with 16: these kernels are not bound by that traffic.
 #ifndef SGLQ_GROUP_M
-#define SGLQ_GROUP_M 8
+#define SGLQ_GROUP_M 4
 #endif
 #ifndef SGLQ_STREAM_NSTAGE
 #define SGLQ_STREAM_NSTAGE 3
@@ -2442,7 +2446,7 @@ static int stream_rows(const GemmArgs& p) {
   // more than 16 rows on large N, where this kernel's per-wave activation copies weigh more.
   int nib = 0;
   if (t_tile == 16) nib = 1;
-  else if (t_tile == 32) nib = p.M <= 32 ? 2 : 0;
+  else if (t_tile == 32) nib = 2;
   else if (t_tile == 0) {
     // 32-row blocks move half the activation bytes per weight byte; they lose where they leave half of the
     // CUs idle (N <= 4096) or their last round is less than half full (N = 10240: 320 blocks on 256 CUs)
@@ -2466,11 +2470,14 @@ static int stream_rows(const GemmArgs& p) {
       // enough blocks (64 x 4096 x 7168: 14.1 -> 10.3 us, 64 x 4096 x 4096: 14.8 -> 8.3 us; but
       // 64 x 8192 x 8192: 22 -> 27 us and 64 x 13824 x 2048: 14.4 -> 15.8 us)
       nib = ((int64_t)p.N * p.K <= (30 << 20) && p.N <= 10240) ? 1 : 0;
+      // ... and with 32-row blocks where those fill exactly one round of the CUs (half the activation bytes per
+      // weight byte of the 16-row blocks; 64 x 8192 x 8192: 21.3 us on the split-K kernel, 20.4 us here,
+      // 33 x 8192 x 8192: 20.2 -> 18.5 us; with 224 blocks, 64 x 7168 x 16384, it loses: 32.7 -> 34.2 us)
+      if (nib == 0 && p.K >= 8192 && blocks32 <= num_cus() && 16 * blocks32 > 15 * num_cus()) nib = 2;
     }
     if (nib == 2 && p.N < 2048) nib = 1;
     if (p.N < 1024) nib = 0;
   }
-  if (p.M > 32 && nib == 2) nib = 0;  // (64 activation rows are built with 16-row blocks only)
   return nib;
 }
 
@@ -2490,7 +2497,8 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
     if (nib == 1) gemm_stream_kernel<KIND, 2, 1, OUT_DT><<<grid, block, 0, st>>>(p);
     else gemm_stream_kernel<KIND, 2, 2, OUT_DT><<<grid, block, 0, st>>>(p);
   } else {
-    gemm_stream_kernel<KIND, 4, 1, OUT_DT><<<grid, block, 0, st>>>(p);
+    if (nib == 1) gemm_stream_kernel<KIND, 4, 1, OUT_DT><<<grid, block, 0, st>>>(p);
+    else gemm_stream_kernel<KIND, 4, 2, OUT_DT><<<grid, block, 0, st>>>(p);
   }
   return true;
 }
