@@ -1378,19 +1378,34 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   // One K step: block u sits in stage `cur`, its activation fragments and first weight
   // fragment are in af / b_cur.  kn: index, inside its tile, of block u + 1 (the copies
   // deferred to a tile's first step); kn2: that of block u + 2 (off_a2 / off_b2).
-  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
+  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag, auto jsw_tag) __attribute__((always_inline)) {
     constexpr bool first = decltype(first_tag)::value;
     constexpr bool last = decltype(last_tag)::value;
+    // Fragments j < JSW of this wave lie in the tile's scale block sb_lo, the others in sb_lo + 1.  JSW is a
+    // compile-time constant here (the tile loop below dispatches on it once per tile): the scale of fragment
+    // (i, j), sfa[i] * sfb of j's block, then takes 8 multiplies per K step and no selects instead of one
+    // multiply and one select per MFMA.  The VALU port also issues the MFMAs and the folds and is the scarce
+    // resource of this loop: with 28 multiplies and 8 selects fewer per step the launch is 5 % shorter.
+    constexpr int JSW = decltype(jsw_tag)::value;
     const char* st = smem + cur * STAGE_BYTES;
     const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
+    float scv[MI] = {0.f, 0.f, 0.f, 0.f};  // sfa[i] * sfb of the scale block of the fragments being multiplied
+    if constexpr (BLOCK) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) scv[i] = sfa_cur[i] * sfb_lo;
+    }
     v4f part_prev = {0.f, 0.f, 0.f, 0.f};
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       v8i b_nxt = b_cur;
-      float sfb_j = 0.f;
-      if constexpr (BLOCK) sfb_j = j < jsw ? sfb_lo : sfb_hi;  // wave-uniform
+      if constexpr (BLOCK) {
+        if (j == JSW) {  // (compile-time: no branch) the fragments from here on lie in the next scale block
+#pragma unroll
+          for (int i = 0; i < MI; ++i) scv[i] = sfa_cur[i] * sfb_hi;
+        }
+      }
       if (j == 1 && !last) {
         // barrier 1: MFMAs 0..3 have consumed this wave's activation fragments, so its LDS
         // reads of block u's activations are complete; behind the barrier that holds for
@@ -1431,7 +1446,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         }
         if constexpr (BLOCK) {
           sc_prev = sc;
-          sc = sfa_cur[i] * sfb_j;
+          sc = scv[i];
         }
         if (j + 1 < NI) {
           if (i == 0) b_nxt = read_frag(st + b_base + (j + 1) * 16 * 128);
@@ -1529,19 +1544,41 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
     uint32_t sc_voff_next = OOB;
     if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
-    k_step(par, 1, 2, std::true_type{}, std::false_type{});
-    for (int kb = 1; kb + 1 < nkb; ++kb) {
-      const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
-      off_a2 = pen ? off_a_next : off_a2;
-      off_b2 = pen ? off_b_next : off_b2;
-      sc_voff2 = pen ? sc_voff_next : sc_voff2;
-      k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{});
-    }
-    // last K block: the scales read behind its last MFMAs are the next tile's; its copies (the
-    // next tile's second block) wait for the next tile's first step
     const int last_stage = (nkb - 1 + par) & 1;
-    if constexpr (BLOCK) set_scale_split(nn0);
-    k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
+    // the tile's K steps, instantiated for the position of the scale-block boundary among this wave's fragments
+    auto tile_steps = [&](auto jsw_tag) __attribute__((always_inline)) {
+      k_step(par, 1, 2, std::true_type{}, std::false_type{}, jsw_tag);
+      for (int kb = 1; kb + 1 < nkb; ++kb) {
+        const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
+        off_a2 = pen ? off_a_next : off_a2;
+        off_b2 = pen ? off_b_next : off_b2;
+        sc_voff2 = pen ? sc_voff_next : sc_voff2;
+        k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{}, jsw_tag);
+      }
+      // last K block: the scales read behind its last MFMAs are the next tile's; its copies (the
+      // next tile's second block) wait for the next tile's first step
+      if constexpr (BLOCK) set_scale_split(nn0);
+      k_step(last_stage, 0, 0, std::false_type{}, std::true_type{}, jsw_tag);
+    };
+    if constexpr (!BLOCK || NI == 8) {
+      tile_steps(std::integral_constant<int, NI>{});  // (256-wide tiles: a wave's 128 columns are one scale block)
+    } else if constexpr (NI == 6) {
+      // 192-wide tiles start at multiples of 64 columns: the boundary is behind fragment 2, 4 or 6 (= none)
+      if (jsw == 2) tile_steps(std::integral_constant<int, 2>{});
+      else if (jsw == 4) tile_steps(std::integral_constant<int, 4>{});
+      else tile_steps(std::integral_constant<int, 6>{});
+    } else {
+      // 224-wide tiles start at multiples of 32 columns, their second wave 112 columns later: any position
+      switch (jsw) {
+        case 1: tile_steps(std::integral_constant<int, 1>{}); break;
+        case 2: tile_steps(std::integral_constant<int, 2>{}); break;
+        case 3: tile_steps(std::integral_constant<int, 3>{}); break;
+        case 4: tile_steps(std::integral_constant<int, 4>{}); break;
+        case 5: tile_steps(std::integral_constant<int, 5>{}); break;
+        case 6: tile_steps(std::integral_constant<int, 6>{}); break;
+        default: tile_steps(std::integral_constant<int, 7>{}); break;
+      }
+    }
     off_a = off_a2;
     off_b = off_b2;
     sc_voff = sc_voff2;
