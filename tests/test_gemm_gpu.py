@@ -658,3 +658,40 @@ def test_shipped_tuned_tables_give_oracle_results(gpu):
                 ref = O.fp8_blockwise_scaled_mm(a[:rows].cpu(), w[cols].cpu().t(), sa[:rows].cpu().contiguous(),
                                                 ws[nb].cpu().t()[:, : 2], torch.float32, acc_dtype=torch.float64)
             torch.testing.assert_close(out[:rows, cols].cpu().float(), ref, rtol=RTOL, atol=ATOL)
+
+
+BASELINE_KERNELS = [
+    # (M, N, K) of the headline step and the kernel the profile summaries under profiles/ name for it
+    ((4096, 24576, 1536), "gemm_pipe_kernel"),
+    ((4096, 32768, 512), "gemm_pipe_kernel"),
+    ((4096, 7168, 16384), "gemm_wide_kernel<7>"),
+    ((4096, 4096, 7168), "gemm_pipe_kernel"),
+    ((4096, 2112, 7168), "gemm_wide_kernel<6>"),
+    # decode launches of the same shapes
+    ((1, 7168, 16384), "gemm_stream_kernel<16 rows>"),
+    ((8, 7168, 16384), "gemm_stream_kernel<16 rows>"),
+    ((64, 7168, 16384), "gemm_skinny_kernel+splitk_reduce_kernel"),
+    ((1, 4096, 7168), "gemm_stream_kernel<16 rows>"),
+    ((64, 4096, 7168), "gemm_stream_kernel<16 rows>"),
+    ((1, 24576, 1536), "gemm_skinny_kernel"),
+    ((64, 24576, 1536), "gemm_skinny_kernel"),
+]
+
+
+@pytest.mark.parametrize("mnk,kernel", BASELINE_KERNELS)
+def test_baseline_shapes_select_the_profiled_kernels(gpu, mnk, kernel):
+    """The kernel selection is a set of measured rules and tuned tables; the profile summaries and the
+    design notes name the kernel that serves each headline shape.  An edit of the rules that moves one of
+    them must show up here (and in those summaries)."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    m, n, k = mnk
+    lib = _lib.load()
+    g = torch.Generator(device=gpu).manual_seed(5)
+    a = torch.randn((m, k), generator=g, device=gpu).to(FP8)
+    b = torch.randn((n, k), generator=g, device=gpu).to(FP8)
+    sa = torch.rand((k // 128, m), generator=g, device=gpu).t() * 0.01 + 0.001
+    sb = torch.rand(((n + 127) // 128, k // 128), generator=g, device=gpu) * 0.01 + 0.001
+    fp8_blockwise_scaled_mm(a, b.t(), sa, sb.t(), torch.bfloat16)
+    assert lib.sglq_debug_last_gemm_kernel().decode() == kernel
