@@ -40,6 +40,7 @@ constexpr bool fp8_operands(int kind) { return kind == KIND_FP8_BLOCK || kind ==
 constexpr bool float_acc(int kind) { return fp8_operands(kind) || kind == KIND_I8_BLOCK; }
 
 constexpr uint32_t OOB = 0x80000000u;  // offset beyond any buffer this library accepts
+constexpr uint32_t SC_NONE = 0x40000000u;  // scalar offset beyond any scale tensor (at most 2^31 / 32 bytes)
 
 struct GemmArgs {
   const char* a;   // [M, K] bytes, row stride lda
@@ -927,20 +928,23 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // Copy j (0..3) of a wave fills activation rows 8 (wave + 8 j) .. + 7 of the stage, and
   // the same rows of the weight half; lane l brings row l / 8 of those, chunk
   // (l % 8) ^ swz(row).  swz depends on l / 8 and the parity of the wave only, so the four
-  // copies share one per-lane offset and differ by a multiple of 64 rows.  Rows past M / N
-  // fall beyond the buffer's extent and read as zero; the K offset travels in the scalar
-  // operand.
+  // copies share one per-lane offset (lane_a / lane_b: the lane's row inside the tile and its
+  // chunk) and everything else travels in the scalar operand: the tile's first row, the copy's
+  // multiple of 64 rows and the K offset.  The buffer's range check covers the sum of both
+  // offsets: rows past M / N fall beyond the extent and read as zero.
   const int l8 = lane >> 3;
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
   const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
+  const uint32_t lane_a = row_in_tile * p.lda + c16, lane_b = row_in_tile * p.ldb + c16;
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
   // off_a / off_b: tile of the block after the current one (copies deferred to a tile's first
-  // step); off_a2 / off_b2: tile of the block two after the current one.
+  // step); off_a2 / off_b2: tile of the block two after the current one.  Scalars: byte offset
+  // of the tile's first row.
   uint32_t off_a = 0, off_a2 = 0, off_b = 0, off_b2 = 0;
   auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
     char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
-                                             off + (uint32_t)j * step_a, k0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16, lane_a,
+                                             off + (uint32_t)j * step_a + (uint32_t)k0, 0, 0);
   };
   // Grouped mode: every tile has its expert's weight; b_cur / b_two are the weights of the
   // tiles of the block after the current one and of the block two after it (like off_b / off_b2).
@@ -950,15 +954,16 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
     if constexpr (MODE == PIPE_GROUPED) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(two_ahead ? b_two : b_cur, p.b_bytes),
-                                               (__attribute__((address_space(3))) void*)dst, 16, off + (uint32_t)j * step_b, k0,
-                                               0, 0);
+                                               (__attribute__((address_space(3))) void*)dst, 16, lane_b,
+                                               off + (uint32_t)j * step_b + (uint32_t)k0, 0, 0);
     } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16,
-                                               off + (uint32_t)j * step_b, k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16, lane_b,
+                                               off + (uint32_t)j * step_b + (uint32_t)k0, 0, 0);
     }
   };
-  auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
-  auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
+  // (a tile past the last one: any offset beyond the extents; the sum with a lane's offset stays below 2^32)
+  auto a_offset = [&](int m0) { return m0 < p.M ? (uint32_t)m0 * p.lda : OOB; };
+  auto b_offset = [&](int n0) { return n0 < p.N ? (uint32_t)n0 * p.ldb : OOB; };
 
   const int sw = (r16 & 7) ^ (r16 >> 3);
   const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
@@ -981,14 +986,17 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // copy per K block: waves 0..3 the activation scales of tile rows 64 w + lane, wave 4 the
   // two weight scales of the tile's two 128-column blocks (lanes 0 and 1), waves 5..7 nothing
   // (all lanes out of range; kept so that the instruction stream has no branch).
-  // sc_voff / sc_voff2: per-lane source offsets for the tile of block u + 1 / u + 2.
+  // lane_s: the lane's offset inside a tile's scales; sc_off / sc_off2 (scalars): those of the
+  // tile of block u + 1 / u + 2.  Rows past M and a second column block past N are not singled
+  // out: what they read (a value inside the scale tensor, or zero beyond it) only reaches
+  // outputs that the epilogue drops.
   const int nkb_all = p.K >> 7;
   const int splits = MODE == PIPE_SPLITK ? p.splits : 1;
   const int nkb = nkb_all / splits;  // K blocks of one work unit (the host makes it divide)
   float sfa_cur[MI];
   float sfb_cur = 0.f;
   __amdgpu_buffer_rsrc_t rsc = ra;
-  uint32_t sc_voff = OOB, sc_voff2 = OOB;
+  uint32_t lane_s = OOB, sc_off = SC_NONE, sc_off2 = SC_NONE;
   int sc_step = 0;
   const int sc_dst = 2 * STAGE_BYTES + wave * 256;  // waves 5..7 land behind the used part
   const int sfa_rd = 2 * STAGE_BYTES + (wm * TM + r16) * 4;
@@ -1000,20 +1008,19 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     if constexpr (MODE == PIPE_GROUPED) sfb_elems += (int64_t)(p.num_experts - 1) * p.sb_expert_stride;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
+    if (wave < 4) lane_s = wave * 64 < BM ? (uint32_t)((wave * 64 + lane) * p.sa_stride_m * 4) : OOB;
+    else lane_s = (wave == 4 && lane < 2) ? (uint32_t)(lane * p.sb_stride_n * 4) : OOB;
   }
+  // (SC_NONE: no tile; beyond both scale tensors, and its sum with OOB does not wrap)
   auto scale_offset = [&](int m0, int n0, int expert) -> uint32_t {
-    if (wave < 4) {
-      const int row = m0 + wave * 64 + lane;
-      return (wave * 64 < BM && row < p.M) ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
-    }
-    const int nblocks = (p.N + 127) >> 7;
-    int nb = (n0 >> 7) + lane;
-    if (nb >= nblocks) nb = nblocks - 1;
-    return (wave == 4 && lane < 2) ? (uint32_t)((nb * p.sb_stride_n + expert * p.sb_expert_stride) * 4) : OOB;
+    if (m0 >= p.M || n0 >= p.N) return SC_NONE;
+    if (wave < 4) return (uint32_t)(m0 * p.sa_stride_m * 4);
+    return (uint32_t)(((n0 >> 7) * p.sb_stride_n + expert * p.sb_expert_stride) * 4);
   };
-  auto copy_scales = [&](int buf, int kb, uint32_t voff) {
+  auto copy_scales = [&](int buf, int kb, uint32_t off) {
     char* dst = smem + buf * SCALE_BYTES + sc_dst;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, voff, kb * sc_step, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kb * sc_step) + off, 0,
+                                             0);
   };
   auto read_sfa = [&](int buf, int i) -> float {
     return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfa_rd + i * 64);
@@ -1084,22 +1091,26 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           if (j == 0) a_nxt = read_frag(st + a_base + (i + 1) * 16 * 128);
         } else {
           // weight fragment j has had its last use in this step: refill it from block u + 1
-          bf[j] = read_frag(sn + b_base + j * 16 * 128);
-          if (j == 0) a_nxt = read_frag(sn + a_base);
-          if (!last && j < NCOPY_A) copy_a(j, cur, kn2 * 128, off_a2);
-          if constexpr (BLOCK) {
-            // scales i < MI - 1 had their last use when the last fragment's scale was formed; its own
-            // scale and sfb_cur are dead as well: `sc` holds their product
+          // (not in a tile's last step: the next tile's first fragments and scales are read behind
+          // the epilogue, which needs the registers)
+          if constexpr (!last) {
+            bf[j] = read_frag(sn + b_base + j * 16 * 128);
+            if (j == 0) a_nxt = read_frag(sn + a_base);
+            if (j < NCOPY_A) copy_a(j, cur, kn2 * 128, off_a2);
+            if constexpr (BLOCK) {
+              // scales i < MI - 1 had their last use when the last fragment's scale was formed; its own
+              // scale and sfb_cur are dead as well: `sc` holds their product
 #pragma unroll
-            for (int q = 0; q < MI / NI; ++q) sfa_cur[(MI / NI) * j + q] = read_sfa(cur ^ 1, (MI / NI) * j + q);
-            if (j == 0) sfb_cur = read_sfb(cur ^ 1);
-            if (j == 0 && !last) copy_scales(cur, kn2, sc_voff2);
+              for (int q = 0; q < MI / NI; ++q) sfa_cur[(MI / NI) * j + q] = read_sfa(cur ^ 1, (MI / NI) * j + q);
+              if (j == 0) sfb_cur = read_sfb(cur ^ 1);
+              if (j == 0) copy_scales(cur, kn2, sc_off2);
+            }
           }
         }
         if constexpr (first) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b, false);
           if (idx >= 8 && idx < 8 + NCOPY_A) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
-          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
+          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_off);
           if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2, true);
         } else if constexpr (!last) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2, true);
@@ -1161,22 +1172,26 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   off_a = off_a2 = a_offset(m0);
   off_b = off_b2 = b_offset(n0);
   if constexpr (MODE == PIPE_GROUPED) b_cur = b_two = p.b + (int64_t)expert * p.b_expert_stride;
-  if constexpr (BLOCK) sc_voff = sc_voff2 = scale_offset(m0, n0, expert);
+  if constexpr (BLOCK) sc_off = sc_off2 = scale_offset(m0, n0, expert);
 #pragma unroll
   for (int j = 0; j < NCOPY_A; ++j) copy_a(j, 0, kb0 * 128, off_a);
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_b(j, 0, kb0 * 128, off_b, false);
-  if constexpr (BLOCK) copy_scales(0, kb0, sc_voff);
+  if constexpr (BLOCK) copy_scales(0, kb0, sc_off);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
+  // a unit's first weight fragments, activation fragment and scales, from stage `stage`
+  auto read_first = [&](int stage) {
 #pragma unroll
-  for (int j = 0; j < NI; ++j) bf[j] = read_frag(smem + b_base + j * 16 * 128);
-  a_cur = read_frag(smem + a_base);
-  if constexpr (BLOCK) {
+    for (int j = 0; j < NI; ++j) bf[j] = read_frag(smem + stage * STAGE_BYTES + b_base + j * 16 * 128);
+    a_cur = read_frag(smem + stage * STAGE_BYTES + a_base);
+    if constexpr (BLOCK) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) sfa_cur[i] = read_sfa(0, i);
-    sfb_cur = read_sfb(0);
-  }
+      for (int i = 0; i < MI; ++i) sfa_cur[i] = read_sfa(stage, i);
+      sfb_cur = read_sfb(stage);
+    }
+  };
+  read_first(0);
 
   while (true) {
     // The block's next unit; past its last one the prefetches are pointed at rows beyond M
@@ -1194,14 +1209,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 
     // (a unit has at least three K blocks, so its first, last-but-one and last step are distinct)
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
-    uint32_t sc_voff_next = OOB;
-    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0, nexpert);
+    uint32_t sc_off_next = SC_NONE;
+    if constexpr (BLOCK) sc_off_next = scale_offset(nm0, nn0, nexpert);
     k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{});
     for (int kb = 1; kb + 1 < nkb; ++kb) {
       const bool pen = kb + 2 == nkb;  // the block two ahead is the next unit's first
       off_a2 = pen ? off_a_next : off_a2;
       off_b2 = pen ? off_b_next : off_b2;
-      sc_voff2 = pen ? sc_voff_next : sc_voff2;
+      sc_off2 = pen ? sc_off_next : sc_off2;
       if constexpr (MODE == PIPE_GROUPED) b_two = pen ? b_next : b_two;
       k_step((kb + par) & 1, kb0 + kb + 1, pen ? nkb0 : kb0 + kb + 2, std::false_type{}, std::false_type{});
     }
@@ -1210,7 +1225,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
     off_a = off_a2;
     off_b = off_b2;
-    sc_voff = sc_voff2;
+    sc_off = sc_off2;
     if constexpr (MODE == PIPE_GROUPED) b_cur = b_two;
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
@@ -1236,6 +1251,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     expert = nexpert;
     m_end = nm_end;
     par = last_stage ^ 1;
+    read_first(par);  // (landed before the last step's second barrier)
   }
 }
 
