@@ -1295,31 +1295,35 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   // Copy j of a wave fills activation rows 8 (wave + 8 j) .. + 7 of the stage, or the same
   // rows of the weight part; lane l brings row l / 8 of those, chunk (l % 8) ^ swz(row).
   // swz depends on l / 8 and the parity of the wave only, so a wave's copies share one
-  // per-lane offset and differ by a multiple of 64 rows.  Rows past M / N fall beyond the
-  // buffer's extent and read as zero; the K offset travels in the scalar operand.  A
-  // weight copy past the tile's width (224-wide tiles: the fourth copy of waves 4..7) is
-  // sent out of range as well and zero-fills stage rows that nobody reads.
+  // per-lane offset (lane_a / lane_b: the lane's row inside the tile and its chunk); the tile's
+  // first row, the copy's multiple of 64 rows and the K offset travel in the scalar operand.
+  // The buffer's range check covers the sum of both offsets: rows past M / N fall beyond the
+  // extent and read as zero.  A weight copy past the tile's width (224-wide tiles: the fourth
+  // copy of waves 4..7) is sent out of range as well and zero-fills stage rows that nobody reads.
   const int l8 = lane >> 3;
   const int c16 = (((lane & 7) ^ l8 ^ (wave & 1)) & 7) * 16;
   const uint32_t row_in_tile = (uint32_t)(wave * 8 + l8);
+  const uint32_t lane_a = row_in_tile * p.lda + c16, lane_b = row_in_tile * p.ldb + c16;
   const uint32_t step_a = 64u * p.lda, step_b = 64u * p.ldb;
   const bool last_b_ok = wave + (NBW - 1) * NW < NB;
   // off_a / off_b: tile of the block after the current one (copies deferred to a tile's first
-  // step); off_a2 / off_b2: tile of the block two after the current one.
+  // step); off_a2 / off_b2: tile of the block two after the current one.  Scalars: byte offset
+  // of the tile's first row.
   uint32_t off_a = 0, off_a2 = 0, off_b = 0, off_b2 = 0;
   auto copy_a = [&](int j, int stage, int k0, uint32_t off) {
     char* dst = smem + stage * STAGE_BYTES + (wave + j * NW) * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16,
-                                             off + (uint32_t)j * step_a, k0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)dst, 16, lane_a,
+                                             off + (uint32_t)j * step_a + (uint32_t)k0, 0, 0);
   };
   auto copy_b = [&](int j, int stage, int k0, uint32_t off_tile) {
     char* dst = smem + stage * STAGE_BYTES + BM * 128 + (wave + j * NW) * 1024;
-    uint32_t off = off_tile + (uint32_t)j * step_b;
+    uint32_t off = off_tile + (uint32_t)j * step_b + (uint32_t)k0;
     if (j == NBW - 1 && NB % NW != 0) off = last_b_ok ? off : OOB;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16, off, k0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)dst, 16, lane_b, off, 0, 0);
   };
-  auto a_offset = [&](int m0) { return (uint32_t)(m0 + row_in_tile) * p.lda + c16; };
-  auto b_offset = [&](int n0) { return (uint32_t)(n0 + row_in_tile) * p.ldb + c16; };
+  // (a tile past the last one: any offset beyond the extents; the sum with a lane's offset stays below 2^32)
+  auto a_offset = [&](int m0) { return m0 < p.M ? (uint32_t)m0 * p.lda : OOB; };
+  auto b_offset = [&](int n0) { return n0 < p.N ? (uint32_t)n0 * p.ldb : OOB; };
 
   const int sw = (r16 & 7) ^ (r16 >> 3);
   const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
@@ -1342,14 +1346,16 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   // 4-byte-per-lane copy per K block: waves 0..3 the activation scales of tile rows
   // 64 w + lane, wave 4 the weight scales of the (up to three) 128-column blocks the tile
   // touches (lanes 0..2), waves 5..7 nothing (all lanes out of range; kept so that the
-  // instruction stream has no branch).  sc_voff / sc_voff2: per-lane source offsets for the
-  // tile of block u + 1 / u + 2.  The wave's weight fragments 0 .. jsw - 1 lie in scale
+  // instruction stream has no branch).  lane_s: the lane's offset inside a tile's scales;
+  // sc_off / sc_off2 (scalars): those of the tile of block u + 1 / u + 2.  Rows past M and
+  // column blocks past N are not singled out: what they read (a value inside the scale tensor,
+  // or zero beyond it) only reaches outputs that the epilogue drops.  The wave's weight fragments 0 .. jsw - 1 lie in scale
   // block sb_lo of the tile's blocks, the others in sb_lo + 1.
   const int nkb = p.K >> 7;
   float sfa_cur[MI];
   float sfb_lo = 0.f, sfb_hi = 0.f;
   __amdgpu_buffer_rsrc_t rsc = ra;
-  uint32_t sc_voff = OOB, sc_voff2 = OOB;
+  uint32_t lane_s = OOB, sc_off = SC_NONE, sc_off2 = SC_NONE;
   int sc_step = 0, jsw = NI;
   // jsw / sfb read offset of the tile whose scales are read next (two tiles can be in flight:
   // the values for the tile of block u + 1 are needed when its scales are read)
@@ -1362,16 +1368,14 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
+    if (wave < 4) lane_s = (uint32_t)((wave * 64 + lane) * p.sa_stride_m * 4);
+    else lane_s = (wave == 4 && lane < 3) ? (uint32_t)(lane * p.sb_stride_n * 4) : OOB;
   }
+  // (SC_NONE: no tile; beyond both scale tensors, and its sum with OOB does not wrap)
   auto scale_offset = [&](int m0, int n0) -> uint32_t {
-    if (wave < 4) {
-      const int row = m0 + wave * 64 + lane;
-      return row < p.M ? (uint32_t)(row * p.sa_stride_m * 4) : OOB;
-    }
-    const int nblocks = (p.N + 127) >> 7;
-    int nb = (n0 >> 7) + lane;
-    if (nb >= nblocks) nb = nblocks - 1;
-    return (wave == 4 && lane < 3) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
+    if (m0 >= p.M || n0 >= p.N) return SC_NONE;
+    if (wave < 4) return (uint32_t)(m0 * p.sa_stride_m * 4);
+    return (uint32_t)((n0 >> 7) * p.sb_stride_n * 4);
   };
   // where this wave's columns start inside the tile's scale blocks
   auto set_scale_split = [&](int n0) {
@@ -1380,9 +1384,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     jsw_nxt = __builtin_amdgcn_readfirstlane(((nb_lo + 1) * 128 - nw) >> 4);
     sfb_rd_nxt = __builtin_amdgcn_readfirstlane(2 * STAGE_BYTES + 1024 + (nb_lo - (n0 >> 7)) * 4);
   };
-  auto copy_scales = [&](int buf, int kb, uint32_t voff) {
+  auto copy_scales = [&](int buf, int kb, uint32_t off) {
     char* dst = smem + buf * SCALE_BYTES + sc_dst;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, voff, kb * sc_step, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kb * sc_step) + off, 0,
+                                             0);
   };
   auto read_sfa = [&](int buf, int i) -> float {
     return *reinterpret_cast<const float*>(smem + buf * SCALE_BYTES + sfa_rd + i * 64);
@@ -1476,13 +1481,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
             sfa_cur[i] = read_sfa(cur ^ 1, i);
             if (i == 0) sfb_lo = read_sfb(cur ^ 1, 0);
             if (i == 1) sfb_hi = read_sfb(cur ^ 1, 1);
-            if (i == 0 && !last) copy_scales(cur, kn2, sc_voff2);
+            if (i == 0 && !last) copy_scales(cur, kn2, sc_off2);
           }
         }
         if constexpr (first) {
           if (idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
           if (idx >= 8 && idx < 8 + NBW) copy_b(idx - 8, cur ^ 1, kn * 128, off_b);
-          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_voff);
+          if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_off);
           if (idx >= 12 && idx < 16) copy_a(idx - 12, cur, kn2 * 128, off_a2);
         } else if constexpr (!last) {
           if (idx >= 4 && idx < 8) copy_a(idx - 4, cur, kn2 * 128, off_a2);
@@ -1521,14 +1526,14 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   off_a = off_a2 = a_offset(m0);
   off_b = off_b2 = b_offset(n0);
   if constexpr (BLOCK) {
-    sc_voff = sc_voff2 = scale_offset(m0, n0);
+    sc_off = sc_off2 = scale_offset(m0, n0);
     set_scale_split(n0);
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
 #pragma unroll
   for (int j = 0; j < NBW; ++j) copy_b(j, 0, 0, off_b);
-  if constexpr (BLOCK) copy_scales(0, 0, sc_voff);
+  if constexpr (BLOCK) copy_scales(0, 0, sc_off);
   __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -1558,8 +1563,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 
     // (K >= 384 for this kernel, so the first, the last-but-one and the last step are distinct)
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
-    uint32_t sc_voff_next = OOB;
-    if constexpr (BLOCK) sc_voff_next = scale_offset(nm0, nn0);
+    uint32_t sc_off_next = SC_NONE;
+    if constexpr (BLOCK) sc_off_next = scale_offset(nm0, nn0);
     const int last_stage = (nkb - 1 + par) & 1;
     // the tile's K steps, instantiated for the position of the scale-block boundary among this wave's fragments
     auto tile_steps = [&](auto jsw_tag) __attribute__((always_inline)) {
@@ -1568,7 +1573,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         const bool pen = kb + 2 == nkb;  // the block two ahead is the next tile's first
         off_a2 = pen ? off_a_next : off_a2;
         off_b2 = pen ? off_b_next : off_b2;
-        sc_voff2 = pen ? sc_voff_next : sc_voff2;
+        sc_off2 = pen ? sc_off_next : sc_off2;
         k_step((kb + par) & 1, kb + 1, pen ? 0 : kb + 2, std::false_type{}, std::false_type{}, jsw_tag);
       }
       // last K block: the scales read behind its last MFMAs are the next tile's; its copies (the
@@ -1597,7 +1602,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     }
     off_a = off_a2;
     off_b = off_b2;
-    sc_voff = sc_voff2;
+    sc_off = sc_off2;
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
