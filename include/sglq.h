@@ -149,7 +149,8 @@ int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b,
  *   x    [M, K] contiguous activations, in_dtype in {BF16, FP16, FP32}, 16-byte aligned, K % 128 == 0
  *   b, sfb, bias (may be NULL), out: as sglq_fp8_blockwise_scaled_mm_bias
  *   eps  lower bound of a group's abs-max (the callers' 1e-10)
- * For M <= 8 (16-bit activations) on the shapes that the decode kernel without split-K takes, one
+ * For M <= 4 (16-bit activations) on the shapes that the decode kernel without split-K takes with
+ * between one and 2.5 blocks per compute unit (where it was measured faster), one
  * kernel quantizes each K block's activations in LDS right before multiplying them: no
  * quantization launch, no round trip of codes and scales through memory, no workspace.  Other
  * shapes run the quantization kernel and the GEMM one after the other; their codes and
