@@ -24,7 +24,7 @@ namespace sglq {
 // the quotient by 448 * (1 + 2^-22), which rounds to the code of 448 anyway, so
 // the explicit clamp is dropped.  The quotient's sign is copied from x so that
 // -0.0 stays -0.0 (the remainder correction would turn it into +0.0).
-template <int DT, int GROUP, int NCH, int UNROLL, bool STRIDED_SCALE, bool TO_INT8, bool CLAMP>
+template <int DT, int GROUP, int NCH, int UNROLL, bool STRIDED_SCALE, bool TO_INT8, bool CLAMP, bool STREAM_IN = false>
 __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
                                                           float* __restrict__ s, uint32_t num_groups,
                                                           FastDiv groups_per_row, int64_t s_stride_row,
@@ -46,7 +46,12 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict
     if (gid < num_groups) {
       const char* p = x + ((int64_t)gid * GROUP + sub * 8) * EB;
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) ch[u][c].load(p + c * (GROUP / NCH) * EB);
+      for (int c = 0; c < NCH; ++c) {
+        // (an input of half the last-level cache and more is read past it: what the cache holds for the
+        // kernels around this one, often the previous GEMM's output still to be written back, stays put)
+        if constexpr (STREAM_IN) ch[u][c].load_once(p + c * (GROUP / NCH) * EB);
+        else ch[u][c].load(p + c * (GROUP / NCH) * EB);
+      }
     }
   }
 #pragma unroll
@@ -502,13 +507,19 @@ static void launch_group_quant(const void* x, void* q, float* s, uint32_t num_gr
   const bool deep = SGLQ_GQ_UNROLL > 1 && num_groups >= (uint32_t)GPB * SGLQ_GQ_UNROLL * 2048;
   const char* xi = static_cast<const char*>(x);
   char* qo = static_cast<char*>(q);
-#define SGLQ_LAUNCH_GQ(U, STR)                                                                              \
-  group_quant_kernel<DT, GROUP, NCH, U, STR, TO_INT8, CLAMP><<<dim3((num_groups + GPB * U - 1) / (GPB * U)), dim3(256), 0, st>>>( \
+  // measured on 4096 x 16384 bf16 (128 MiB) right behind a GEMM that wrote 268 MB: 49.3 -> 38.5 us; timed alone
+  // 8192 x 16384 70.4 -> 64.3 us, 4096 x 28672 63.3 -> 61.2 us, but 8192 x 7168 (112 MiB) 33.3 -> 33.8 us and
+  // 8192 x 1536 (24 MiB) 7.8 -> 9.0 us: hence the threshold
+  const bool stream_in = (int64_t)num_groups * GROUP * elem_bytes<DT>() >= ((int64_t)128 << 20);
+#define SGLQ_LAUNCH_GQ(U, STR, ONCE)                                                                        \
+  group_quant_kernel<DT, GROUP, NCH, U, STR, TO_INT8, CLAMP, ONCE><<<dim3((num_groups + GPB * U - 1) / (GPB * U)), dim3(256), 0, st>>>( \
       xi, qo, s, num_groups, fd, sr, sc, eps, qmin, qmax, rq)
-  if (deep) {
-    if (strided) SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, true); else SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, false);
+  if (stream_in) {
+    if (strided) SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, true, true); else SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, false, true);
+  } else if (deep) {
+    if (strided) SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, true, false); else SGLQ_LAUNCH_GQ(SGLQ_GQ_UNROLL, false, false);
   } else {
-    if (strided) SGLQ_LAUNCH_GQ(1, true); else SGLQ_LAUNCH_GQ(1, false);
+    if (strided) SGLQ_LAUNCH_GQ(1, true, false); else SGLQ_LAUNCH_GQ(1, false, false);
   }
 #undef SGLQ_LAUNCH_GQ
 }

@@ -18,6 +18,9 @@ struct Chunk8<SGLQ_BF16> {
   v4u raw;
   static constexpr int kBytes = 16;
   SGLQ_MEM void load(const void* p) { raw = *reinterpret_cast<const v4u*>(p); }
+  // for data that is read exactly once: the non-temporal hint keeps it from displacing what the
+  // last-level cache holds for the kernels around this one
+  SGLQ_MEM void load_once(const void* p) { raw = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p)); }
   SGLQ_MEM uint32_t amax_bits() const {
     // |bf16| orders like its low 15 bits taken as an integer: packed 16-bit max.
     v2us m = {0, 0};
@@ -40,6 +43,9 @@ struct Chunk8<SGLQ_FP16> {
   v4u raw;
   static constexpr int kBytes = 16;
   SGLQ_MEM void load(const void* p) { raw = *reinterpret_cast<const v4u*>(p); }
+  // for data that is read exactly once: the non-temporal hint keeps it from displacing what the
+  // last-level cache holds for the kernels around this one
+  SGLQ_MEM void load_once(const void* p) { raw = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p)); }
   SGLQ_MEM float get(int i) const {
     uint32_t w = raw[i >> 1];
     unsigned short h = (i & 1) ? (unsigned short)(w >> 16) : (unsigned short)(w & 0xffffu);
@@ -60,6 +66,10 @@ struct Chunk8<SGLQ_FP32> {
   SGLQ_MEM void load(const void* p) {
     raw[0] = reinterpret_cast<const v4u*>(p)[0];
     raw[1] = reinterpret_cast<const v4u*>(p)[1];
+  }
+  SGLQ_MEM void load_once(const void* p) {
+    raw[0] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+    raw[1] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p) + 1);
   }
   SGLQ_MEM float get(int i) const { return u2f(raw[i >> 2][i & 3]); }
   SGLQ_MEM uint32_t amax_bits() const {
