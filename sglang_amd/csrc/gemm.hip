@@ -1263,7 +1263,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 // ahead.  The tile width is chosen on the host so that the tile count fills whole rounds of
 // the chip's CUs: 7168 columns are 32 tiles of 224 (two full rounds at M = 4096) instead
 // of 28 tiles of 256 (one full round and a 3/4 one).  A wave's columns can straddle two
-// 128-column scale blocks, so the weight scale is selected per fragment.  Here the
+// 128-column scale blocks: the K steps are instantiated per position of that boundary among the
+// wave's fragments and the tile loop dispatches on it once per tile.  Here the
 // activation half of a stage is the one that is free early (barrier 1, behind MFMA 3: all
 // four activation fragments are in registers) and is refilled two K blocks ahead; the
 // weight copies of block u + 2 follow behind the last weight fragment's MFMAs.
