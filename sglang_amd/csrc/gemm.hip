@@ -1627,16 +1627,22 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 // contiguous range of K blocks (split-K across blocks); its four waves take 32
 // rows each.  Weight tiles (16 KiB), the activation tile and, for the block-scaled
 // kind, the activation scales of each K block are copied global -> LDS through a
-// ring of NSTAGE stages, NSTAGE - 1 copies ahead of the MFMAs (80-100 KiB in
-// flight per CU).  All copies of a stage are vector-memory loads that retire in
-// order, so "stage t has landed" is a vmcnt wait that leaves the younger stages'
-// loads outstanding.  With splits > 1 the partial sums go to a workspace and
+// ring of NSTAGE stages (80-100 KiB in flight per CU); a K block's fragments are read
+// from LDS into registers one step before its MFMAs, so the block's stage is free for
+// the copy NSTAGE blocks ahead as soon as the step starts, and the LDS reads, the
+// copies and the scale-and-accumulate of each MFMA's result overlap the MFMAs (a block
+// may be alone on its CU, one wave per SIMD).  All copies of a stage are vector-memory
+// loads that retire in order, so "stage t has landed" is a vmcnt wait that leaves the
+// younger stages' loads outstanding.  With splits > 1 the partial sums go to a workspace and
 // splitk_reduce_kernel applies the epilogue.  For 64 < M <= 512 there are several 64-row
 // tiles per weight tile; they run side by side on one XCD, so the weights still come from
 // HBM once and from that XCD's L2 after that.
 // ---------------------------------------------------------------------------
 template <int KIND, int MI, int OUT_DT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
+// (two waves per SIMD asked for: with at most 256 registers per lane the MFMAs write plain
+// VGPRs; given 512 the compiler puts their results into accumulation registers and copies
+// each one out behind a full MFMA latency of wait states)
+__global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int BN = 128, NI = 2;
   constexpr int AR = MI * 16 < 32 ? 32 : MI * 16;  // activation rows staged (at least one copy per wave)
   constexpr int ACW = AR / 32;                     // activation copies per wave per stage
@@ -1645,8 +1651,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 2048 : 0;  // 4 x 256 B of activation scales, then the weight scale
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
   // 60-78 KiB of LDS: two blocks (eight waves) per CU.  A ring of six stages (one block per CU,
-  // five stages in flight) was measured and is no faster: a launch of 256 blocks asks for its
-  // first stages all at once, and what the memory system delivers to that burst sets the time.
+  // five stages in flight) is slower wherever it was tried, also for launches of fewer blocks than
+  // CUs whose blocks walk 56 K blocks each (64 x 2048 x 7168 without split-K: 29.5 us with three stages,
+  // 32.9 with six): what a CU's load path delivers sets the step time, not the depth of the ring.
   constexpr int NSTAGE = 3;
   constexpr bool IS_FP8 = fp8_operands(KIND);
 
@@ -1733,48 +1740,100 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
-#pragma unroll
-  for (int t = 0; t < NSTAGE - 1; ++t)
-    if (t < nsteps) issue_group(t);
-
-  for (int t = 0; t < nsteps; ++t) {
-    // wait for stage t: at most NSTAGE - 2 younger groups may stay in flight
-    if (nsteps - 1 - t >= NSTAGE - 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NSTAGE - 2) * CPW));
-    else __builtin_amdgcn_s_waitcnt(0);
-    __builtin_amdgcn_s_barrier();  // visible to all waves; and everyone is done with stage (t - 1) % NSTAGE
-    if (t + NSTAGE - 1 < nsteps) issue_group(t + NSTAGE - 1);
-
+  // Every stage of the ring is filled before the first MFMA; after that, step t runs on the
+  // fragments of K block t that step t - 1 read from LDS into registers, and while its MFMAs
+  // run it reads the fragments of block t + 1 and refills block t's stage with block t + NSTAGE.
+  // Two register sets take turns (the loop below is unrolled by two), so nothing is moved.
+  struct Frags {
+    v8i f[NI + MI];  // weight fragments, then activation fragments
+    float sa[MI], sb;
+  };
+  Frags fa, fb;
+  auto read_one = [&](int t, Frags& d, int k) {  // k-th LDS read group of K block t
     const char* st = smem + (t % NSTAGE) * STAGE_BYTES;
-    v8i wf[NI], af[MI];
-#pragma unroll
-    for (int j = 0; j < NI; ++j) wf[j] = read_frag(st + (wave * 32 + j * 16) * 128);
-#pragma unroll
-    for (int i = 0; i < MI; ++i) af[i] = read_frag(st + W_BYTES + i * 16 * 128);
-    float sc[MI];
-    if constexpr (BLOCK) {
-      const float sfb = *reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + 1024);
+    if (k < NI) d.f[k] = read_frag(st + (wave * 32 + k * 16) * 128);
+    else if (k < NI + MI) d.f[k] = read_frag(st + W_BYTES + (k - NI) * 16 * 128);
+    else if constexpr (BLOCK) {
+      d.sb = *reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + 1024);
       const float* sfa = reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + wave * 256);
 #pragma unroll
-      for (int i = 0; i < MI; ++i) sc[i] = sfa[i * 16 + r16] * sfb;
+      for (int i = 0; i < MI; ++i) d.sa[i] = sfa[i * 16 + r16];
     }
+  };
+  constexpr int NREAD = NI + MI + 1;
+  // "K block u has landed" with the blocks up to u + younger issued: copies retire in order
+  static_assert((NSTAGE - 1) * CPW < 64, "vmcnt holds six bits");
+  static_assert(NSTAGE == 3, "wait_landed counts at most two younger blocks");
+  auto wait_landed = [&](int younger) {
+    if (younger >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * CPW));
+    else if (younger == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(CPW));
+    else __builtin_amdgcn_s_waitcnt(0);
+  };
+
+  auto step = [&](int t, Frags& cur, Frags& nxt) {
+    // Block t + 1 has landed (the blocks up to t + NSTAGE - 1 are issued), and this wave's LDS
+    // reads of block t are complete; behind the barrier both hold for every wave, so block t's
+    // stage can be refilled.
+    const int issued = t + NSTAGE - 1 < nsteps - 1 ? t + NSTAGE - 1 : nsteps - 1;
+    wait_landed(issued - (t + 1));
+    __builtin_amdgcn_s_barrier();
+    if (t + NSTAGE < nsteps) issue_group(t + NSTAGE);
+    float sc[MI];
+    if constexpr (BLOCK) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
+      for (int i = 0; i < MI; ++i) sc[i] = cur.sa[i] * cur.sb;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    constexpr int NMFMA = MI * NI;
+    // the result of MFMA idx is folded into the accumulator while MFMA idx + 1 runs
+    v4f part[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        if constexpr (BLOCK) {
-          v4f part = block_mfma<KIND>(wf[j], af[i]);
+    for (int idx = 0; idx < NMFMA; ++idx) {
+      const int i = idx / NI, j = idx % NI;
+      if constexpr (BLOCK) {
+        part[idx & 1] = block_mfma<KIND>(cur.f[j], cur.f[NI + i]);
+      } else if constexpr (KIND == KIND_FP8_ROWCOL) {
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(cur.f[j], cur.f[NI + i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      } else {
+        const v8i &w = cur.f[j], &a = cur.f[NI + i];
+        const v4i b0 = {w[0], w[1], w[2], w[3]}, b1 = {w[4], w[5], w[6], w[7]};
+        const v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // the LDS reads of block t + 1 are spread over the MFMAs (after the last block: of a stage
+      // that holds an older block, unused)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(block_value<KIND>(part[e]), sc[i], acc[i][j][e]);
-        } else if constexpr (KIND == KIND_FP8_ROWCOL) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
-        } else {
-          const v4i b0 = {wf[j][0], wf[j][1], wf[j][2], wf[j][3]}, b1 = {wf[j][4], wf[j][5], wf[j][6], wf[j][7]};
-          const v4i a0 = {af[i][0], af[i][1], af[i][2], af[i][3]}, a1 = {af[i][4], af[i][5], af[i][6], af[i][7]};
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, a0, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
+      for (int k = 0; k < NREAD; ++k)
+        if (k * NMFMA / NREAD == idx) read_one(t + 1, nxt, k);
+      if constexpr (BLOCK) {
+        if (idx > 0) {
+          const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[pi][pj][e] = __builtin_fmaf(block_value<KIND>(part[(idx - 1) & 1][e]), sc[pi], acc[pi][pj][e]);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (BLOCK) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[MI - 1][NI - 1][e] = __builtin_fmaf(block_value<KIND>(part[(NMFMA - 1) & 1][e]), sc[MI - 1], acc[MI - 1][NI - 1][e]);
+    }
+  };
+
+#pragma unroll
+  for (int t = 0; t < NSTAGE; ++t)
+    if (t < nsteps) issue_group(t);
+  wait_landed(nsteps - 1 < NSTAGE - 1 ? nsteps - 1 : NSTAGE - 1);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int k = 0; k < NREAD; ++k) read_one(0, fa, k);
+
+  for (int t = 0; t < nsteps; t += 2) {
+    step(t, fa, fb);
+    if (t + 1 < nsteps) step(t + 1, fb, fa);
   }
 
   if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, m_base, n0 + wave * 32, r16, g);
@@ -2461,26 +2520,46 @@ static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
-// Decode path: choose the split-K factor so that every CU streams weights.
+// The split-K factor of the decode path without the caller's workspace limits: so that every CU streams weights.
+static int skinny_splits(int M, int N, int K) {
+  const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
+  const int nkb = K >> 7;
+  // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
+  // more blocks only add partial-sum traffic.
+  int splits = 256 / tiles;
+  int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
+  if (tiles_m > 1) {
+    // Several row tiles share a weight tile's traffic.  The split is the cheapest under a model fitted to
+    // sweeps of the split factor (256 x 2048 x 7168, 64 tiles: 29.8 / 21.0 / 17.5 / 16.3 / 18.3 / 18.8 us with
+    // 1 / 2 / 3 / 4 / 6 / 8 splits; 160 x 7168 x 2048, 168 tiles: 17.4 us with two splits, 12.7 us for the 224
+    // tiles of 256 rows with one; 512 x 2112 x 7168, 136 tiles: 29.9 us with one, 24.2 with two): 0.5 us per K
+    // block while the blocks fit one per CU, proportionally more beyond; with a split, 4 us for the second
+    // launch plus the partial sums written and read at 4 TB/s.  At most eight splits, at least four K blocks each.
+    const int max_splits = nkb / 4 > 8 ? 8 : (nkb / 4 > 0 ? nkb / 4 : 1);
+    double best = 0.0;
+    splits = 1;
+    for (int sp = 1; sp <= max_splits; ++sp) {
+      const int blocks = tiles * sp;
+      const double steps = (double)((nkb + sp - 1) / sp);
+      double cost = steps * 0.5 * (blocks > 256 ? blocks / 256.0 : 1.0);
+      if (sp > 1) cost += 4.0 + (double)M * N * 4.0 * sp * 2.0 / 4e6;
+      if (sp == 1 || cost < best) {
+        best = cost;
+        splits = sp;
+      }
+    }
+    return splits;
+  }
+  if (splits > by_steps) splits = by_steps;
+  return splits < 1 ? 1 : splits;
+}
+
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + 63) / 64;
   p.tiles_n = (p.N + 127) / 128;
   const int nkb = p.K >> 7;
-  // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
-  // more blocks only add partial-sum traffic.
-  int splits = 256 / (p.tiles_n * p.tiles_m);
-  int by_steps = nkb / 2 > 0 ? nkb / 2 : 1;  // at least two K blocks per split
-  if (p.tiles_m > 1) {
-    // several row tiles share a weight tile's traffic: somewhat more blocks pay (96 x 6144 x 4096: 19.3 us
-    // with two splits, 17.9 with three), no more than eight splits (96 x 1536 x 7168: 16.9 us with 13, 14.8
-    // with 8), at least four K blocks per split
-    splits = 320 / (p.tiles_n * p.tiles_m);
-    if (splits > 8) splits = 8;
-    by_steps = nkb / 4 > 0 ? nkb / 4 : 1;
-  }
-  if (splits > by_steps) splits = by_steps;
-  if (splits < 1) splits = 1;
+  int splits = skinny_splits(p.M, p.N, p.K);
   if (t_splits > 0) splits = t_splits < nkb ? t_splits : nkb;
   const int64_t per_split = (int64_t)p.M * p.N * 4;
   if (!p.ws || ws_bytes < per_split * 2) splits = 1;
@@ -2617,28 +2696,25 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   if ((p.K & 127) == 0 && p.M <= 64 && g_use_dma && (t_tile == 0 || t_tile == 16 || t_tile == 32) &&
       launch_stream<KIND, OUT_DT>(p, st))
     return;
-  // ... and up to 128 rows (two 64-row tiles side by side) with K <= 8192 it still beats the
-  // 128 x 128 kernel (measured, e.g. 128 x 24576 x 1536: 28.3 -> 16.3 us, 128 x 4096 x 7168:
-  // 21.2 -> 17.9 us; at K = 16384 the 128 x 128 kernel wins, 35 against 49 us).
-  // (not with large weights: 96 x 57344 x 8192 takes 194 us there against 115 us on the pipelined kernel)
+  // The same kernel with several 64-row tiles per weight tile (side by side on one XCD) takes up to 512 rows
+  // from the 128-row kernels where its blocks fit the chip at once (two per CU), a block has at most 56 K
+  // blocks to walk after the split, and, beyond two row tiles, the weights are small enough for the row tiles'
+  // re-reads to stay in the caches.  Measured per kind over M = 96 ... 512 on 17 weight shapes, e.g. block-scaled
+  // FP8 256 x 4096 x 7168: 24.6 us on the pipelined 128-row kernel, 21.8 us here; 512 x 4096 x 4096: 24.7 -> 19.7;
+  // 128 x 14336 x 4096: 28.8 -> 22.3; but 160 x 14336 x 4096 (59 MB, three row tiles): 30.7 against 33.5,
+  // 160 x 8192 x 8192 (64 K blocks per block): 31.2 against 35.2, 160 x 24576 x 1536 (576 tiles): 18.5 against 22.9.
   const int64_t weight_bytes = (int64_t)p.N * p.K;
-  // The kinds without block scales (no scale folds between the MFMAs) keep it longer: up to 128 rows on
-  // weights below 64 MB (128 x 14336 x 4096 INT8: 28.7 us on the pipelined kernel, 23.5 us here) and up to
-  // 512 rows on weights of up to 26 MB (512 x 4096 x 4096 FP8: 24.9 -> 19.5 us).
-  const bool plain_scales = !is_block(KIND);
-  const bool skinny_rows = p.M <= 64 || (p.M <= 128 && p.K <= 8192 && weight_bytes < (48 << 20)) ||
-                           (plain_scales && p.M <= 128 && weight_bytes < (64 << 20)) ||
-                           // (not on wide weights, whose many row tiles re-read them past the L2: 512 x 32768 x 512
-                           // 25.4 us here, 16.9 us on the 256-row kernel; 512 x 16384 x 1024 19.2 against 14.3 us)
-                           (plain_scales && p.M <= 512 && weight_bytes <= (26 << 20) && (p.N <= 8192 || (p.M <= 256 && p.N <= 16384))) ||
-                           (p.M <= 256 && weight_bytes < (16 << 20)) ||  // (256 x 7168 x 2048 block-FP8: 21.2 -> 15.5 us)
-                           // (160 x 8192 x 2048: 17.9 -> 14.6 us; on N = 32768 the row tiles' second reads of the weights miss the L2)
-                           (p.M <= 256 && weight_bytes <= (16 << 20) && p.K <= 2048 && p.N <= 16384) ||
-                           // narrow and deep (160 x 1024 x 16384: 25.0 -> 19.2 us, 160 x 2048 x 8192: 20.8 -> 18.0 us)
-                           (weight_bytes <= (16 << 20) && (p.N <= 1024 ? p.M <= 256 : p.N <= 2048 && p.M <= 192)) ||
-                           // small weights, deep K (512 x 1024 x 4096: 22.4 -> 16.9 us, 512 x 512 x 7168: 19.4 -> 15.6 us)
-                           (p.M <= 512 && weight_bytes <= (6 << 20) && p.K >= 4096) ||
-                           (t_tile == 64 && p.M <= 512);
+  // (K blocks per block counted with no more blocks than CUs: 96 x 7168 x 16384 with three splits, 336 blocks of
+  // 43 K blocks over 117 MB of weights, takes 50 us against 35; and, for the block-scaled kinds, not 41-56 K blocks on
+  // fewer than 224 blocks: 384 x 4096 x 7168, 192 blocks, 30 us against 26-28, where the 256 blocks of 512 rows take 30
+  // against 32; per-channel FP8 takes 23 us there against 28)
+  const int skinny_tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
+  int skinny_fit = skinny_splits(p.M, p.N, p.K);
+  if (skinny_fit * skinny_tiles > 256) skinny_fit = 256 / skinny_tiles > 0 ? 256 / skinny_tiles : 1;
+  const int skinny_steps = ((p.K >> 7) + skinny_fit - 1) / skinny_fit;
+  const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && (p.M <= 128 || weight_bytes < (48 << 20)) &&
+                          !(is_block(KIND) && skinny_steps > 40 && skinny_fit * skinny_tiles < 224);
+  const bool skinny_rows = p.M <= 64 || skinny_mid || (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
