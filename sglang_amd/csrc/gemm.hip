@@ -2608,6 +2608,8 @@ static int stream_rows(const GemmArgs& p) {
       // enough blocks (64 x 4096 x 7168: 14.1 -> 10.3 us, 64 x 4096 x 4096: 14.8 -> 8.3 us; but
       // 64 x 8192 x 8192: 22 -> 27 us and 64 x 13824 x 2048: 14.4 -> 15.8 us)
       nib = ((int64_t)p.N * p.K <= (30 << 20) && p.N <= 10240) ? 1 : 0;
+      // (32-row blocks where they fill most of one round: 64 x 6144 x 4096, 192 blocks, 13.4 -> 10.1 us)
+      if (nib == 1 && 8 * blocks32 >= 5 * num_cus() && blocks32 <= num_cus()) nib = 2;
       // ... and with 32-row blocks where those fill exactly one round of the CUs (half the activation bytes per
       // weight byte of the 16-row blocks; 64 x 8192 x 8192: 21.3 us on the split-K kernel, 20.4 us here,
       // 33 x 8192 x 8192: 20.2 -> 18.5 us; with 224 blocks, 64 x 7168 x 16384, it loses: 32.7 -> 34.2 us)
@@ -2702,7 +2704,9 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   // re-reads to stay in the caches.  Measured per kind over M = 96 ... 512 on 17 weight shapes, e.g. block-scaled
   // FP8 256 x 4096 x 7168: 24.6 us on the pipelined 128-row kernel, 21.8 us here; 512 x 4096 x 4096: 24.7 -> 19.7;
   // 128 x 14336 x 4096: 28.8 -> 22.3; but 160 x 14336 x 4096 (59 MB, three row tiles): 30.7 against 33.5,
-  // 160 x 8192 x 8192 (64 K blocks per block): 31.2 against 35.2, 160 x 24576 x 1536 (576 tiles): 18.5 against 22.9.
+  // 160 x 8192 x 8192 (64 K blocks per block): 31.2 against 35.2, 160 x 24576 x 1536 (576 tiles): 18.5 against 22.9;
+  // with two row tiles up to 64 MB of weights (128 x 8192 x 8192: 29.8 -> 27.3 us, but 96 x 5120 x 13824, 68 MB:
+  // 28.5 against 35.3, 96 x 18432 x 7168: 43.5 against 55.4).
   const int64_t weight_bytes = (int64_t)p.N * p.K;
   // (K blocks per block counted with no more blocks than CUs: 96 x 7168 x 16384 with three splits, 336 blocks of
   // 43 K blocks over 117 MB of weights, takes 50 us against 35; and, for the block-scaled kinds, not 41-56 K blocks on
@@ -2712,7 +2716,7 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   int skinny_fit = skinny_splits(p.M, p.N, p.K);
   if (skinny_fit * skinny_tiles > 256) skinny_fit = 256 / skinny_tiles > 0 ? 256 / skinny_tiles : 1;
   const int skinny_steps = ((p.K >> 7) + skinny_fit - 1) / skinny_fit;
-  const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && (p.M <= 128 || weight_bytes < (48 << 20)) &&
+  const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && weight_bytes <= (p.M <= 128 ? (64 << 20) : (48 << 20) - 1) &&
                           !(is_block(KIND) && skinny_steps > 40 && skinny_fit * skinny_tiles < 224);
   const bool skinny_rows = p.M <= 64 || skinny_mid || (t_tile == 64 && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {

@@ -670,7 +670,7 @@ BASELINE_KERNELS = [
     # decode launches of the same shapes
     ((1, 7168, 16384), "gemm_stream_kernel<16 rows>"),
     ((8, 7168, 16384), "gemm_stream_kernel<16 rows>"),
-    ((64, 7168, 16384), "gemm_skinny_kernel+splitk_reduce_kernel"),
+    ((64, 7168, 16384), "gemm_kernel+splitk_reduce_kernel"),  # (tuned table entry)
     ((1, 4096, 7168), "gemm_stream_kernel<16 rows>"),
     ((64, 4096, 7168), "gemm_stream_kernel<16 rows>"),
     ((1, 24576, 1536), "gemm_skinny_kernel"),
