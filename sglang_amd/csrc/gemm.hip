@@ -2491,14 +2491,18 @@ static void launch_wide(GemmArgs& p, hipStream_t st) {
 // Tile width of the 256-row kernels.  Every CU works through ceil(tiles / CUs) tiles, each
 // costing in proportion to its width: take the width with the least rounds x width (7168
 // columns at M = 4096: 2 x 224 against 2 x 256; 2112 columns: 1 x 192 against 1 x 256).
-static int pick_tile_width(const GemmArgs& p) {
+// narrow_only: not the 256-wide kernel (block-scaled INT8 on short K, where its epilogue weighs most and its
+// two MFMAs per K block leave no registers to spare: 4096 x 32768 x 512 163 us there, 120 us on 192-wide tiles;
+// 4096 x 24576 x 1536 227 -> 197 us)
+static int pick_tile_width(const GemmArgs& p, bool narrow_only = false) {
   const int tiles_m = (p.M + 255) / 256;
-  int best = 256;
+  const int widest = narrow_only ? 224 : 256;
+  int best = widest;
   int64_t best_cost = 0;
-  for (int bn = 256; bn >= 192; bn -= 32) {
+  for (int bn = widest; bn >= 192; bn -= 32) {
     const int tiles = tiles_m * ((p.N + bn - 1) / bn);
     const int64_t cost = (int64_t)((tiles + num_cus() - 1) / num_cus()) * bn;
-    if (bn == 256 || cost < best_cost) {
+    if (bn == widest || cost < best_cost) {
       best = bn;
       best_cost = cost;
     }
@@ -2739,7 +2743,7 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   }
   const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 192 || t_tile == 224 || t_tile == 257;
   if ((p.K & 127) == 0 && (forced_256 || (t_tile == 0 && g_use_dma && p.M > 64 && (big_tiles >= 140 || deep)))) {
-    int width = t_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p) : 256) : t_tile;
+    int width = t_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p, KIND == KIND_I8_BLOCK && p.K <= 2048 && p.M >= 2048) : 256) : t_tile;
     if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
