@@ -2555,6 +2555,8 @@ static int skinny_splits(int M, int N, int K) {
     return splits;
   }
   if (splits > by_steps) splits = by_steps;
+  // (a handful of weight tiles: 64 x 512 x 7168, four tiles, 15.2 us with 28 splits, 11.9 us with 8)
+  if (tiles < 8 && splits > 8) splits = 8;
   return splits < 1 ? 1 : splits;
 }
 
@@ -2620,7 +2622,9 @@ static int stream_rows(const GemmArgs& p) {
       if (nib == 0 && p.K >= 8192 && blocks32 <= num_cus() && 16 * blocks32 > 15 * num_cus()) nib = 2;
     }
     if (nib == 2 && p.N < 2048) nib = 1;
-    if (p.N < 1024) nib = 0;
+    // narrow weights: 16-row blocks up to 32 rows (8 x 512 x 7168: 14.2 us on the split-K kernel, two launches,
+    // 5.8 us here; 32 x 256 x 7168: 14.1 -> 6.8 us), the split-K kernel above that (64 x 512 x 7168: 11.9 us)
+    if (p.N < 1024) nib = p.M <= 32 ? 1 : 0;
   }
   return nib;
 }
@@ -2742,7 +2746,11 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     if (model_pipe_splits(p, 128, ws_bytes, s128) < model_pipe_splits(p, 256, ws_bytes, s256)) deep = false;
   }
   const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 192 || t_tile == 224 || t_tile == 257;
-  if ((p.K & 127) == 0 && (forced_256 || (t_tile == 0 && g_use_dma && p.M > 64 && (big_tiles >= 140 || deep)))) {
+  // (up to 128 rows a 256-row tile is half empty: 96 x 36864 x 7168 73.2 us on 192-wide tiles, 65.1 us on 128-row
+  // tiles; block-scaled INT8 with one or two K blocks runs 20-35 % faster on the 128 x 128 kernel than on the
+  // unpipelined 256 x 256 one: 4096 x 7168 x 128 33.0 -> 27.3 us, 3072 x 7168 x 256 35.7 -> 26.2 us)
+  const bool rows_256 = p.M > 128 && !(KIND == KIND_I8_BLOCK && p.K < 384);
+  if ((p.K & 127) == 0 && (forced_256 || (t_tile == 0 && g_use_dma && rows_256 && (big_tiles >= 140 || deep)))) {
     int width = t_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p, KIND == KIND_I8_BLOCK && p.K <= 2048 && p.M >= 2048) : 256) : t_tile;
     if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);

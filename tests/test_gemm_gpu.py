@@ -660,6 +660,26 @@ def test_shipped_tuned_tables_give_oracle_results(gpu):
             torch.testing.assert_close(out[:rows, cols].cpu().float(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("mnk,kernel", [((8, 576, 7168), "gemm_stream_kernel<16 rows>"), ((32, 256, 7168), "gemm_stream_kernel<16 rows>"),
+                                        ((64, 512, 7168), "gemm_skinny_kernel+splitk_reduce_kernel"),
+                                        ((96, 36864, 2048), "gemm_pipe_kernel<128 rows>")])
+def test_narrow_weights_and_few_rows(gpu, mnk, kernel):
+    """Shapes of the reference's tuned tables at the edges of the selection rules (N = 256 ... 576 of the
+    DeepSeek-V3 projections; up to 128 rows on a wide weight): the kernel the rules choose, against the oracle."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    say("narrow / few rows", mnk, kernel)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = sample_rows(m, 16)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    xs_cm = xs.t().contiguous().to(gpu).t()
+    out = fp8_blockwise_scaled_mm(xq.to(gpu), wq.to(gpu).t(), xs_cm, ws.to(gpu).t(), torch.bfloat16)
+    assert _lib.load().sglq_debug_last_gemm_kernel().decode() == kernel
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+
+
 BASELINE_KERNELS = [
     # (M, N, K) of the headline step and the kernel the profile summaries under profiles/ name for it
     ((4096, 24576, 1536), "gemm_pipe_kernel"),
