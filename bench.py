@@ -532,9 +532,10 @@ def time_kernel(fn, iters, rotate=1):
 def config_summary(args):
     """Every configuration of the baseline, graph-timed as --sweep does, condensed for the one JSON line:
     per (config, shape) the quantization and GEMM device times and the fraction of the roofline that bounds
-    the GEMM there (HBM for the decode-sized M, MFMA for the prefill-sized ones)."""
+    the GEMM there: of the two lower bounds on its time, algorithmic bytes / 8 TB/s and operations / 5 P(FL)OP/s,
+    the larger one."""
     rows = []
-    run_sweep(args, collect=rows, cfg2_ms=(64, 8192), only={"0", "1", "2", "3", "4"})
+    run_sweep(args, collect=rows, cfg2_ms=(1, 64, 512, 8192), only={"0", "1", "2", "3", "4"})
     out = {}
     for r in rows:
         cfg = f"cfg{r['cfg']}"
@@ -543,7 +544,7 @@ def config_summary(args):
                                                                       "frac_mfma": round(r["TFLOPs"] / PEAK_FP8_TFLOPS, 4)})
             continue
         m = r["M"]
-        hbm_bound = m <= 128
+        hbm_bound = r["gemm_frac_hbm"] >= r["gemm_frac_mfma"]
         e = {"M": m, "N": r["N"], "K": r["K"], "quant_us": r["quant_us"], "gemm_us": r["gemm_us"],
              "bound": "hbm" if hbm_bound else "mfma",
              "frac": r["gemm_frac_hbm"] if hbm_bound else r["gemm_frac_mfma"]}
