@@ -82,7 +82,8 @@ class BenchKernels:
     loop, the clock probe and the streaming passes.  Measurement helpers only; the operators never load it."""
 
     VARIANTS = {0: "16x16x128 accumulate in place", 1: "16x16x128 from zero + fold FMAs (block-scaled kind)",
-                2: "32x32x64 accumulate in place", 3: "32x32x64 pairs from zero + fold FMAs"}
+                2: "32x32x64 accumulate in place", 3: "32x32x64 pairs from zero + fold FMAs",
+                4: "16x16x128 with per-lane exponent bytes for both operands, accumulate in place (power-of-two block scales)"}
 
     def __init__(self, dev):
         import ctypes
@@ -179,25 +180,34 @@ def run_launches(args):
     import torch
 
     from sglang_amd import _lib
-    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.quantization.fp8_kernel import per_token_group_quant_fp8_pow2, sglang_per_token_group_quant_fp8
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_ue8m0
 
     lib = _lib.load()
     dev = torch.device("cuda:0")
     if args.calibrate_copy:
         calibrate_copy(dev)
+    if args.ue8m0:
+        quant = lambda x: per_token_group_quant_fp8_pow2(x, 128, column_major_scales=True)
+        gemm = fp8_blockwise_scaled_mm_ue8m0
+    else:
+        quant = lambda x: sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+        gemm = fp8_blockwise_scaled_mm
     rows = []
     for i, spec in enumerate(args.launches.split(";")):
         m, n, k = (int(v) for v in spec.split(","))
         wq, ws = make_block_weight(n, k, 7000 + i, dev)
+        if args.ue8m0:
+            ws = torch.exp2(torch.ceil(torch.log2(ws)))
         x = make_activation(m, k, 7100 + i, dev)
-        xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
-        fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+        xq, xs = quant(x)
+        gemm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
         torch.cuda.synchronize()
         t = Timer()
         for _ in range(args.launch_reps):
-            xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
-            t.time(lambda: fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+            xq, xs = quant(x)
+            t.time(lambda: gemm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
         torch.cuda.synchronize()
         us = t.total_ms() / t.count() * 1e3
         rows.append({"M": m, "N": n, "K": k, "kernel": lib.sglq_debug_last_gemm_kernel().decode(), "gemm_us": round(us, 2),
@@ -218,7 +228,7 @@ def run_ceiling(args):
            "published_peak_TFLOPs": PEAK_FP8_TFLOPS, "cus": bk.cus, "runs": []}
     for kind in ("random", "small_integers"):
         ops = bk.operands(kind)
-        for v in range(4):
+        for v in range(5):
             r = bk.mfma_ceiling(v, ops)
             r["operands"] = kind
             r["frac_of_published_peak"] = round(r["TFLOPs"] / PEAK_FP8_TFLOPS, 3)
@@ -277,6 +287,82 @@ def cpu_baseline(m_sample):
         "cores": cores,
         "kind": "port",
         "sample": f"{m_sample} of 4096 activation rows of each of the 5 shapes, full weights, {PASSES} passes, {secs:.1f} s of CPU time",
+    }
+
+
+def ue8m0_summary(args, layers, m, bk, ops_rand):
+    """The headline step once more with power-of-two (UE8M0) scales: per_token_group_quant_fp8_pow2 and
+    fp8_blockwise_scaled_mm_ue8m0, whose matrix instructions apply the scales and accumulate in place (the reference's
+    deepgemm_w8a8_block_fp8_linear_with_fallback under DEEPGEMM_SCALE_UE8M0).  Reported next to the headline, which
+    stays the fp32-scale operator; same shapes, same timing method (wall clock over the timed steps, then a pass with
+    events per launch)."""
+    import torch
+
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import per_token_group_quant_fp8_pow2
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_ue8m0
+
+    lib = _lib.load()
+    ws2 = [torch.exp2(torch.ceil(torch.log2(ws))) for (_, _, _, _, ws) in layers]
+    hw = {}
+
+    def step(tq=None, tg=None):
+        for li, (n, k, x, wq, _) in enumerate(layers):
+            if tq is None:
+                xq, xs = per_token_group_quant_fp8_pow2(x, 128, column_major_scales=True)
+                fp8_blockwise_scaled_mm_ue8m0(xq, wq.t(), xs, ws2[li].t(), torch.bfloat16)
+            else:
+                xq, xs = tq[li].time(lambda: per_token_group_quant_fp8_pow2(x, 128, column_major_scales=True))
+                tg[li].time(lambda: fp8_blockwise_scaled_mm_ue8m0(xq, wq.t(), xs, ws2[li].t(), torch.bfloat16))
+                hw[li] = (lib.sglq_debug_last_gemm_kernel().decode(), bool(lib.sglq_debug_last_gemm_hw_scaled()))
+
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.05:  # (the clocks are settled by the headline's steps; a few more to switch kernels)
+        step()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    tq, tg = [Timer() for _ in layers], [Timer() for _ in layers]
+    for _ in range(args.steps):
+        step(tq, tg)
+    torch.cuda.synchronize()
+    flops_step = sum(2.0 * m * n * k for n, k, *_ in layers)
+    ms_per_step = wall * 1e3 / args.steps
+    per_shape = []
+    for li, ((n, k, *_), a, b) in enumerate(zip(layers, tq, tg)):
+        qm, gm = a.total_ms() / args.steps, b.total_ms() / args.steps
+        per_shape.append({"N": n, "K": k, "gemm_kernel": hw[li][0], "scales_applied_by_the_mfma": hw[li][1],
+                          "quant_us": round(qm * 1e3, 1), "quant_GBs": round(group_quant_bytes(m, k) / qm / 1e6, 1),
+                          "gemm_us": round(gm * 1e3, 1), "gemm_TFLOPs": round(2.0 * m * n * k / gm / 1e9, 1),
+                          "gemm_frac": round(2.0 * m * n * k / gm / 1e9 / PEAK_FP8_TFLOPS, 4)})
+    dom = max(range(len(layers)), key=lambda i: tg[i].total_ms())
+    dom_tflops = per_shape[dom]["gemm_TFLOPs"]
+    gemm_ms = sum(t.total_ms() for t in tg) / args.steps
+    ceil = bk.mfma_ceiling(4, ops_rand, iters=10000)
+    return {
+        "what": "the same step with power-of-two (UE8M0) scales: per_token_group_quant_fp8_pow2 + fp8_blockwise_scaled_mm_ue8m0, "
+                "the MFMAs apply the scales (v_mfma_scale_f32_16x16x128_f8f6f4) and accumulate in place; weights' block scales "
+                "rounded up to powers of two, values synthetic",
+        "value": round(flops_step / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "roofline": {"kernel": f"fp8_blockwise_scaled_mm_ue8m0: sglq::{per_shape[dom]['gemm_kernel']} on {m} x {layers[dom][0]} x {layers[dom][1]}",
+                     "bound": "mfma", "achieved": dom_tflops, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(dom_tflops / PEAK_FP8_TFLOPS, 4),
+                     "avg_launch_ms": round(tg[dom].total_ms() / tg[dom].count(), 4),
+                     "practical_peak": {"value": ceil["TFLOPs"], "clock_mhz": ceil["clock_mhz"],
+                                        "mfma_pipe_utilisation": ceil["mfma_pipe_utilisation"],
+                                        "what": "register-only loop of the scaled MFMA accumulating in place, N(0,1) e4m3 operands",
+                                        "frac_of_it": round(dom_tflops / ceil["TFLOPs"], 4)},
+                     "all_gemm_launches_of_the_step": {"achieved": round(flops_step / (gemm_ms * 1e-3) / 1e12, 2),
+                                                       "frac": round(flops_step / (gemm_ms * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}},
+        "per_shape": per_shape,
     }
 
 
@@ -488,6 +574,7 @@ def run_headline(args):
                                "counter, sampled per compute unit on the launch stream before and after them (median over the CUs)",
                    "nominal_clock_mhz": getattr(props, "clock_rate", 0) // 1000},
     }
+    out["ue8m0_scales"] = ue8m0_summary(args, layers, m, bk, ops_rand)
     if not args.no_configs:
         out["configs"] = config_summary(args)
     if not args.no_cpu:
@@ -785,6 +872,8 @@ def main():
     ap.add_argument("--launches", type=str, default=None,
                     help='"M,N,K;M,N,K;...": run these block-FP8 linears as plain launches in this order and exit (for profiler counter runs)')
     ap.add_argument("--launch-reps", type=int, default=5)
+    ap.add_argument("--ue8m0", action="store_true",
+                    help="with --launches: power-of-two scales (per_token_group_quant_fp8_pow2 + fp8_blockwise_scaled_mm_ue8m0)")
     ap.add_argument("--ceiling", action="store_true", help="only measure the MFMA pipe's sustained rate (register-only loop) and exit")
     ap.add_argument("--graph", action="store_true", help="also time the K steps replayed as one HIP graph (graph_ms_per_step)")
     ap.add_argument("--prewarm-ms", type=float, default=150.0, help="untimed steps for this long before the warm-up steps")

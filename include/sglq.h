@@ -61,6 +61,16 @@ int sglq_per_token_group_quant_fp8_ue8m0(const void* input, int in_dtype, void* 
                                          int64_t num_tokens, int64_t hidden, int64_t s_stride_col, float eps,
                                          float fp8_min, float fp8_max, void* stream);
 
+/* sglq_per_token_group_quant_fp8_ue8m0's scales as fp32 instead of packed exponent bytes: the scale of a
+ * group of 128 is the smallest power of two >= max(amax / fp8_max, 1e-10) (per_token_group_quant_8bit.cu:86-89),
+ * stored like sglq_per_token_group_quant_fp8 stores its scales (element (row, g) at
+ * output_s[row*s_stride_row + g*s_stride_col]); the codes are the same bytes as that entry point's.  It feeds
+ * sglq_fp8_blockwise_scaled_mm_ue8m0 in the place of the quantization call of
+ * deepgemm_w8a8_block_fp8_linear_with_fallback (python/sglang/srt/layers/quantization/fp8_utils.py:240-246). */
+int sglq_per_token_group_quant_fp8_pow2(const void* input, int in_dtype, void* output_q, float* output_s,
+                                        int64_t num_tokens, int64_t hidden, int64_t s_stride_row, int64_t s_stride_col,
+                                        float eps, float fp8_min, float fp8_max, void* stream);
+
 /* Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_int8
  * (per_token_group_quant_8bit.cu:219-228; schema common_extension.cc:121-124):
  * same arithmetic with an int8 destination, the float-to-int8 cast truncating
@@ -131,6 +141,22 @@ int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int6
                                  int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                  int64_t workspace_bytes, void* stream);
+
+/* sglq_fp8_blockwise_scaled_mm for scales that are all powers of two (UE8M0 values held as fp32: what
+ * ceil_to_ue8m0 produces, python/sglang/srt/layers/quantization/fp8_utils.py:485-486).  It stands in for the
+ * DeepGEMM call of the reference's w8a8_block_fp8_matmul_deepgemm (fp8_kernel.py; a third-party kernel there),
+ * whose caller deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:214-258) quantizes with such scales.
+ * Same arguments, layouts and checks as sglq_fp8_blockwise_scaled_mm, same result for such scales.  For bf16
+ * outputs on the shapes of the 256- and 128-row pipelined kernels (roughly M > 128) the matrix instruction
+ * applies the scales itself (v_mfma_scale_f32_16x16x128_f8f6f4 takes one exponent byte per lane and operand)
+ * and accumulates in place; only the exponent bits of the scales are read there, so a scale that is not a
+ * power of two is silently rounded down to one: the caller guarantees the property (it is not checked: the
+ * scales are device data).  Every other shape runs exactly as sglq_fp8_blockwise_scaled_mm. */
+int sglq_fp8_blockwise_scaled_mm_ue8m0(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                       int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                       int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                       int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                       int64_t workspace_bytes, void* stream);
 
 /* sglq_fp8_blockwise_scaled_mm fused with the bias add that its caller performs on the
  * result (python/sglang/srt/layers/quantization/fp8_utils.py:207-211: the GEMM, then
@@ -349,6 +375,9 @@ void sglq_debug_grouped_tile(int rows);
 /* Test and measurement hook: name of the GEMM kernel that the calling thread's last GEMM
  * call launched ("" before the first call); the string is static. */
 const char* sglq_debug_last_gemm_kernel(void);
+/* 1 if the calling thread's last block-scaled FP8 GEMM ran on the kernels whose MFMAs apply the scales
+ * (sglq_fp8_blockwise_scaled_mm_ue8m0 on the shapes they are built for), else 0. */
+int sglq_debug_last_gemm_hw_scaled(void);
 
 #ifdef __cplusplus
 }

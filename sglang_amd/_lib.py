@@ -28,10 +28,13 @@ SIGNATURES = {
     "sglq_per_token_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_token_quant_int8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_per_token_group_quant_fp8_ue8m0": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_void_p],
+    "sglq_per_token_group_quant_fp8_pow2": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_void_p],
     "sglq_per_tensor_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p],
     "sglq_static_quant_fp8": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                      c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
+    "sglq_fp8_blockwise_scaled_mm_ue8m0": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                           c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_noalloc": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                              c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
     "sglq_init": [],
@@ -92,6 +95,8 @@ def load() -> ctypes.CDLL:
     lib.sglq_debug_grouped_tile.restype = None
     lib.sglq_debug_last_gemm_kernel.argtypes = []
     lib.sglq_debug_last_gemm_kernel.restype = ctypes.c_char_p
+    lib.sglq_debug_last_gemm_hw_scaled.argtypes = []
+    lib.sglq_debug_last_gemm_hw_scaled.restype = ctypes.c_int
     _lib = lib
     if os.environ.get("SGLQ_NO_TUNED_CONFIGS", "0") != "1":
         # per-(N, K) kernel selections shipped beside the package (sglang_amd/quantization/configs/)

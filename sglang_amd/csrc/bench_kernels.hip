@@ -22,6 +22,7 @@ constexpr int ACCUMULATE_16 = 0;  // 16x16x128, accumulating in place (per-row/p
 constexpr int FOLD_16 = 1;        // 16x16x128 from a zero accumulator, result folded in with 4 FMAs (block-scaled kind)
 constexpr int ACCUMULATE_32 = 2;  // 32x32x64, accumulating in place
 constexpr int FOLD_32 = 3;        // 32x32x64 in pairs (one 128-byte K block), the pair's result folded in with 16 FMAs
+constexpr int SCALED_16 = 4;      // 16x16x128 with an exponent byte per lane for each operand, accumulating in place (power-of-two block scales)
 
 struct ClockSample {
   uint64_t shader_cycles, realtime_ticks;
@@ -47,7 +48,10 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(const v8i* __restrict
   const float scale = 1.0f + 1e-6f * (float)lane;
 
   ClockSample t0 = read_clocks();
-  if constexpr (VARIANT == ACCUMULATE_16 || VARIANT == FOLD_16) {
+  if constexpr (VARIANT == ACCUMULATE_16 || VARIANT == FOLD_16 || VARIANT == SCALED_16) {
+    int sa[8], sb = 125 + (iters & 1);  // exponent bytes near 127 (2^0), per fragment as in the kernels
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sa[i] = 124 + ((lane + i) & 7);
     v4f acc[8][4];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -60,10 +64,13 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(const v8i* __restrict
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         asm volatile("" : "+v"(a[i & 1]));  // a new activation fragment as far as the compiler knows
+        if constexpr (VARIANT == SCALED_16) asm volatile("" : "+v"(sa[i]), "+v"(sb));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if constexpr (VARIANT == ACCUMULATE_16) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], a[i & 1], acc[i][j], 0, 0, 0, 0, 0, 0);
+          } else if constexpr (VARIANT == SCALED_16) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], a[i & 1], acc[i][j], 0, 0, 0, sb, 0, sa[i]);
           } else {
             const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], a[i & 1], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
             const int idx = i * 4 + j;
@@ -194,6 +201,7 @@ int sglqb_mfma_ceiling(int variant, int iters, const void* operands, float* sink
     case FOLD_16: mfma_ceiling_kernel<FOLD_16><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
     case ACCUMULATE_32: mfma_ceiling_kernel<ACCUMULATE_32><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
     case FOLD_32: mfma_ceiling_kernel<FOLD_32><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
+    case SCALED_16: mfma_ceiling_kernel<SCALED_16><<<blocks, 512, 0, st>>>(ops, iters, sink, clocks); break;
     default: return -1;
   }
   return (int)hipGetLastError();

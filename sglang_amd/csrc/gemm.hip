@@ -34,9 +34,16 @@ constexpr int KIND_FP8_ROWCOL = 1;  // a6: sa[m] * (sb[n] * acc) + bias[n]
 constexpr int KIND_I8_ROWCOL = 2;   // a5: float(acc) * (sb[n] * sa[m]) + bias[n]
 constexpr int KIND_I8_RAW = 3;      // INT32 accumulators
 constexpr int KIND_I8_BLOCK = 4;    // block-scaled INT8: sum_kb float(P_kb) * sfa[m,kb] * sfb[kb,n/128]
+// KIND_FP8_BLOCK whose scales are all powers of two (UE8M0 values held as fp32): the MFMA applies them itself
+// (v_mfma_scale_f32_16x16x128_f8f6f4 takes an exponent byte per lane for each operand) and accumulates in place,
+// so there is no scale-and-accumulate pass behind every MFMA.  Only the 256- and 128-row pipelined kernels are
+// built for it; everywhere else such scales run as KIND_FP8_BLOCK, with the same result.
+constexpr int KIND_FP8_BLOCK_POW2 = 5;
 
-constexpr bool is_block(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_I8_BLOCK; }
-constexpr bool fp8_operands(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_FP8_ROWCOL; }
+constexpr bool is_block(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_I8_BLOCK || kind == KIND_FP8_BLOCK_POW2; }
+constexpr bool fp8_operands(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_FP8_ROWCOL || kind == KIND_FP8_BLOCK_POW2; }
+// the biased exponent of a positive power of two = its UE8M0 code, in byte 0 as the scaled MFMA reads it
+SGLQ_DEV int ue8m0_of(float pow2) { return (int)(__builtin_bit_cast(uint32_t, pow2) >> 23); }
 constexpr bool float_acc(int kind) { return fp8_operands(kind) || kind == KIND_I8_BLOCK; }
 
 constexpr uint32_t OOB = 0x80000000u;  // offset beyond any buffer this library accepts
@@ -61,6 +68,7 @@ struct GemmArgs {
   int64_t b_expert_stride, sb_expert_stride;  // grouped GEMM: bytes / floats between experts' weights / weight scales
   int num_experts;
   int stream_out;  // the output is larger than the last-level cache: store it with the non-temporal hint
+  int pow2_scales;  // block-scaled FP8: every scale is a power of two (KIND_FP8_BLOCK_POW2 where it is built)
   float quant_eps;  // fused quantization (gemm_stream_quant_kernel): lower bound of a group's abs-max
 };
 
@@ -910,6 +918,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr int NCOPY_A = BM / 64;  // activation copies per wave per stage
   constexpr bool IS_FP8 = fp8_operands(KIND);
   constexpr bool BLOCK = is_block(KIND);
+  constexpr bool HW = KIND == KIND_FP8_BLOCK_POW2;  // the MFMA applies the block scales
+  constexpr bool FOLD = BLOCK && !HW;               // they are applied to each MFMA's result
   static_assert(NI == 4 && (MI == 8 || MI == 4), "the copy schedule below is written for 4 x 8 or 4 x 4 fragments");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
@@ -1037,14 +1047,17 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
     v4f part_prev = {0.f, 0.f, 0.f, 0.f};
+    int ea = 0;                                 // HW: exponent byte of the fragment's activation scale (per lane: its row)
+    const int eb = HW ? ue8m0_of(sfb_cur) : 0;  // ... and of the block's weight scale
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       v8i a_nxt = a_cur;
-      if constexpr (BLOCK) {
+      if constexpr (FOLD) {
         sc_prev = sc;
         sc = sfa_cur[i] * sfb_cur;
       }
+      if constexpr (HW) ea = ue8m0_of(sfa_cur[i]);
       if (i == 1 && !last) {
         // barrier 1: MFMAs 0..3 have consumed this wave's weight fragments, so its LDS reads
         // of block u's weights are complete; behind the barrier that holds for every wave.
@@ -1068,8 +1081,11 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       for (int j = 0; j < NI; ++j) {
         const int idx = i * NI + j;
         v4f part = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (BLOCK) {
+        if constexpr (FOLD) {
           part = block_mfma<KIND>(bf[j], a_cur);
+        } else if constexpr (HW) {
+          const v4f c0 = first ? v4f{0.f, 0.f, 0.f, 0.f} : acc[i][j];
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], a_cur, c0, 0, 0, 0, eb, 0, ea);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           // (a tile's first step starts from zero instead of clearing 128 registers beforehand)
           const v4f c0 = first ? v4f{0.f, 0.f, 0.f, 0.f} : acc[i][j];
@@ -1099,7 +1115,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
             if (j < NCOPY_A) copy_a(j, cur, kn2 * 128, off_a2);
             if constexpr (BLOCK) {
               // scales i < MI - 1 had their last use when the last fragment's scale was formed; its own
-              // scale and sfb_cur are dead as well: `sc` holds their product
+              // scale and sfb_cur are dead as well: `sc` holds their product (HW: `ea` and `eb` their exponents)
 #pragma unroll
               for (int q = 0; q < MI / NI; ++q) sfa_cur[(MI / NI) * j + q] = read_sfa(cur ^ 1, (MI / NI) * j + q);
               if (j == 0) sfb_cur = read_sfb(cur ^ 1);
@@ -1115,7 +1131,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         } else if constexpr (!last) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2, true);
         }
-        if constexpr (BLOCK) {
+        if constexpr (FOLD) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pi = (idx - 1) / NI, pj = (idx - 1) % NI;
             const float s_use = (pi == i) ? sc : sc_prev;
@@ -1130,7 +1146,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
       }
       a_cur = a_nxt;
     }
-    if constexpr (BLOCK) {
+    if constexpr (FOLD) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         acc[MI - 1][NI - 1][e] = first ? block_value<KIND>(part_prev[e]) * sc
@@ -1278,6 +1294,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   constexpr int NBW = (NB + NW - 1) / NW; // ... per wave (the last one only for waves < NB % 8)
   constexpr bool IS_FP8 = fp8_operands(KIND);
   constexpr bool BLOCK = is_block(KIND);
+  constexpr bool HW = KIND == KIND_FP8_BLOCK_POW2;  // the MFMA applies the block scales
+  constexpr bool FOLD = BLOCK && !HW;               // they are applied to each MFMA's result
   static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
@@ -1413,16 +1431,27 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
     float scv[MI] = {0.f, 0.f, 0.f, 0.f};  // sfa[i] * sfb of the scale block of the fragments being multiplied
-    if constexpr (BLOCK) {
+    if constexpr (FOLD) {
 #pragma unroll
       for (int i = 0; i < MI; ++i) scv[i] = sfa_cur[i] * sfb_lo;
+    }
+    // HW: the exponent bytes of the fragments' activation scales (per lane: its row) and of the two weight scales
+    // (HW runs one instantiation of the step for every position of the boundary, JSW = NI, and selects per
+    // fragment at run time: instantiated per position like the other block kinds, the accumulators change
+    // registers between the instantiations and the kernel spills)
+    int ea[MI] = {0, 0, 0, 0};
+    const int eb_lo = HW ? ue8m0_of(sfb_lo) : 0, eb_hi = HW ? ue8m0_of(sfb_hi) : 0;
+    const int jsw_now = jsw;
+    if constexpr (HW) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) ea[i] = ue8m0_of(sfa_cur[i]);
     }
     v4f part_prev = {0.f, 0.f, 0.f, 0.f};
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       v8i b_nxt = b_cur;
-      if constexpr (BLOCK) {
+      if constexpr (FOLD) {
         if (j == JSW) {  // (compile-time: no branch) the fragments from here on lie in the next scale block
 #pragma unroll
           for (int i = 0; i < MI; ++i) scv[i] = sfa_cur[i] * sfb_hi;
@@ -1450,8 +1479,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       for (int i = 0; i < MI; ++i) {
         const int idx = j * MI + i;
         v4f part = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (BLOCK) {
+        if constexpr (FOLD) {
           part = block_mfma<KIND>(b_cur, af[i]);
+        } else if constexpr (HW) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, j < jsw_now ? eb_lo : eb_hi, 0, ea[i]);
         } else if constexpr (KIND == KIND_FP8_ROWCOL) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_cur, af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
@@ -1466,7 +1497,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, a1, acc[i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (BLOCK) {
+        if constexpr (FOLD) {
           sc_prev = sc;
           sc = scv[i];
         }
@@ -1493,7 +1524,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         } else if constexpr (!last) {
           if (idx >= 4 && idx < 8) copy_a(idx - 4, cur, kn2 * 128, off_a2);
         }
-        if constexpr (BLOCK) {
+        if constexpr (FOLD) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
             const int pj = (idx - 1) / MI, pi = (idx - 1) % MI;
             acc[pi][pj][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc_prev, acc[pi][pj][0]);
@@ -1507,13 +1538,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       }
       b_cur = b_nxt;
     }
-    if constexpr (BLOCK) {
+    if constexpr (FOLD) {
       acc[MI - 1][NI - 1][0] = __builtin_fmaf(block_value<KIND>(part_prev[0]), sc, acc[MI - 1][NI - 1][0]);
       acc[MI - 1][NI - 1][1] = __builtin_fmaf(block_value<KIND>(part_prev[1]), sc, acc[MI - 1][NI - 1][1]);
       acc[MI - 1][NI - 1][2] = __builtin_fmaf(block_value<KIND>(part_prev[2]), sc, acc[MI - 1][NI - 1][2]);
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
-      jsw = jsw_nxt;
     }
+    if constexpr (BLOCK) jsw = jsw_nxt;
   };
 
   // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
@@ -1582,7 +1613,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       if constexpr (BLOCK) set_scale_split(nn0);
       k_step(last_stage, 0, 0, std::false_type{}, std::true_type{}, jsw_tag);
     };
-    if constexpr (!BLOCK || NI == 8) {
+    if constexpr (!BLOCK || NI == 8 || HW) {
       tile_steps(std::integral_constant<int, NI>{});  // (256-wide tiles: a wave's 128 columns are one scale block)
     } else if constexpr (NI == 6) {
       // 192-wide tiles start at multiples of 64 columns: the boundary is behind fragment 2, 4 or 6 (= none)
@@ -2258,6 +2289,7 @@ static thread_local int g_force_splits = 0;  // test hook: > 0 fixes the split-K
 static thread_local int t_tile = 0, t_splits = 0;
 static thread_local int g_grouped_tile = 0;  // test hook: 32 / 64 / 128 / 256 fixes the grouped GEMM's row tile, 130 = 128 rows pipelined (0 = from the average group)
 static thread_local const char* g_last_kernel = "";  // which GEMM kernel the calling thread's last call launched
+static thread_local bool g_last_hw_scaled = false;   // ... and whether its MFMAs applied the block scales (KIND_FP8_BLOCK_POW2)
 
 template <int KIND, int OUT_DT>
 static void launch_reduce(GemmArgs& p, hipStream_t st);
@@ -2358,6 +2390,15 @@ static thread_local int g_force_tile = 0;
 
 static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws_bytes, int& splits);
 
+// Whether this launch takes the kernels whose MFMAs apply the block scales (built for bf16 outputs without a
+// fused bias, what the reference's call of that GEMM produces: fp8_utils.py:225-258).
+template <int KIND, int OUT_DT>
+static bool hw_scaled(const GemmArgs& p) {
+  const bool hw = KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16 && p.pow2_scales && !p.bias;
+  if (hw) g_last_hw_scaled = true;
+  return hw;
+}
+
 template <int KIND, int OUT_DT>
 static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.tiles_m = (p.M + 255) / 256;
@@ -2393,10 +2434,16 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     g_last_kernel = splits > 1 ? "gemm_pipe_kernel+splitk_reduce_kernel" : "gemm_pipe_kernel";
     const dim3 grid((uint32_t)blocks), block(512);
     if (splits > 1) {
-      gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK><<<grid, block, 0, st>>>(p);
+      if (hw_scaled<KIND, OUT_DT>(p)) {
+        if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_SPLITK><<<grid, block, 0, st>>>(p);
+      } else {
+        gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK><<<grid, block, 0, st>>>(p);
+      }
       launch_reduce<KIND, OUT_DT>(p, st);  // (adds the bias)
     } else if (is_block(KIND) && p.bias) {
       if constexpr (is_block(KIND)) gemm_pipe_kernel<KIND, OUT_DT, PIPE_BIAS><<<grid, block, 0, st>>>(p);
+    } else if (hw_scaled<KIND, OUT_DT>(p)) {
+      if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
     } else {
       gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
     }
@@ -2464,10 +2511,16 @@ static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const dim3 grid((uint32_t)(units < num_cus() ? units : num_cus())), block(512);
   g_last_kernel = splits > 1 ? "gemm_pipe_kernel<128 rows>+splitk_reduce_kernel" : "gemm_pipe_kernel<128 rows>";
   if (splits > 1) {
-    gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK, 128><<<grid, block, 0, st>>>(p);
+    if (hw_scaled<KIND, OUT_DT>(p)) {
+      if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_SPLITK, 128><<<grid, block, 0, st>>>(p);
+    } else {
+      gemm_pipe_kernel<KIND, OUT_DT, PIPE_SPLITK, 128><<<grid, block, 0, st>>>(p);
+    }
     launch_reduce<KIND, OUT_DT>(p, st);  // (adds the bias)
   } else if (is_block(KIND) && p.bias) {
     if constexpr (is_block(KIND)) gemm_pipe_kernel<KIND, OUT_DT, PIPE_BIAS, 128><<<grid, block, 0, st>>>(p);
+  } else if (hw_scaled<KIND, OUT_DT>(p)) {
+    if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_PLAIN, 128><<<grid, block, 0, st>>>(p);
   } else {
     gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN, 128><<<grid, block, 0, st>>>(p);
   }
@@ -2483,6 +2536,8 @@ static void launch_wide(GemmArgs& p, hipStream_t st) {
   g_last_kernel = NI == 6 ? "gemm_wide_kernel<6>" : NI == 7 ? "gemm_wide_kernel<7>" : "gemm_wide_kernel<8>";
   if (is_block(KIND) && p.bias) {
     if constexpr (is_block(KIND)) gemm_wide_kernel<KIND, OUT_DT, NI, true><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
+  } else if (hw_scaled<KIND, OUT_DT>(p)) {
+    if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_wide_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, NI, false><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
   } else {
     gemm_wide_kernel<KIND, OUT_DT, NI, false><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
   }
@@ -2879,12 +2934,13 @@ extern "C" void sglq_debug_grouped_tile(int rows) {
   g_grouped_tile = (rows == 32 || rows == 64 || rows == 128 || rows == 130 || rows == 256) ? rows : 0;
 }
 extern "C" const char* sglq_debug_last_gemm_kernel(void) { return g_last_kernel; }
+extern "C" int sglq_debug_last_gemm_hw_scaled(void) { return g_last_hw_scaled ? 1 : 0; }
 
 template <int KIND>
 static int blockwise_entry(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb, int64_t sfb_stride_k,
                            int64_t sfb_stride_n, const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M,
-                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream, bool pow2_scales = false) {
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
@@ -2906,6 +2962,8 @@ static int blockwise_entry(const char* name, const void* a, int64_t lda, const v
   p.sb_stride_k = sfb_stride_k;
   p.sb_stride_n = sfb_stride_n;
   p.ws = workspace;
+  p.pow2_scales = pow2_scales ? 1 : 0;
+  g_last_hw_scaled = false;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (out_dtype == SGLQ_BF16) launch_kind<KIND, SGLQ_BF16>(p, workspace_bytes, st);
   else launch_kind<KIND, SGLQ_FP16>(p, workspace_bytes, st);
@@ -2920,6 +2978,16 @@ extern "C" int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const vo
   return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
                                          sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N, K, workspace,
                                          workspace_bytes, stream);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_mm_ue8m0(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
+                                                  int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb,
+                                                  int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                                  int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm_ue8m0", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
+                                         sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N, K, workspace,
+                                         workspace_bytes, stream, true);
 }
 
 extern "C" int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,

@@ -24,7 +24,10 @@ namespace sglq {
 // the quotient by 448 * (1 + 2^-22), which rounds to the code of 448 anyway, so
 // the explicit clamp is dropped.  The quotient's sign is copied from x so that
 // -0.0 stays -0.0 (the remainder correction would turn it into +0.0).
-template <int DT, int GROUP, int NCH, int UNROLL, bool STRIDED_SCALE, bool TO_INT8, bool CLAMP, bool STREAM_IN = false>
+// POW2: the scale is the smallest power of two >= max(amax / qmax, 1e-10) (the UE8M0 rule of
+// per_token_group_quant_8bit.cu:86-89, see group_quant_ue8m0_kernel), stored as fp32; the codes are
+// x times its exact inverse, clamped as that kernel clamps them.
+template <int DT, int GROUP, int NCH, int UNROLL, bool STRIDED_SCALE, bool TO_INT8, bool CLAMP, bool STREAM_IN = false, bool POW2 = false>
 __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict__ x, char* __restrict__ q,
                                                           float* __restrict__ s, uint32_t num_groups,
                                                           FastDiv groups_per_row, int64_t s_stride_row,
@@ -63,15 +66,24 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const char* __restrict
       for (int c = 1; c < NCH; ++c) mb = umax(mb, ch[u][c].amax_bits());
       mb = group_umax<LPG>(mb);
       const float amax = u2f(umax(mb, f2u(eps)));
-      const float y_s = div_by(amax, qmax, rqmax);
-      const float r = 1.0f / y_s;
+      float y_s = div_by(amax, qmax, rqmax);
+      float r = 1.0f / y_s;
+      if constexpr (POW2) {
+        const uint32_t bits = f2u(__builtin_fmaxf(y_s, 1e-10f));  // positive and normal
+        const uint32_t biased = (bits >> 23) + ((bits & 0x7fffffu) != 0 ? 1u : 0u);
+        y_s = u2f(biased << 23);
+        r = u2f((254u - biased) << 23);  // exact
+      }
       char* qp = q + (int64_t)gid * GROUP + sub * 8;
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         float v[8];
         v2u o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = quantize_elem<CLAMP>(ch[u][c].get(i), y_s, r, qmin, qmax);
+        for (int i = 0; i < 8; ++i) {
+          if constexpr (POW2) v[i] = __builtin_fminf(__builtin_fmaxf(ch[u][c].get(i) * r, qmin), qmax);
+          else v[i] = quantize_elem<CLAMP>(ch[u][c].get(i), y_s, r, qmin, qmax);
+        }
         if constexpr (TO_INT8) o = I8Pack::pack(v); else o = Fp8Pack::pack(v);
         *reinterpret_cast<v2u*>(qp + c * (GROUP / NCH)) = o;
       }
@@ -576,6 +588,68 @@ static int group_quant_entry(const char* name, const void* input, int in_dtype, 
   return SGLQ_EUNSUPPORTED;
 }
 
+// sgl_per_token_group_quant_fp8 with power-of-two scales stored as fp32 (group 128): group_quant_kernel<POW2>.
+template <int DT>
+static void launch_group_quant_pow2(const void* x, void* q, float* s, uint32_t num_groups, uint32_t gpr, bool strided, int64_t sr,
+                                    int64_t sc, float eps, float qmin, float qmax, hipStream_t st) {
+  constexpr int GROUP = 128, NCH = 2, GPB = 256 / (GROUP / (8 * NCH));
+  FastDiv fd;
+  fd.init(gpr);
+  const float rq = 1.0f / qmax;
+  const char* xi = static_cast<const char*>(x);
+  char* qo = static_cast<char*>(q);
+  const bool stream_in = (int64_t)num_groups * GROUP * elem_bytes<DT>() >= ((int64_t)128 << 20);  // (as launch_group_quant)
+  const dim3 grid((num_groups + GPB - 1) / GPB), block(256);
+#define SGLQ_LAUNCH_P2(STR, ONCE) \
+  group_quant_kernel<DT, GROUP, NCH, 1, STR, false, false, ONCE, true><<<grid, block, 0, st>>>(xi, qo, s, num_groups, fd, sr, sc, eps, qmin, qmax, rq)
+  if (stream_in) {
+    if (strided) SGLQ_LAUNCH_P2(true, true); else SGLQ_LAUNCH_P2(false, true);
+  } else {
+    if (strided) SGLQ_LAUNCH_P2(true, false); else SGLQ_LAUNCH_P2(false, false);
+  }
+#undef SGLQ_LAUNCH_P2
+}
+
+static int group_quant_pow2_entry(const void* input, int in_dtype, void* output_q, float* output_s, int64_t num_tokens,
+                                  int64_t hidden, int64_t sr, int64_t sc, float eps, float qmin, float qmax, void* stream) {
+  const char* name = "sgl_per_token_group_quant_fp8 (power-of-two fp32 scales)";
+  if (!input || !output_q || !output_s) {
+    if (num_tokens == 0) return SGLQ_OK;
+    set_error("%s: null pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (num_tokens < 0 || hidden <= 0 || hidden % 128 != 0) {
+    set_error("%s: hidden (%lld) must be a positive multiple of 128", name, (long long)hidden);
+    return SGLQ_EINVAL;
+  }
+  if (!(qmax > 0.f) || !(eps > 0.f)) {
+    set_error("%s: eps and the 8-bit maximum must be positive", name);
+    return SGLQ_EINVAL;
+  }
+  if ((reinterpret_cast<uintptr_t>(input) & 15) || (reinterpret_cast<uintptr_t>(output_q) & 7)) {
+    set_error("%s: input must be 16-byte and output_q 8-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  const int64_t gpr = hidden / 128;
+  const int64_t ng = num_tokens * gpr;
+  if (ng == 0) return SGLQ_OK;
+  if (ng >= (1ll << 32) - 65536) {
+    set_error("%s: too many groups (%lld)", name, (long long)ng);
+    return SGLQ_EINVAL;
+  }
+  const bool strided = !(sc == 1 && sr == gpr);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (in_dtype) {
+    case SGLQ_BF16: launch_group_quant_pow2<SGLQ_BF16>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, sc, eps, qmin, qmax, st); break;
+    case SGLQ_FP16: launch_group_quant_pow2<SGLQ_FP16>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, sc, eps, qmin, qmax, st); break;
+    case SGLQ_FP32: launch_group_quant_pow2<SGLQ_FP32>(input, output_q, output_s, (uint32_t)ng, (uint32_t)gpr, strided, sr, sc, eps, qmin, qmax, st); break;
+    default:
+      set_error("%s: unsupported in_dtype %d", name, in_dtype);
+      return SGLQ_EUNSUPPORTED;
+  }
+  return check_launch(name);
+}
+
 static int group_quant_ue8m0_entry(const void* input, int in_dtype, void* output_q, void* output_s, int64_t num_tokens,
                                    int64_t hidden, int64_t s_stride_col, float eps, float qmin, float qmax, void* stream) {
   const char* name = "sgl_per_token_group_quant_fp8 (scale_ue8m0)";
@@ -868,6 +942,13 @@ extern "C" int sglq_per_token_group_quant_fp8_ue8m0(const void* input, int in_dt
                                                     float fp8_min, float fp8_max, void* stream) {
   return sglq::group_quant_ue8m0_entry(input, in_dtype, output_q, output_s, num_tokens, hidden, s_stride_col, eps, fp8_min,
                                        fp8_max, stream);
+}
+
+extern "C" int sglq_per_token_group_quant_fp8_pow2(const void* input, int in_dtype, void* output_q, float* output_s,
+                                                   int64_t num_tokens, int64_t hidden, int64_t s_stride_row, int64_t s_stride_col,
+                                                   float eps, float fp8_min, float fp8_max, void* stream) {
+  return sglq::group_quant_pow2_entry(input, in_dtype, output_q, output_s, num_tokens, hidden, s_stride_row, s_stride_col, eps,
+                                      fp8_min, fp8_max, stream);
 }
 
 extern "C" int sglq_per_token_group_quant_int8(const void* input, int in_dtype, void* output_q, float* output_s,

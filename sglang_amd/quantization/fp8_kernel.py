@@ -204,3 +204,85 @@ def w8a8_block_fp8_matmul(
 
 # the Triton kernel behind it (:870-948) computes the same sums
 w8a8_block_fp8_matmul_triton = w8a8_block_fp8_matmul
+
+
+def per_token_group_quant_fp8_pow2(x: torch.Tensor, group_size: int = 128, eps: float = 1e-10,
+                                   column_major_scales: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """sglang_per_token_group_quant_fp8(..., scale_ue8m0=True) (fp8_kernel.py:344-372) with the scales as fp32
+    instead of four exponent bytes per int32: each group's scale is the smallest power of two >=
+    max(amax / 448, 1e-10), the codes are the same.  The input of w8a8_block_fp8_matmul_deepgemm here."""
+    assert group_size == 128, "power-of-two scales are built for groups of 128"
+    assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
+    assert x.is_contiguous(), "`x` is not contiguous"
+    if not x.is_cuda:
+        raise RuntimeError("per_token_group_quant_fp8_pow2: input must be a CUDA tensor")
+    if x.dtype not in DTYPE_CODE:
+        raise RuntimeError("per_token_group_quant_fp8_pow2: input must be Half, BFloat16 or Float")
+    x_q = torch.empty_like(x, device=x.device, dtype=fp8_dtype)
+    x_s = create_per_token_group_quant_fp8_output_scale(tuple(x.shape), x.device, group_size, column_major_scales, False, False)
+    hidden = x.shape[-1]
+    tokens = x.numel() // hidden
+    if tokens > 0:
+        s2 = x_s.reshape(tokens, hidden // group_size) if x_s.ndim != 2 else x_s
+        rc = _lib.load().sglq_per_token_group_quant_fp8_pow2(
+            x.data_ptr(), DTYPE_CODE[x.dtype], x_q.data_ptr(), s2.data_ptr(), tokens, hidden, s2.stride(0), s2.stride(1),
+            eps, fp8_min, fp8_max, _lib.stream_ptr(x.device))
+        _lib.check(rc, "per_token_group_quant_fp8_pow2")
+    return x_q, x_s
+
+
+def unpack_ue8m0_scales(x_s: torch.Tensor, num_groups: int) -> torch.Tensor:
+    """The fp32 powers of two [M, num_groups] of packed UE8M0 scales [M, ceil(num_groups / 4)] int32 (byte g % 4 of
+    word [row, g / 4] is the biased exponent of group g: per_token_group_quant_8bit.cu:57-64,94)."""
+    assert x_s.dtype == torch.int32 and x_s.ndim == 2
+    shifts = torch.tensor([0, 8, 16, 24], device=x_s.device, dtype=torch.int32)
+    e = (x_s.unsqueeze(-1) >> shifts) & 0xFF
+    return (e.reshape(x_s.shape[0], -1)[:, :num_groups] << 23).contiguous().view(torch.float32)
+
+
+def w8a8_block_fp8_matmul_deepgemm(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    block_size,
+    output_dtype: torch.dtype,
+) -> torch.Tensor:
+    """fp8_kernel.py:849-867: the block-scaled FP8 GEMM for scales that are powers of two, DeepGEMM's
+    gemm_nt_f8f8bf16 in the reference, here sglq_fp8_blockwise_scaled_mm_ue8m0 (the matrix instruction applies
+    the scales and accumulates in place).  A e4m3fn [..., K] contiguous; B e4m3fn [N, K] contiguous; As fp32
+    powers of two [..., K/128] in any layout (per_token_group_quant_fp8_pow2), or the packed int32 form of
+    sglang_per_token_group_quant_fp8(scale_ue8m0=True), which is unpacked first; Bs fp32 powers of two
+    [N/128, K/128] (per_block_cast_to_fp8 / requant_weight_ue8m0_inplace).  bf16 output only, as there (:859-860)."""
+    assert len(block_size) == 2
+    if block_size[0] != 128 or block_size[1] != 128:
+        raise NotImplementedError("w8a8_block_fp8_matmul_deepgemm: only 128 x 128 weight blocks are built")
+    assert output_dtype == torch.bfloat16, "only BFloat16 outputs (fp8_kernel.py:859-860)"
+    assert A.shape[-1] == B.shape[-1]
+    assert A.is_contiguous() and B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
+    N, K = B.shape
+    assert K % 128 == 0, "K must be a multiple of 128 (fp8_utils.py:228)"
+    M = A.numel() // K
+    if not (A.is_cuda and B.is_cuda and As.is_cuda and Bs.is_cuda):
+        raise RuntimeError("w8a8_block_fp8_matmul_deepgemm: tensors must be CUDA tensors")
+    if A.dtype != fp8_dtype or B.dtype != fp8_dtype:
+        raise RuntimeError("w8a8_block_fp8_matmul_deepgemm: A and B must be Float8_e4m3fn")
+    assert -(-N // 128) == Bs.shape[0] and K // 128 == Bs.shape[1]
+    if Bs.dtype != torch.float32:
+        raise NotImplementedError("w8a8_block_fp8_matmul_deepgemm: Bs must be Float32 powers of two [N/128, K/128]")
+    C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
+    if M == 0 or N == 0:
+        return C
+    if As.dtype == torch.int32:
+        As2 = unpack_ue8m0_scales(As.reshape(M, As.shape[-1]), K // 128)
+    elif As.dtype == torch.float32:
+        assert As.shape[-1] == K // 128 and As.numel() == M * (K // 128)
+        As2 = As.reshape(M, K // 128) if As.ndim != 2 else As
+    else:
+        raise NotImplementedError("w8a8_block_fp8_matmul_deepgemm: As must be Float32 or packed Int32")
+    rc = _lib.load().sglq_fp8_blockwise_scaled_mm_ue8m0(
+        A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
+        Bs.data_ptr(), Bs.stride(1), Bs.stride(0), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,
+        *_lib.workspace(A.device), _lib.stream_ptr(A.device))
+    _lib.check(rc, "w8a8_block_fp8_matmul_deepgemm")
+    return C

@@ -3,6 +3,7 @@
 
 from __future__ import annotations
 
+import os
 from typing import List, Optional
 
 import torch
@@ -11,6 +12,8 @@ from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from ..sgl_kernel.gemm import block_fp8_linear, fp8_blockwise_scaled_mm_bias
 from .fp8_kernel import (
     per_token_group_quant_fp8,
+    per_token_group_quant_fp8_pow2,
+    w8a8_block_fp8_matmul_deepgemm,
     scaled_fp8_quant,
     sglang_per_token_quant_fp8,
     static_quant_fp8,
@@ -140,6 +143,13 @@ def apply_fp8_linear(
 cutlass_w8a8_block_fp8_linear_with_fallback = w8a8_block_fp8_linear
 
 
+# The reference's deep_gemm_wrapper.DEEPGEMM_SCALE_UE8M0 (true on the hardware whose DeepGEMM wants power-of-two
+# scales): when set, deepgemm_w8a8_block_fp8_linear_with_fallback quantizes with power-of-two scales and runs the
+# GEMM whose matrix instructions apply them; the weights must then have been through requant_weight_ue8m0_inplace,
+# as the reference's loaders do under that flag.  Off by default (SGLANG_AMD_SCALE_UE8M0=1 or assignment turns it on).
+DEEPGEMM_SCALE_UE8M0 = os.environ.get("SGLANG_AMD_SCALE_UE8M0", "0").lower() in ("1", "true", "yes")
+
+
 def deepgemm_w8a8_block_fp8_linear_with_fallback(
     input: torch.Tensor,
     weight: torch.Tensor,
@@ -148,19 +158,25 @@ def deepgemm_w8a8_block_fp8_linear_with_fallback(
     input_scale: Optional[torch.Tensor] = None,
     bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """The call sequence of deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:215-258):
-    the activation scales are column-major with the row count padded to a multiple of four
-    (`scale_tma_aligned=True`), fp32 (the packed UE8M0 form is the reference's Blackwell-only
-    variant); the GEMM is this library's block-scaled kernel, which takes the scales' strides as
-    they are.  Outputs other than bfloat16 and weights whose N is not a multiple of 64 take the
-    row-major path, as in the reference."""
+    """The call sequence of deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:215-258): column-major
+    activation scales, the GEMM that is DeepGEMM's there, `output += bias`; outputs other than bfloat16 and
+    weights whose N is not a multiple of 64 take the row-major path, as in the reference (:227-234).
+    With DEEPGEMM_SCALE_UE8M0 (:245): power-of-two activation scales (kept as fp32 rather than packed four
+    to an int32: per_token_group_quant_fp8_pow2) and w8a8_block_fp8_matmul_deepgemm, which lets the matrix
+    instructions apply the scales; the weight's block scales must be powers of two (requant_weight_ue8m0_inplace).
+    Without: fp32 scales with the row count padded to a multiple of four (`scale_tma_aligned=True`) and this
+    library's block-scaled kernel, which takes the scales' strides as they are."""
     assert input_scale is None
     if not (input.dtype == torch.bfloat16 and weight.shape[0] % 64 == 0 and weight.shape[1] % 128 == 0):
         return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[0]]
-    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True, scale_tma_aligned=True)
-    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
+    if DEEPGEMM_SCALE_UE8M0:
+        q_input, x_scale = per_token_group_quant_fp8_pow2(input_2d, block_size[1], column_major_scales=True)
+        output = w8a8_block_fp8_matmul_deepgemm(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
+    else:
+        q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True, scale_tma_aligned=True)
+        output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input.dtype)
     if bias is not None:
         output += bias
     return output.to(dtype=input.dtype).view(*output_shape)
@@ -241,6 +257,24 @@ def channel_quant_to_tensor_quant(x_q_channel: torch.Tensor, x_s: torch.Tensor):
 def ceil_to_ue8m0(x: torch.Tensor) -> torch.Tensor:
     """The next power of two at or above abs(x) (fp8_utils.py:485-486)."""
     return torch.pow(2.0, torch.ceil(torch.log2(x.abs())))
+
+
+def _requant_weight_ue8m0(weight: torch.Tensor, weight_scale_inv: torch.Tensor, weight_block_size: List[int]):
+    """fp8_utils.py:432-463 up to the scale layout: the weight dequantized to bf16 and block-quantized again with
+    power-of-two scales.  The scales stay fp32 [N/128, K/128] (the reference goes on to expand and pack them into
+    DeepGEMM's column-major int32 layout, :453-461, which the GEMM here does not use)."""
+    assert list(weight_block_size) == [128, 128]
+    *_, n, k = weight.shape
+    dequant = block_quant_dequant(weight, weight_scale_inv, weight_block_size, torch.bfloat16)
+    out_w, out_s = per_block_cast_to_fp8(dequant.view((-1, k)))
+    return out_w.view(weight.shape), out_s.view(weight_scale_inv.shape)
+
+
+def requant_weight_ue8m0_inplace(weight, weight_scale_inv, weight_block_size):
+    """fp8_utils.py:424-429."""
+    assert isinstance(weight, torch.nn.Parameter)
+    assert isinstance(weight_scale_inv, torch.nn.Parameter)
+    weight.data, weight_scale_inv.data = _requant_weight_ue8m0(weight, weight_scale_inv, weight_block_size)
 
 
 def per_block_cast_to_fp8(x: torch.Tensor):

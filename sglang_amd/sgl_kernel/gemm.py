@@ -186,6 +186,29 @@ def _fp8_blockwise_scaled_mm_impl(mat_a, mat_b, scales_a, scales_b, out_dtype):
     return out
 
 
+def fp8_blockwise_scaled_mm_ue8m0(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    """fp8_blockwise_scaled_mm for scales that are all powers of two (UE8M0 values as fp32, what
+    ceil_to_ue8m0 of fp8_utils.py:485-486 produces): same arguments and result.  For bf16 outputs of more
+    than 128 rows the matrix instruction applies the scales itself and accumulates in place, reading only
+    their exponent bits; the caller guarantees that they are powers of two.  No counterpart among the
+    reference's ops: there this GEMM is DeepGEMM's (w8a8_block_fp8_matmul_deepgemm, fp8_kernel.py)."""
+    check_mm_common(mat_a, mat_b, out_dtype, FP8, "Float8_e4m3fn")
+    check_blockwise_scales(mat_a, mat_b, scales_a, scales_b)
+    m, k = mat_a.shape
+    n = mat_b.size(1)
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((m, n), dtype=out_dtype, device=mat_a.device)
+    lib = _lib.load()
+    rc = lib.sglq_fp8_blockwise_scaled_mm_ue8m0(
+        mat_a.data_ptr(), mat_a.stride(0) if m > 1 else k, mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
+        scales_b.data_ptr(), scales_b.stride(0), scales_b.stride(1),
+        out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype], m, n, k, *_lib.workspace(mat_a.device),
+        _lib.stream_ptr(mat_a.device))
+    _lib.check(rc, "fp8_blockwise_scaled_mm_ue8m0")
+    return out
+
+
 def fp8_blockwise_scaled_mm_bias(mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
     """fp8_blockwise_scaled_mm followed by the caller's `output += bias`
     (fp8_utils.py:207-211) in one kernel; no counterpart among the reference's ops."""

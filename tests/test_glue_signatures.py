@@ -87,6 +87,16 @@ def test_quant_wrappers_bind_the_linear_functions_calls():
           input_scale=None, bias=T)
 
 
+def test_ue8m0_path_binds_the_reference_calls():
+    # fp8_utils.py:248-250: the GEMM call of deepgemm_w8a8_block_fp8_linear_with_fallback
+    a = binds(fp8_kernel.w8a8_block_fp8_matmul_deepgemm, T, T, T, T, [128, 128], output_dtype=torch.bfloat16)
+    assert list(a) == ["A", "B", "As", "Bs", "block_size", "output_dtype"]
+    # fp8_utils.py:424-429 (called by the loaders as requant_weight_ue8m0_inplace(weight, weight_scale_inv, weight_block_size))
+    assert list(inspect.signature(fp8_utils.requant_weight_ue8m0_inplace).parameters) == ["weight", "weight_scale_inv", "weight_block_size"]
+    # the flag the reference keeps in deep_gemm_wrapper (fp8_utils.py:245); off unless asked for
+    assert fp8_utils.DEEPGEMM_SCALE_UE8M0 in (False, True)
+
+
 def test_gemm_wrappers_bind_the_linear_functions_calls():
     import sgl_kernel
     import sgl_kernel.gemm as G
