@@ -76,6 +76,20 @@ def build():
     d["w_tensor_codes"], d["w_tensor_scales"] = bits8(wq2), bits32(ws2)
     d["fp8_mm_bf16"] = bits16(O.fp8_scaled_mm(qf, wq2.t(), sf, ws2, torch.bfloat16, bias))
     d["fp8_mm_fp32"] = bits32(O.fp8_scaled_mm(qf, wq2.t(), sf, ws2, torch.float32, bias))
+    # power-of-two (UE8M0) group scales: codes, exponent bytes, packed words; the block-scaled GEMM on them with a
+    # weight whose block scales are rounded up to powers of two (python/sglang/srt/layers/quantization/fp8_utils.py:468-486)
+    uq, ue, up = O.per_token_group_quant_fp8_ue8m0(x)
+    d["group128_ue8m0_codes"], d["group128_ue8m0_exponents"] = bits8(uq), ue.numpy()
+    d["group128_ue8m0_packed"] = up.contiguous().numpy()
+    blocks = w.float().view(n // 128, 128, k // 128, 128)
+    y = blocks.abs().amax(dim=(1, 3), keepdim=True).clamp(1e-4) / 448.0
+    yb = y.view(torch.int32)
+    sf = (((yb >> 23) + ((yb & 0x7FFFFF) != 0).to(torch.int32)) << 23).view(torch.float32)
+    wq_u = (blocks / sf).to(torch.float8_e4m3fn).view(n, k).contiguous()
+    ws_u = sf.view(n // 128, k // 128).contiguous()
+    d["w_block_ue8m0_codes"], d["w_block_ue8m0_scales"] = bits8(wq_u), bits32(ws_u)
+    us = torch.pow(2.0, ue.float() - 127.0)
+    d["block_ue8m0_mm_fp32"] = bits32(O.fp8_blockwise_scaled_mm(uq, wq_u.t(), us, ws_u.t(), torch.float32))
     return d
 
 

@@ -125,3 +125,27 @@ def test_gemm_kernels_reproduce_the_fixture(gpu):
     out = fp8_scaled_mm(af, wt.t(), sf, wts, torch.bfloat16, bias)
     torch.testing.assert_close(out.cpu().float(), f32(z["fp8_mm_fp32"]), rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(out.cpu().float(), t16(z["fp8_mm_bf16"]).float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.gpu
+def test_power_of_two_scale_kernels_reproduce_the_fixture(gpu):
+    """UE8M0 group quantization (fp32 powers of two and the packed words of scale_ue8m0=True) bit for bit,
+    the block-scaled GEMM that applies such scales inside the matrix instruction within tolerance."""
+    from sglang_amd.quantization.fp8_kernel import per_token_group_quant_fp8_pow2, sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_ue8m0
+
+    print("golden: power-of-two scales", flush=True)
+    z = load()
+    x = t16(z["x_bf16"]).to(gpu)
+    want_s = torch.pow(2.0, torch.from_numpy(z["group128_ue8m0_exponents"].astype(np.float32)) - 127.0)
+    for cm in (False, True):
+        q, s = per_token_group_quant_fp8_pow2(x, 128, column_major_scales=cm)
+        same_bits(q, z["group128_ue8m0_codes"], "UE8M0 codes")
+        assert torch.equal(s.cpu(), want_s), "UE8M0 scales are not 2^(exponent byte - 127)"
+    q, packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    same_bits(q, z["group128_ue8m0_codes"], "UE8M0 codes (packed-scale kernel)")
+    assert np.array_equal(packed.cpu().contiguous().numpy(), z["group128_ue8m0_packed"]), "packed UE8M0 words differ from the fixture"
+    xq, wq = t8(z["group128_ue8m0_codes"]).to(gpu), t8(z["w_block_ue8m0_codes"]).to(gpu)
+    xs, ws = want_s.to(gpu), f32(z["w_block_ue8m0_scales"]).to(gpu)
+    out = fp8_blockwise_scaled_mm_ue8m0(xq, wq.t(), xs.t().contiguous().t(), ws.t(), torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), f32(z["block_ue8m0_mm_fp32"]), rtol=1e-2, atol=1e-2)
