@@ -359,7 +359,8 @@ int sglq_tuned_clear(void);
  * bytes through registers.  Both must give identical results. */
 void sglq_debug_set_direct_lds(int on);
 /* Test hook: 0 = choose the GEMM kernel and tile by shape (default); 16 / 32 = the M <= 32
- * kernel whose blocks own 16 / 32 weight rows and all of K; 64 = the M <= 64 split-K kernel;
+ * kernel whose blocks own 16 / 32 weight rows and all of K; 64 = the split-K decode kernel
+ * (M <= 512) with 128 weight rows per block, 66 = with 64 weight rows per block (M > 32);
  * 128 = the 128x128 kernel; 256 = the plain 256x256 kernel; 258 = the pipelined 256x256
  * kernel; 130 = the same kernel with 128-row tiles; 192 / 224 / 257 = the pipelined 4x2-wave
  * kernel with tiles 192 / 224 / 256 wide.

@@ -1669,23 +1669,25 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
 // tiles per weight tile; they run side by side on one XCD, so the weights still come from
 // HBM once and from that XCD's L2 after that.
 // ---------------------------------------------------------------------------
-template <int KIND, int MI, int OUT_DT>
+template <int KIND, int MI, int OUT_DT, int BN = 128>
 // (two waves per SIMD asked for: with at most 256 registers per lane the MFMAs write plain
 // VGPRs; given 512 the compiler puts their results into accumulation registers and copies
 // each one out behind a full MFMA latency of wait states)
 __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
-  constexpr int BN = 128, NI = 2;
+  static_assert(BN == 128 || BN == 64, "a wave takes 32 or 16 of the block's weight rows");
+  constexpr int NI = BN / 64;
+  constexpr int WCW = BN / 32;                     // weight copies per wave per stage
   constexpr int AR = MI * 16 < 32 ? 32 : MI * 16;  // activation rows staged (at least one copy per wave)
   constexpr int ACW = AR / 32;                     // activation copies per wave per stage
   constexpr bool BLOCK = is_block(KIND);
-  constexpr int CPW = 4 + ACW + (BLOCK ? 2 : 0);   // vector-memory loads per wave per stage
+  constexpr int CPW = WCW + ACW + (BLOCK ? 2 : 0);  // vector-memory loads per wave per stage
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 2048 : 0;  // 4 x 256 B of activation scales, then the weight scale
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
   // 60-78 KiB of LDS: two blocks (eight waves) per CU.  A ring of six stages (one block per CU,
   // five stages in flight) is slower wherever it was tried, also for launches of fewer blocks than
   // CUs whose blocks walk 56 K blocks each (64 x 2048 x 7168 without split-K: 29.5 us with three stages,
   // 32.9 with six): what a CU's load path delivers sets the step time, not the depth of the ring.
-  constexpr int NSTAGE = 3;
+  constexpr int NSTAGE = BN == 64 ? 4 : 3;
   constexpr bool IS_FP8 = fp8_operands(KIND);
 
   __shared__ __attribute__((aligned(1024))) char smem[NSTAGE * STAGE_BYTES];
@@ -1733,7 +1735,7 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
     // dword, brought by lane 0 of wave 0 (the other lanes and waves are out of range; the
     // instruction stays so that every wave counts the same number of copies per stage)
     const int nblocks = (p.N + 127) >> 7;
-    const int nb = tile_n < nblocks ? tile_n : nblocks - 1;
+    const int nb = (n0 >> 7) < nblocks ? (n0 >> 7) : nblocks - 1;
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
     rsb = make_rsrc_sgpr(p.sb, (uint32_t)(sfb_elems * 4));
     off_sb = (wave == 0 && lane == 0) ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
@@ -1745,7 +1747,7 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
     const uint32_t st = smem_base + (uint32_t)(t % NSTAGE) * STAGE_BYTES;
     const uint32_t k0 = (uint32_t)(kb0 + t * kstride) * 128u;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) lds_copy16(rb, st + (wave + 4 * j) * 1024, off_w + j * step_w, k0);
+    for (int j = 0; j < WCW; ++j) lds_copy16(rb, st + (wave + 4 * j) * 1024, off_w + j * step_w, k0);
 #pragma unroll
     for (int j = 0; j < ACW; ++j) lds_copy16(ra, st + W_BYTES + (wave + 4 * j) * 1024, off_a + j * step_a, k0);
     // one dword per lane: its row's activation scale for this K block
@@ -1782,7 +1784,7 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
   Frags fa, fb;
   auto read_one = [&](int t, Frags& d, int k) {  // k-th LDS read group of K block t
     const char* st = smem + (t % NSTAGE) * STAGE_BYTES;
-    if (k < NI) d.f[k] = read_frag(st + (wave * 32 + k * 16) * 128);
+    if (k < NI) d.f[k] = read_frag(st + (wave * (BN / 4) + k * 16) * 128);
     else if (k < NI + MI) d.f[k] = read_frag(st + W_BYTES + (k - NI) * 16 * 128);
     else if constexpr (BLOCK) {
       d.sb = *reinterpret_cast<const float*>(st + W_BYTES + A_BYTES + 1024);
@@ -1794,9 +1796,10 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
   constexpr int NREAD = NI + MI + 1;
   // "K block u has landed" with the blocks up to u + younger issued: copies retire in order
   static_assert((NSTAGE - 1) * CPW < 64, "vmcnt holds six bits");
-  static_assert(NSTAGE == 3, "wait_landed counts at most two younger blocks");
+  static_assert(NSTAGE <= 4, "wait_landed counts at most three younger blocks");
   auto wait_landed = [&](int younger) {
-    if (younger >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * CPW));
+    if (younger >= 3) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(3 * CPW));
+    else if (younger == 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * CPW));
     else if (younger == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(CPW));
     else __builtin_amdgcn_s_waitcnt(0);
   };
@@ -1867,8 +1870,8 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
     if (t + 1 < nsteps) step(t + 1, fb, fa);
   }
 
-  if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, m_base, n0 + wave * 32, r16, g);
-  else store_partials<MI, NI>(p, acc, split, m_base, n0 + wave * 32, r16, g);
+  if (p.splits == 1) epilogue<KIND, OUT_DT, MI, NI>(p, acc, m_base, n0 + wave * (BN / 4), r16, g);
+  else store_partials<MI, NI>(p, acc, split, m_base, n0 + wave * (BN / 4), r16, g);
 }
 
 // ---------------------------------------------------------------------------
@@ -2571,17 +2574,32 @@ static void launch_reduce(GemmArgs& p, hipStream_t st) {
   splitk_reduce_kernel<KIND, OUT_DT><<<dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st>>>(p);
 }
 
-template <int KIND, int MI, int OUT_DT>
+template <int KIND, int MI, int OUT_DT, int BN = 128>
 static void launch_skinny_mi(GemmArgs& p, hipStream_t st) {
-  g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
+  if (BN == 64) g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel<64 columns>+splitk_reduce_kernel" : "gemm_skinny_kernel<64 columns>";
+  else g_last_kernel = p.splits > 1 ? "gemm_skinny_kernel+splitk_reduce_kernel" : "gemm_skinny_kernel";
   const dim3 grid((uint32_t)(p.tiles_n * p.splits * p.tiles_m)), block(256);
-  gemm_skinny_kernel<KIND, MI, OUT_DT><<<grid, block, 0, st>>>(p);
+  gemm_skinny_kernel<KIND, MI, OUT_DT, BN><<<grid, block, 0, st>>>(p);
   if (p.splits > 1) launch_reduce<KIND, OUT_DT>(p, st);
 }
 
+// Modelled time (us, without what every launch pays) of gemm_skinny_kernel on M > 64 rows with tiles of `bn` weight rows
+// and `sp` splits of K.  Fitted to sweeps of M = 96 .. 512, N = 2048 .. 8192, K = 2048 .. 7168: a K step of a block
+// that has its CU to itself takes 0.5 us with 128 weight rows and 0.32 us with 64 (0.4 / 0.24 us for the kinds
+// without block scales), proportionally more once there are more blocks than CUs; a split costs 4 us for the second
+// launch plus the partial sums written and read at 4 TB/s.
+static double skinny_cost(int M, int N, int K, int bn, int sp) {
+  const int tiles = ((M + 63) / 64) * ((N + bn - 1) / bn), nkb = K >> 7;
+  const int blocks = tiles * sp;
+  const double steps = (double)((nkb + sp - 1) / sp);
+  double cost = steps * (bn == 64 ? 0.32 : 0.5) * (blocks > 256 ? blocks / 256.0 : 1.0);
+  if (sp > 1) cost += 4.0 + (double)M * N * 4.0 * sp * 2.0 / 4e6;
+  return cost;
+}
+
 // The split-K factor of the decode path without the caller's workspace limits: so that every CU streams weights.
-static int skinny_splits(int M, int N, int K) {
-  const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
+static int skinny_splits(int M, int N, int K, int bn = 128) {
+  const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + bn - 1) / bn);
   const int nkb = K >> 7;
   // Measured: the fastest split factor puts about one block on every CU (192-256 blocks);
   // more blocks only add partial-sum traffic.
@@ -2598,10 +2616,7 @@ static int skinny_splits(int M, int N, int K) {
     double best = 0.0;
     splits = 1;
     for (int sp = 1; sp <= max_splits; ++sp) {
-      const int blocks = tiles * sp;
-      const double steps = (double)((nkb + sp - 1) / sp);
-      double cost = steps * 0.5 * (blocks > 256 ? blocks / 256.0 : 1.0);
-      if (sp > 1) cost += 4.0 + (double)M * N * 4.0 * sp * 2.0 / 4e6;
+      const double cost = skinny_cost(M, N, K, bn, sp);
       if (sp == 1 || cost < best) {
         best = cost;
         splits = sp;
@@ -2617,10 +2632,17 @@ static int skinny_splits(int M, int N, int K) {
 
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  // Weight rows per block: 128, or 64 where several row tiles share the weight tiles (M > 64) and the model above
+  // says that twice as many blocks with two thirds of the bytes each are faster: up to about 200 tiles of 128.
+  bool narrow = t_tile == 66 && p.M > 32;
+  if (t_tile == 0 && p.M > 64) {
+    const int sw = skinny_splits(p.M, p.N, p.K, 128), sn = skinny_splits(p.M, p.N, p.K, 64);
+    narrow = skinny_cost(p.M, p.N, p.K, 64, sn) < skinny_cost(p.M, p.N, p.K, 128, sw);
+  }
   p.tiles_m = (p.M + 63) / 64;
-  p.tiles_n = (p.N + 127) / 128;
+  p.tiles_n = narrow ? (p.N + 63) / 64 : (p.N + 127) / 128;
   const int nkb = p.K >> 7;
-  int splits = skinny_splits(p.M, p.N, p.K);
+  int splits = skinny_splits(p.M, p.N, p.K, narrow ? 64 : 128);
   if (t_splits > 0) splits = t_splits < nkb ? t_splits : nkb;
   const int64_t per_split = (int64_t)p.M * p.N * 4;
   if (!p.ws || ws_bytes < per_split * 2) splits = 1;
@@ -2629,6 +2651,7 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   p.splits = splits;
   if (p.M <= 16) launch_skinny_mi<KIND, 1, OUT_DT>(p, st);
   else if (p.M <= 32) launch_skinny_mi<KIND, 2, OUT_DT>(p, st);
+  else if (narrow) launch_skinny_mi<KIND, 4, OUT_DT, 64>(p, st);
   else launch_skinny_mi<KIND, 4, OUT_DT>(p, st);  // (64-row tiles for any M > 32)
 }
 
@@ -2781,8 +2804,8 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const int skinny_steps = ((p.K >> 7) + skinny_fit - 1) / skinny_fit;
   const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && weight_bytes <= (p.M <= 128 ? (64 << 20) : (48 << 20) - 1) &&
                           !(is_block(KIND) && skinny_steps > 40 && skinny_fit * skinny_tiles < 224);
-  const bool skinny_rows = p.M <= 64 || skinny_mid || (t_tile == 64 && p.M <= 512);
-  if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64)) {
+  const bool skinny_rows = p.M <= 64 || skinny_mid || ((t_tile == 64 || t_tile == 66) && p.M <= 512);
+  if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64 || t_tile == 66)) {
     launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
@@ -2914,7 +2937,7 @@ extern "C" int sglq_tuned_clear(void) {
   return SGLQ_OK;
 }
 extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
-  static const int tiles[] = {0, 16, 32, 64, 128, 130, 192, 224, 256, 257, 258};
+  static const int tiles[] = {0, 16, 32, 64, 66, 128, 130, 192, 224, 256, 257, 258};
   bool known = false;
   for (int t : tiles) known = known || t == tile;
   if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {

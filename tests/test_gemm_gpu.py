@@ -36,9 +36,9 @@ def load_path(request):
 
 
 # tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel, 130 the same kernel with 128-row tiles,
-# 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32],
-                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32"])
+# 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block, 66 the split-K decode kernel with 64 weight rows per block (M <= 512)
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32, 66],
+                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32", "skinny64"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -425,19 +425,21 @@ def test_decode_kernel_split_k(gpu, splits, mnk):
 
 
 @pytest.mark.parametrize("mnk", [(65, 264, 1024), (100, 2112, 1536), (128, 4096, 512), (129, 640, 2048), (300, 384, 1024),
-                                 (512, 256, 4096)])
-def test_decode_kernel_row_tiles(gpu, splits, mnk):
-    """The weight-streaming kernel with a second grid dimension of 64-row tiles (up to M = 512
-    when forced; the heuristic takes it up to M = 128): every kind, any split factor, ragged
-    last tile."""
+                                 (512, 256, 4096), (256, 4096, 4096), (200, 1096, 896)])
+@pytest.mark.parametrize("weight_rows", [128, 64])
+def test_decode_kernel_row_tiles(gpu, splits, mnk, weight_rows):
+    """The weight-streaming kernel with a second grid dimension of 64-row tiles (up to M = 512), with
+    128 or 64 weight rows per block: every kind, any split factor, ragged last tiles in both directions."""
     from sglang_amd import _lib
 
-    say("decode kernel, row tiles", mnk, "splits", splits)
+    say("decode kernel, row tiles", mnk, "splits", splits, "weight rows per block", weight_rows)
     lib = _lib.load()
-    lib.sglq_debug_force_tile(64)
+    lib.sglq_debug_force_tile(64 if weight_rows == 128 else 66)
     try:
         check_every_kind(gpu, *mnk)
-        assert lib.sglq_debug_last_gemm_kernel().decode().startswith("gemm_skinny_kernel")
+        name = lib.sglq_debug_last_gemm_kernel().decode()
+        assert name.startswith("gemm_skinny_kernel<64 columns>" if weight_rows == 64 else "gemm_skinny_kernel") and \
+            ("<64 columns>" in name) == (weight_rows == 64), name
     finally:
         lib.sglq_debug_force_tile(0)
 
