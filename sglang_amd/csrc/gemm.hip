@@ -1886,7 +1886,7 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const GemmArgs p) {
 // NSTAGE - 1 younger stages outstanding; past the wave's last K block the copies are pointed
 // out of range (zero fill, no memory traffic), which keeps that count constant.
 // ---------------------------------------------------------------------------
-template <int KIND, int MI, int NIB, int OUT_DT>
+template <int KIND, int MI, int NIB, int OUT_DT, bool ROW_TILES = false>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
   constexpr int BN = NIB * 16, AR = MI * 16;
   constexpr bool BLOCK = is_block(KIND);
@@ -1895,17 +1895,29 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
   constexpr int CPW = WC + AC + (BLOCK ? 2 : 0);   // vector-memory loads per stage
   constexpr int W_BYTES = BN * 128, A_BYTES = AR * 128, S_BYTES = BLOCK ? 512 : 0;
   constexpr int STAGE_BYTES = W_BYTES + A_BYTES + S_BYTES;
-  constexpr int NSTAGE = SGLQ_STREAM_NSTAGE;
+  // (64 x 64 tiles: two stages of 16.5 KiB per wave, 132 KiB per block)
+  constexpr int NSTAGE = MI * NIB >= 16 ? 2 : SGLQ_STREAM_NSTAGE;
   constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
   static_assert((NSTAGE - 1) * CPW <= 63, "vmcnt holds 6 bits");
   static_assert(MI * NIB * 1024 <= RING_BYTES, "the partial sums are exchanged through a wave's ring");
+  static_assert(4 * RING_BYTES <= 160 * 1024, "LDS of one CU");
 
   __shared__ __attribute__((aligned(1024))) char smem[4 * RING_BYTES];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4, l8 = lane >> 3;
-  const int n0 = blockIdx.x * BN;
+  // ROW_TILES (M > 64): a second grid dimension of 64-row tiles.  The row tiles of one weight tile get block ids
+  // 8 apart inside a group of eight weight tiles, so they are dispatched together and (blocks go to the eight
+  // XCDs round-robin) to the same XCD, whose L2 serves the weight tile's later readers.
+  int n0 = blockIdx.x * BN, m_base = 0;
+  if constexpr (ROW_TILES) {
+    const int group = (int)blockIdx.x / (8 * p.tiles_m);
+    const int in_group = (int)blockIdx.x - group * 8 * p.tiles_m;
+    const int width = p.tiles_n - group * 8 < 8 ? p.tiles_n - group * 8 : 8;
+    n0 = (group * 8 + in_group % width) * BN;
+    m_base = (in_group / width) * AR;
+  }
   const int nkb = p.K >> 7;
   const int nsteps = (nkb - wave + 3) >> 2;  // K blocks wave, wave + 4, ...
 
@@ -1917,7 +1929,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
   // swz(row) = (row & 7) ^ ((row >> 3) & 1) = (l / 8) ^ (gj & 1).
   const int c16_even = (((lane & 7) ^ l8) & 7) * 16, c16_odd = (((lane & 7) ^ l8 ^ 1) & 7) * 16;
   const uint32_t offw_even = (uint32_t)(n0 + l8) * p.ldb + c16_even, offw_odd = (uint32_t)(n0 + l8) * p.ldb + c16_odd;
-  const uint32_t offa_even = (uint32_t)l8 * p.lda + c16_even, offa_odd = (uint32_t)l8 * p.lda + c16_odd;
+  const uint32_t offa_even = (uint32_t)(m_base + l8) * p.lda + c16_even, offa_odd = (uint32_t)(m_base + l8) * p.lda + c16_odd;
   const uint32_t step_w = 8u * p.ldb, step_a = 8u * p.lda;
   uint32_t off_sa = OOB, off_sb = OOB;
   int sfa_step = 0, sfb_step = 0;
@@ -1927,7 +1939,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
     rsa = make_rsrc_sgpr(p.sa, (uint32_t)(sfa_elems * 4));
     rsb = make_rsrc_sgpr(p.sb, (uint32_t)(sfb_elems * 4));
-    off_sa = lane < p.M ? (uint32_t)(lane * p.sa_stride_m * 4) : OOB;  // lane = activation row
+    off_sa = m_base + lane < p.M ? (uint32_t)((m_base + lane) * p.sa_stride_m * 4) : OOB;  // lane = activation row of the tile
     int nb = n0 >> 7;  // BN divides 128: one scale block per block of rows
     if (nb >= nblocks) nb = nblocks - 1;
     off_sb = lane == 0 ? (uint32_t)(nb * p.sb_stride_n * 4) : OOB;
@@ -2033,7 +2045,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const GemmArgs p) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc[i][j][e] += t[e];
         }
-    epilogue<KIND, OUT_DT, MI, NIB>(p, acc, 0, n0, r16, g);
+    epilogue<KIND, OUT_DT, MI, NIB>(p, acc, m_base, n0, r16, g);
   }
 }
 
@@ -2729,6 +2741,37 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
   return true;
 }
 
+// 64 < M <= 512 on the full-K decode kernel: 64 x 64 tiles, one block per tile (its four waves take every fourth K
+// block each and read their operands from LDS once, where the split-K kernel's waves all read the tile's
+// activation rows).  A K block takes 0.22 us there whatever the kind, against 0.32 us (block-scaled kinds) on the
+// split-K kernel with 64 weight rows per block: it pays for the block-scaled kinds while the tiles fit one per CU
+// (256 x 4096 x 7168: 22.5 -> 17.1 us, 512 x 2048 x 7168: 22.5 -> 17.0 us, 256 x 4096 x 4096: 14.9 -> 12.5 us), not beyond
+// (one block per CU: 512 x 4096 x 4096 21.9 against 18.9 us) and not where the split-K kernel splits well
+// (128 x 2048 x 7168: 16.4 against 13.3 us).
+template <int KIND>
+static bool stream_tiles_pays(const GemmArgs& p) {
+  if (!is_block(KIND) || p.M <= 64 || p.K < 512) return false;
+  const int tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+  if (tiles > num_cus()) return false;
+  // (few tiles and a long K: the split-K kernel spreads the K blocks over the CUs that this kernel leaves idle;
+  // 128 x 4096 x 7168, 128 tiles: 18.9 us here, 16.4 us there with four splits)
+  const int nkb = p.K >> 7;
+  if (!(2 * tiles > num_cus() || (nkb <= 32 && 4 * tiles > num_cus()) || nkb <= 16)) return false;
+  const double wide = skinny_cost(p.M, p.N, p.K, 128, skinny_splits(p.M, p.N, p.K, 128));
+  const double narrow = skinny_cost(p.M, p.N, p.K, 64, skinny_splits(p.M, p.N, p.K, 64));
+  // (1 us more than the split-K kernel per launch: the partial sums' way through LDS at the end)
+  return 1.0 + 0.22 * nkb < 0.95 * (wide < narrow ? wide : narrow);
+}
+
+template <int KIND, int OUT_DT>
+static void launch_stream_tiles(GemmArgs& p, hipStream_t st) {
+  p.splits = 1;
+  p.tiles_m = (p.M + 63) / 64;
+  p.tiles_n = (p.N + 63) / 64;
+  g_last_kernel = "gemm_stream_kernel<64 x 64 tiles>";
+  gemm_stream_kernel<KIND, 4, 4, OUT_DT, true><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(256), 0, st>>>(p);
+}
+
 // Tuned kernel selections per problem, the counterpart of the reference's per-(N, K) JSON
 // tables for its Triton kernels (python/sglang/srt/layers/quantization/fp8_kernel.py:738-776,
 // layers/quantization/configs/): an entry names the kernel (a code of sglq_debug_force_tile)
@@ -2804,9 +2847,14 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const int skinny_steps = ((p.K >> 7) + skinny_fit - 1) / skinny_fit;
   const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && weight_bytes <= (p.M <= 128 ? (64 << 20) : (48 << 20) - 1) &&
                           !(is_block(KIND) && skinny_steps > 40 && skinny_fit * skinny_tiles < 224);
+  if ((p.K & 127) == 0 && p.K >= 512 && g_use_dma && t_tile == 68 && p.M > 32 && p.M <= 1024) {
+    launch_stream_tiles<KIND, OUT_DT>(p, st);
+    return;
+  }
   const bool skinny_rows = p.M <= 64 || skinny_mid || ((t_tile == 64 || t_tile == 66) && p.M <= 512);
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64 || t_tile == 66)) {
-    launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
+    if (t_tile == 0 && stream_tiles_pays<KIND>(p)) launch_stream_tiles<KIND, OUT_DT>(p, st);
+    else launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
   // Measured crossover: the 256 x 256 kernel wins once its tiles cover more than half of
@@ -2937,7 +2985,7 @@ extern "C" int sglq_tuned_clear(void) {
   return SGLQ_OK;
 }
 extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
-  static const int tiles[] = {0, 16, 32, 64, 66, 128, 130, 192, 224, 256, 257, 258};
+  static const int tiles[] = {0, 16, 32, 64, 66, 68, 128, 130, 192, 224, 256, 257, 258};
   bool known = false;
   for (int t : tiles) known = known || t == tile;
   if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {

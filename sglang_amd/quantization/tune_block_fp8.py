@@ -34,6 +34,8 @@ def candidates(m: int, n: int, k: int):
         out += [(64, s) for s in (0, 2, 4, 8) if s == 0 or s <= nkb // 2]
         if m > 64:
             out += [(66, s) for s in (0, 1, 2, 4) if s <= 1 or s <= nkb // 4]
+            if k >= 512:
+                out += [(68, 0)]
     out += [(128, s) for s in (0, 2, 4) if s == 0 or s <= nkb // 4]
     if k >= 384 and m > 64:
         out += [(130, s) for s in (0, 1, 2, 4, 8) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]

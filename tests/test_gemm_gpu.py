@@ -37,8 +37,10 @@ def load_path(request):
 
 # tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel, 130 the same kernel with 128-row tiles,
 # 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block, 66 the split-K decode kernel with 64 weight rows per block (M <= 512)
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32, 66],
-                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32", "skinny64"])
+# 68 the full-K decode kernel on 64 x 64 tiles (32 < M <= 1024)
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32, 66, 68],
+                ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32", "skinny64",
+                     "stream64x64"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -440,6 +442,23 @@ def test_decode_kernel_row_tiles(gpu, splits, mnk, weight_rows):
         name = lib.sglq_debug_last_gemm_kernel().decode()
         assert name.startswith("gemm_skinny_kernel<64 columns>" if weight_rows == 64 else "gemm_skinny_kernel") and \
             ("<64 columns>" in name) == (weight_rows == 64), name
+    finally:
+        lib.sglq_debug_force_tile(0)
+
+
+@pytest.mark.parametrize("mnk", [(65, 264, 1024), (100, 2112, 1536), (128, 4096, 512), (129, 640, 2048), (300, 384, 1024),
+                                 (512, 256, 4096), (256, 4096, 4096), (200, 1096, 896), (1000, 200, 640)])
+def test_full_k_decode_kernel_on_row_tiles(gpu, mnk):
+    """The full-K decode kernel on 64 x 64 tiles (several row tiles per weight tile, the four waves of a block
+    take every fourth K block): every kind, ragged last tiles in both directions, fewer K blocks than waves + 1."""
+    from sglang_amd import _lib
+
+    say("full-K decode kernel, 64 x 64 tiles", mnk)
+    lib = _lib.load()
+    lib.sglq_debug_force_tile(68)
+    try:
+        check_every_kind(gpu, *mnk)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_stream_kernel<64 x 64 tiles>"
     finally:
         lib.sglq_debug_force_tile(0)
 

@@ -119,7 +119,7 @@ def test_two_streams_do_not_share_partial_sums(gpu):
 
     print("two streams", flush=True)
     lib = _lib.load()
-    m, n, k = 300, 2112, 7168
+    m, n, k = 96, 2112, 7168
     wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=21))
     wq, ws = wq.to(gpu), ws.to(gpu)
     cases = []
