@@ -594,6 +594,7 @@ def time_kernel(fn, iters, rotate=1):
         fn(i % rotate)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
+    iters = max(iters, rotate)  # every copy takes its turn inside the graph
     with torch.cuda.graph(g):
         for i in range(iters):
             fn(i % rotate)
@@ -643,7 +644,8 @@ def config_summary(args):
         sh = d.get("shapes", [])
         if sh:
             d["linear_us_sum"] = round(sum(x["quant_us"] + x["gemm_us"] for x in sh), 1)
-    out["timing"] = "device time per call from a HIP graph of 20 calls, inputs and weights rotated past the last-level cache"
+    out["timing"] = ("device time per call from a HIP graph of 20 calls or more, the weights rotated over copies of 320 MB and more in total "
+                     "(past the 256 MiB last-level cache), every copy inside the graph")
     return out
 
 
@@ -678,8 +680,11 @@ def run_sweep(args, collect=None, cfg2_ms=None, only=None):
         f.flush()
         print(json.dumps(kw), flush=True)
 
-    def rot_count(nbytes):  # rotate over enough copies to exceed the 256 MiB last-level cache
+    def rot_count(nbytes):  # activations: up to eight copies (they come from the layer before and are cache-warm in use)
         return max(1, min(8, int(600e6 // max(nbytes, 1))))
+
+    def weight_copies(nbytes):  # weights: enough copies to exceed the 256 MiB last-level cache (320 MB and more in rotation)
+        return max(2, min(48, -(-320_000_000 // max(nbytes, 1))))
 
     def block_case(cfg, name, m, n, k, seed):
         wq, ws = make_block_weight(n, k, seed, dev)
@@ -687,7 +692,7 @@ def run_sweep(args, collect=None, cfg2_ms=None, only=None):
         xs_in = [make_activation(m, k, seed + j, dev) for j in range(r)]
         tq = time_kernel(lambda j: sglang_per_token_group_quant_fp8(xs_in[j], 128, column_major_scales=True), args.iters, r)
         xq, xs = sglang_per_token_group_quant_fp8(xs_in[0], 128, column_major_scales=True)
-        rw = rot_count(n * k)
+        rw = weight_copies(n * k)
         wqs = [wq] + [wq.clone() for _ in range(rw - 1)]
         tg = time_kernel(lambda j: fp8_blockwise_scaled_mm(xq, wqs[j].t(), xs, ws.t(), torch.bfloat16), args.iters, rw)
         fl = 2.0 * m * n * k
@@ -739,7 +744,7 @@ def run_sweep(args, collect=None, cfg2_ms=None, only=None):
         sc = w.abs().amax() / 448.0
         wq = (w / sc).clamp(-448, 448).to(torch.float8_e4m3fn)
         ws = sc.reshape(1, 1).expand(n, 1).contiguous()
-        rw = rot_count(n * k)
+        rw = weight_copies(n * k)
         wqs = [wq] + [wq.clone() for _ in range(rw - 1)]
         for m in (1, 32, 256, 2048):
             x = make_activation(m, k, 3000 + m, dev)

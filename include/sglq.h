@@ -361,7 +361,7 @@ void sglq_debug_set_direct_lds(int on);
 /* Test hook: 0 = choose the GEMM kernel and tile by shape (default); 16 / 32 = the M <= 32
  * kernel whose blocks own 16 / 32 weight rows and all of K; 64 = the split-K decode kernel
  * (M <= 512) with 128 weight rows per block, 66 = with 64 weight rows per block (M > 32);
- * 68 = the full-K decode kernel on 64 x 64 tiles (32 < M <= 1024, K >= 512);
+ * 68 / 69 = the full-K decode kernel on 64 x 64 / 32 x 64 tiles (32 < M <= 1024, K >= 512);
  * 128 = the 128x128 kernel; 256 = the plain 256x256 kernel; 258 = the pipelined 256x256
  * kernel; 130 = the same kernel with 128-row tiles; 192 / 224 / 257 = the pipelined 4x2-wave
  * kernel with tiles 192 / 224 / 256 wide.

@@ -2604,7 +2604,11 @@ static double skinny_cost(int M, int N, int K, int bn, int sp) {
   const int tiles = ((M + 63) / 64) * ((N + bn - 1) / bn), nkb = K >> 7;
   const int blocks = tiles * sp;
   const double steps = (double)((nkb + sp - 1) / sp);
-  double cost = steps * (bn == 64 ? 0.32 : 0.5) * (blocks > 256 ? blocks / 256.0 : 1.0);
+  // (more blocks than CUs: the CUs that hold two set the pace; with 64 weight rows per block a step then takes
+  // 1.75 times as long at once, 288 .. 512 blocks alike)
+  double crowd = blocks > 256 ? blocks / 256.0 : 1.0;
+  if (bn == 64 && blocks > 256) crowd = crowd * 1.2 > 1.75 ? crowd * 1.2 : 1.75;
+  double cost = steps * (bn == 64 ? 0.32 : 0.5) * crowd;
   if (sp > 1) cost += 4.0 + (double)M * N * 4.0 * sp * 2.0 / 4e6;
   return cost;
 }
@@ -2743,33 +2747,49 @@ static bool launch_stream(GemmArgs& p, hipStream_t st) {
 
 // 64 < M <= 512 on the full-K decode kernel: 64 x 64 tiles, one block per tile (its four waves take every fourth K
 // block each and read their operands from LDS once, where the split-K kernel's waves all read the tile's
-// activation rows).  A K block takes 0.22 us there whatever the kind, against 0.32 us (block-scaled kinds) on the
+// activation rows).  A K block takes 0.24 us there whatever the kind, against 0.32 us (block-scaled kinds) on the
 // split-K kernel with 64 weight rows per block: it pays for the block-scaled kinds while the tiles fit one per CU
-// (256 x 4096 x 7168: 22.5 -> 17.1 us, 512 x 2048 x 7168: 22.5 -> 17.0 us, 256 x 4096 x 4096: 14.9 -> 12.5 us), not beyond
-// (one block per CU: 512 x 4096 x 4096 21.9 against 18.9 us) and not where the split-K kernel splits well
-// (128 x 2048 x 7168: 16.4 against 13.3 us).
+// (256 x 4096 x 7168: 23.1 -> 20.9 us, 512 x 2048 x 7168: 22.5 -> 19.0 us, 384 x 2048 x 4096: 14.3 -> 12.8 us), not beyond
+// (one block per CU: 512 x 4096 x 4096 24.5 against 20.7 us) and not where the split-K kernel splits well
+// (128 x 2048 x 7168: 20.1 against 13.7 us).  All times with the weights rotated past the last-level cache.
 template <int KIND>
-static bool stream_tiles_pays(const GemmArgs& p) {
-  if (!is_block(KIND) || p.M <= 64 || p.K < 512) return false;
-  const int tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
-  if (tiles > num_cus()) return false;
-  // (few tiles and a long K: the split-K kernel spreads the K blocks over the CUs that this kernel leaves idle;
-  // 128 x 4096 x 7168, 128 tiles: 18.9 us here, 16.4 us there with four splits)
+static int stream_tiles_choice(const GemmArgs& p) {  // 0: the split-K kernel; 68: 64 x 64 tiles; 69: 32 x 64 tiles
+  if (p.M <= 64 || p.K < 512) return 0;
   const int nkb = p.K >> 7;
-  if (!(2 * tiles > num_cus() || (nkb <= 32 && 4 * tiles > num_cus()) || nkb <= 16)) return false;
   const double wide = skinny_cost(p.M, p.N, p.K, 128, skinny_splits(p.M, p.N, p.K, 128));
   const double narrow = skinny_cost(p.M, p.N, p.K, 64, skinny_splits(p.M, p.N, p.K, 64));
+  // (the split-K kernel's steps are a quarter shorter for the kinds without block scales than the model's)
+  const double split_k = 0.95 * (is_block(KIND) ? 1.0 : 0.8) * (wide < narrow ? wide : narrow);
+  // 32 x 64 tiles while those fit one per CU: three stages of 12.5 KiB per wave, 100 KiB in flight per CU instead of
+  // 66, and a K block of half the work takes 0.17 us with the weights coming from HBM (256 x 2048 x 7168 block-FP8:
+  // 16.7 us on the split-K kernel, 19.3 us on 64 x 64 tiles, 14.6 us here; 256 x 2048 x 4096: 14.3 / 12.9 / 10.2 us;
+  // 128 x 4096 x 4096 per-channel FP8: 13.1 -> 11.2 us); any kind.  Few tiles and a long K stay with the split-K
+  // kernel, which spreads the K blocks over the idle CUs (96 x 2048 x 7168: 12.6 us there, 15.2 us here).
+  const int tiles32 = ((p.M + 31) / 32) * ((p.N + 63) / 64);
+  if (tiles32 <= num_cus() && 1.0 + 0.17 * nkb < split_k) return 69;
+  if (!is_block(KIND)) return 0;
+  const int tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+  if (tiles > num_cus()) return 0;
+  // (few tiles and a long K: the split-K kernel spreads the K blocks over the CUs that this kernel leaves idle;
+  // 128 x 4096 x 7168, 128 tiles: 18.9 us here, 16.4 us there with four splits)
+  if (!(2 * tiles > num_cus() || (nkb <= 32 && 4 * tiles > num_cus()) || nkb <= 16)) return 0;
   // (1 us more than the split-K kernel per launch: the partial sums' way through LDS at the end)
-  return 1.0 + 0.22 * nkb < 0.95 * (wide < narrow ? wide : narrow);
+  return 1.0 + 0.24 * nkb < split_k ? 68 : 0;
 }
 
 template <int KIND, int OUT_DT>
-static void launch_stream_tiles(GemmArgs& p, hipStream_t st) {
+static void launch_stream_tiles(GemmArgs& p, hipStream_t st, bool half_rows = false) {
   p.splits = 1;
-  p.tiles_m = (p.M + 63) / 64;
+  p.tiles_m = half_rows ? (p.M + 31) / 32 : (p.M + 63) / 64;
   p.tiles_n = (p.N + 63) / 64;
-  g_last_kernel = "gemm_stream_kernel<64 x 64 tiles>";
-  gemm_stream_kernel<KIND, 4, 4, OUT_DT, true><<<dim3((uint32_t)(p.tiles_m * p.tiles_n)), dim3(256), 0, st>>>(p);
+  const dim3 grid((uint32_t)(p.tiles_m * p.tiles_n)), block(256);
+  if (half_rows) {
+    g_last_kernel = "gemm_stream_kernel<32 x 64 tiles>";
+    gemm_stream_kernel<KIND, 2, 4, OUT_DT, true><<<grid, block, 0, st>>>(p);
+  } else {
+    g_last_kernel = "gemm_stream_kernel<64 x 64 tiles>";
+    gemm_stream_kernel<KIND, 4, 4, OUT_DT, true><<<grid, block, 0, st>>>(p);
+  }
 }
 
 // Tuned kernel selections per problem, the counterpart of the reference's per-(N, K) JSON
@@ -2847,14 +2867,21 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   const int skinny_steps = ((p.K >> 7) + skinny_fit - 1) / skinny_fit;
   const bool skinny_mid = p.M <= 512 && skinny_tiles <= 512 && skinny_steps <= 56 && weight_bytes <= (p.M <= 128 ? (64 << 20) : (48 << 20) - 1) &&
                           !(is_block(KIND) && skinny_steps > 40 && skinny_fit * skinny_tiles < 224);
-  if ((p.K & 127) == 0 && p.K >= 512 && g_use_dma && t_tile == 68 && p.M > 32 && p.M <= 1024) {
-    launch_stream_tiles<KIND, OUT_DT>(p, st);
+  if ((p.K & 127) == 0 && p.K >= 512 && g_use_dma && (t_tile == 68 || t_tile == 69) && p.M > 32 && p.M <= 1024) {
+    launch_stream_tiles<KIND, OUT_DT>(p, st, t_tile == 69);
     return;
   }
   const bool skinny_rows = p.M <= 64 || skinny_mid || ((t_tile == 64 || t_tile == 66) && p.M <= 512);
+  if ((p.K & 127) == 0 && g_use_dma && t_tile == 0 && p.M > 64 && p.M <= 512) {
+    // (32 x 64 tiles also where the split-K kernel is not in the running: K blocks beyond its 56 per block)
+    const int tiles_code = stream_tiles_choice<KIND>(p);
+    if (tiles_code == 69 || (tiles_code == 68 && skinny_rows)) {
+      launch_stream_tiles<KIND, OUT_DT>(p, st, tiles_code == 69);
+      return;
+    }
+  }
   if ((p.K & 127) == 0 && skinny_rows && g_use_dma && (t_tile == 0 || t_tile == 64 || t_tile == 66)) {
-    if (t_tile == 0 && stream_tiles_pays<KIND>(p)) launch_stream_tiles<KIND, OUT_DT>(p, st);
-    else launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
+    launch_skinny<KIND, OUT_DT>(p, ws_bytes, st);
     return;
   }
   // Measured crossover: the 256 x 256 kernel wins once its tiles cover more than half of
@@ -2985,7 +3012,7 @@ extern "C" int sglq_tuned_clear(void) {
   return SGLQ_OK;
 }
 extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
-  static const int tiles[] = {0, 16, 32, 64, 66, 68, 128, 130, 192, 224, 256, 257, 258};
+  static const int tiles[] = {0, 16, 32, 64, 66, 68, 69, 128, 130, 192, 224, 256, 257, 258};
   bool known = false;
   for (int t : tiles) known = known || t == tile;
   if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {

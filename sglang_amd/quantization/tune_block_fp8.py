@@ -35,7 +35,7 @@ def candidates(m: int, n: int, k: int):
         if m > 64:
             out += [(66, s) for s in (0, 1, 2, 4) if s <= 1 or s <= nkb // 4]
             if k >= 512:
-                out += [(68, 0)]
+                out += [(68, 0), (69, 0)]
     out += [(128, s) for s in (0, 2, 4) if s == 0 or s <= nkb // 4]
     if k >= 384 and m > 64:
         out += [(130, s) for s in (0, 1, 2, 4, 8) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]
@@ -67,7 +67,9 @@ def tune(n: int, k: int, ms, iters: int, margin: float, dev, dtype: str = "fp8_w
     else:
         w = (torch.randn((n, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
     ws = torch.rand(((n + 127) // 128, (k + 127) // 128), generator=g, device=dev) * 1e-2 + 1e-3
-    copies = max(1, min(8, int(600e6 // (n * k))))
+    # weights in rotation past the 256 MiB last-level cache (320 MB and more), as a model's layers come by in use
+    copies = max(2, min(48, -(-320_000_000 // (n * k))))
+    iters = max(iters, copies)
     wq = [w] + [w.clone() for _ in range(copies - 1)]
     table = {}
     for m in ms:

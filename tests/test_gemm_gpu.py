@@ -37,10 +37,10 @@ def load_path(request):
 
 # tile_auto sends M <= 64 to the decode kernel; 192 / 224 / 257 are the 4 x 2-wave kernel's tile widths (257 = 256 wide), 258 the pipelined 256 x 256 kernel, 130 the same kernel with 128-row tiles,
 # 16 / 32 the M <= 32 full-K decode kernel with that many weight rows per block, 66 the split-K decode kernel with 64 weight rows per block (M <= 512)
-# 68 the full-K decode kernel on 64 x 64 tiles (32 < M <= 1024)
-@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32, 66, 68],
+# 68 / 69 the full-K decode kernel on 64 x 64 / 32 x 64 tiles (32 < M <= 1024)
+@pytest.fixture(params=[0, 128, 256, 192, 224, 257, 258, 130, 16, 32, 66, 68, 69],
                 ids=["tile_auto", "tile128", "tile256", "wide192", "wide224", "wide256", "pipe256", "pipe128", "stream16", "stream32", "skinny64",
-                     "stream64x64"])
+                     "stream64x64", "stream32x64"])
 def tile(request):
     from sglang_amd import _lib
 
@@ -448,17 +448,18 @@ def test_decode_kernel_row_tiles(gpu, splits, mnk, weight_rows):
 
 @pytest.mark.parametrize("mnk", [(65, 264, 1024), (100, 2112, 1536), (128, 4096, 512), (129, 640, 2048), (300, 384, 1024),
                                  (512, 256, 4096), (256, 4096, 4096), (200, 1096, 896), (1000, 200, 640)])
-def test_full_k_decode_kernel_on_row_tiles(gpu, mnk):
-    """The full-K decode kernel on 64 x 64 tiles (several row tiles per weight tile, the four waves of a block
-    take every fourth K block): every kind, ragged last tiles in both directions, fewer K blocks than waves + 1."""
+@pytest.mark.parametrize("rows", [64, 32])
+def test_full_k_decode_kernel_on_row_tiles(gpu, mnk, rows):
+    """The full-K decode kernel on 64 x 64 and 32 x 64 tiles (several row tiles per weight tile, the four waves of
+    a block take every fourth K block): every kind, ragged last tiles in both directions, fewer K blocks than waves + 1."""
     from sglang_amd import _lib
 
-    say("full-K decode kernel, 64 x 64 tiles", mnk)
+    say("full-K decode kernel,", rows, "x 64 tiles", mnk)
     lib = _lib.load()
-    lib.sglq_debug_force_tile(68)
+    lib.sglq_debug_force_tile(68 if rows == 64 else 69)
     try:
         check_every_kind(gpu, *mnk)
-        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_stream_kernel<64 x 64 tiles>"
+        assert lib.sglq_debug_last_gemm_kernel().decode() == f"gemm_stream_kernel<{rows} x 64 tiles>"
     finally:
         lib.sglq_debug_force_tile(0)
 
@@ -711,7 +712,7 @@ BASELINE_KERNELS = [
     # decode launches of the same shapes
     ((1, 7168, 16384), "gemm_stream_kernel<16 rows>"),
     ((8, 7168, 16384), "gemm_stream_kernel<16 rows>"),
-    ((64, 7168, 16384), "gemm_kernel+splitk_reduce_kernel"),  # (tuned table entry)
+    ((64, 7168, 16384), "gemm_skinny_kernel+splitk_reduce_kernel"),
     ((1, 4096, 7168), "gemm_stream_kernel<16 rows>"),
     ((64, 4096, 7168), "gemm_stream_kernel<16 rows>"),
     ((1, 24576, 1536), "gemm_skinny_kernel"),

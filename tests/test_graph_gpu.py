@@ -119,27 +119,33 @@ def test_two_streams_do_not_share_partial_sums(gpu):
 
     print("two streams", flush=True)
     lib = _lib.load()
-    m, n, k = 96, 2112, 7168
-    wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=21))
-    wq, ws = wq.to(gpu), ws.to(gpu)
-    cases = []
-    for seed in (22, 23):
-        xq, xs = sglang_per_token_group_quant_fp8(O.gen_activation(m, k, seed=seed).to(gpu), 128, column_major_scales=True)
-        alone = fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
-        assert "splitk_reduce_kernel" in lib.sglq_debug_last_gemm_kernel().decode()
-        cases.append((xq, xs, alone))
-    torch.cuda.synchronize()
-    streams = [torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)]
-    pointers = set()
-    got = [[], []]
-    for rep in range(20):
-        for i, s in enumerate(streams):
-            with torch.cuda.stream(s):
-                pointers.add(_lib.workspace(gpu)[0])
-                xq, xs, _ = cases[i]
-                got[i].append(fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
-    torch.cuda.synchronize()
-    assert len(pointers) == 2
-    for i in range(2):
-        for y in got[i]:
-            assert torch.equal(y, cases[i][2])
+    m, n, k = 300, 2112, 7168
+    lib.sglq_debug_force_tile(64)  # the split-K decode kernel, four splits
+    lib.sglq_debug_force_splits(4)
+    try:
+        wq, ws = O.block_quant_weight(O.gen_weight(n, k, seed=21))
+        wq, ws = wq.to(gpu), ws.to(gpu)
+        cases = []
+        for seed in (22, 23):
+            xq, xs = sglang_per_token_group_quant_fp8(O.gen_activation(m, k, seed=seed).to(gpu), 128, column_major_scales=True)
+            alone = fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16)
+            assert "splitk_reduce_kernel" in lib.sglq_debug_last_gemm_kernel().decode()
+            cases.append((xq, xs, alone))
+        torch.cuda.synchronize()
+        streams = [torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)]
+        pointers = set()
+        got = [[], []]
+        for rep in range(20):
+            for i, s in enumerate(streams):
+                with torch.cuda.stream(s):
+                    pointers.add(_lib.workspace(gpu)[0])
+                    xq, xs, _ = cases[i]
+                    got[i].append(fp8_blockwise_scaled_mm(xq, wq.t(), xs, ws.t(), torch.bfloat16))
+        torch.cuda.synchronize()
+        assert len(pointers) == 2
+        for i in range(2):
+            for y in got[i]:
+                assert torch.equal(y, cases[i][2])
+    finally:
+        lib.sglq_debug_force_tile(0)
+        lib.sglq_debug_force_splits(0)
