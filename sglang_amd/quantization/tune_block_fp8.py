@@ -32,7 +32,7 @@ def candidates(m: int, n: int, k: int):
         out += [(16, 0), (32, 0)]
     if m <= 512:
         out += [(64, s) for s in (0, 2, 4, 8) if s == 0 or s <= nkb // 2]
-        if m > 64:
+        if m > 32:
             out += [(66, s) for s in (0, 1, 2, 4) if s <= 1 or s <= nkb // 4]
             if k >= 512:
                 out += [(68, 0), (69, 0)]
