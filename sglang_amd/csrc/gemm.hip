@@ -2655,6 +2655,9 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     const int sw = skinny_splits(p.M, p.N, p.K, 128), sn = skinny_splits(p.M, p.N, p.K, 64);
     narrow = skinny_cost(p.M, p.N, p.K, 64, sn) < skinny_cost(p.M, p.N, p.K, 128, sw);
   }
+  // 33 .. 64 rows: 64 weight rows per block on narrow weights and on short K (64 x 2048 x 16384: 19.8 -> 18.2 us,
+  // 64 x 7168 x 256: 4.8 -> 4.1 us); 128 on wide ones (64 x 10240 x 8192: 25.2 against 27.5 us)
+  if (t_tile == 0 && p.M > 32 && p.M <= 64) narrow = p.N <= 4096 || p.K <= 512;
   p.tiles_m = (p.M + 63) / 64;
   p.tiles_n = narrow ? (p.N + 63) / 64 : (p.N + 127) / 128;
   const int nkb = p.K >> 7;
@@ -2716,9 +2719,9 @@ static int stream_rows(const GemmArgs& p) {
       if (nib == 0 && p.K >= 8192 && blocks32 <= num_cus() && 16 * blocks32 > 15 * num_cus()) nib = 2;
     }
     if (nib == 2 && p.N < 2048) nib = 1;
-    // narrow weights: 16-row blocks up to 32 rows (8 x 512 x 7168: 14.2 us on the split-K kernel, two launches,
-    // 5.8 us here; 32 x 256 x 7168: 14.1 -> 6.8 us), the split-K kernel above that (64 x 512 x 7168: 11.9 us)
-    if (p.N < 1024) nib = p.M <= 32 ? 1 : 0;
+    // narrow weights: 16-row blocks (8 x 512 x 7168: 14.2 us on the split-K kernel, two launches, 5.8 us here;
+    // 32 x 256 x 7168: 14.1 -> 6.8 us; 64 x 512 x 7168: 11.4 -> 8.4 us, 64 x 768 x 2048: 9.2 -> 4.7 us)
+    if (p.N < 1024) nib = 1;
   }
   return nib;
 }

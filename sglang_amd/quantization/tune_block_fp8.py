@@ -28,7 +28,7 @@ def candidates(m: int, n: int, k: int):
     nkb = k // 128
     if k % 128:
         return out
-    if m <= 32 and k >= 512:
+    if m <= 64 and k >= 512:
         out += [(16, 0), (32, 0)]
     if m <= 512:
         out += [(64, s) for s in (0, 2, 4, 8) if s == 0 or s <= nkb // 2]

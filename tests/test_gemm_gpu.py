@@ -683,7 +683,7 @@ def test_shipped_tuned_tables_give_oracle_results(gpu):
 
 
 @pytest.mark.parametrize("mnk,kernel", [((8, 576, 7168), "gemm_stream_kernel<16 rows>"), ((32, 256, 7168), "gemm_stream_kernel<16 rows>"),
-                                        ((64, 512, 7168), "gemm_stream_kernel<32 x 64 tiles>"),  # (tuned table entry)
+                                        ((64, 512, 7168), "gemm_stream_kernel<16 rows>"),
                                         ((96, 36864, 2048), "gemm_pipe_kernel<128 rows>")])
 def test_narrow_weights_and_few_rows(gpu, mnk, kernel):
     """Shapes of the reference's tuned tables at the edges of the selection rules (N = 256 ... 576 of the
