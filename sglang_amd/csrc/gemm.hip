@@ -2657,7 +2657,12 @@ static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   }
   // 33 .. 64 rows: 64 weight rows per block on narrow weights and on short K (64 x 2048 x 16384: 19.8 -> 18.2 us,
   // 64 x 7168 x 256: 4.8 -> 4.1 us); 128 on wide ones (64 x 10240 x 8192: 25.2 against 27.5 us)
-  if (t_tile == 0 && p.M > 32 && p.M <= 64) narrow = p.N <= 4096 || p.K <= 512;
+  // ... and where 64-row blocks fill most of one round of the CUs without a split while 128-row blocks need two
+  // splits and the second launch (64 x 14336 x 4096: 19.8 -> 16.0 us)
+  if (t_tile == 0 && p.M > 32 && p.M <= 64) {
+    const int t64 = (p.N + 63) / 64;
+    narrow = p.N <= 4096 || p.K <= 512 || (4 * t64 > 3 * num_cus() && t64 <= num_cus() && (p.K >> 7) <= 40);
+  }
   p.tiles_m = (p.M + 63) / 64;
   p.tiles_n = narrow ? (p.N + 63) / 64 : (p.N + 127) / 128;
   const int nkb = p.K >> 7;
