@@ -250,3 +250,13 @@ def test_tuned_config_tables(tmp_path):
         assert lib.sglq_tuned_add(0, 128, 128, 0, 10, 64, 0) == 2 and b"1024 entries" in lib.sglq_last_error()
     finally:
         T.load_tuned_configs()  # back to the tables shipped with the package
+
+
+def test_shipped_tuned_tables_load_into_the_library():
+    """Every table shipped under quantization/configs is accepted by the library as it stands (known kernel
+    codes, split factors in range, no more entries than the table holds)."""
+    from sglang_amd.quantization import tuned_configs as T
+
+    files = [p for p in T.CONFIG_DIR.iterdir() if T.parse_file_name(p.name) is not None]
+    assert len(files) >= 60
+    assert 0 < T.load_tuned_configs() <= 1024
