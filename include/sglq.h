@@ -188,6 +188,29 @@ int sglq_w8a8_block_fp8_linear(const void* x, int in_dtype, const void* b, int64
                                int out_dtype, int64_t M, int64_t N, int64_t K, float eps, void* workspace,
                                int64_t workspace_bytes, void* stream);
 
+/* The call pairs of the per-token linears as one entry point each:
+ *   sglq_w8a8_int8_linear  per_token_quant_int8 + int8_scaled_mm, W8A8Int8LinearMethod.apply
+ *                          (python/sglang/srt/layers/quantization/w8a8_int8.py:387-391);
+ *   sglq_w8a8_fp8_linear   sgl_per_token_quant_fp8 + fp8_scaled_mm, apply_fp8_linear's dynamic per-token
+ *                          branch (python/sglang/srt/layers/quantization/fp8_utils.py:693,725-732).
+ * The fused form is the one the reference's CPU backend has, int8_scaled_mm_with_quant
+ * (sgl-kernel/csrc/cpu/gemm_int8.cpp:423-489).
+ *   x    [M, K] contiguous activations, in_dtype in {BF16, FP16, FP32}, 16-byte aligned
+ *   b, scales_b, bias (may be NULL), out: as sglq_int8_scaled_mm / sglq_fp8_scaled_mm
+ * For M <= 2 (16-bit activations, K % 128 == 0) on the shapes that the decode kernel without
+ * split-K takes, one kernel forms the rows' scales in its prologue and quantizes each K block's
+ * activations in LDS right before multiplying them: no quantization launch, no round trip of codes
+ * and scales through memory, no workspace.  Other shapes run the quantization kernel and the GEMM
+ * one after the other; their codes and row scales need M * K + 4 * M bytes (each rounded up to
+ * 256) at the head of the 16-byte aligned workspace, the rest serves the GEMM's split-K as usual.
+ * The output is bit-identical to the two operators called in turn. */
+int sglq_w8a8_int8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* scales_b,
+                          const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+int sglq_w8a8_fp8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* scales_b,
+                         const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
 /* No counterpart in the reference.  sglq_fp8_blockwise_scaled_mm for callers that cannot
  * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
  * forbid it) and therefore have no workspace to pass: the split-K partial sums go through a

@@ -40,6 +40,10 @@ SIGNATURES = {
     "sglq_init": [],
     "sglq_w8a8_block_fp8_linear": [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int,
                                    c_int64, c_int64, c_int64, c_float, c_void_p, c_int64, c_void_p],
+    "sglq_w8a8_int8_linear": [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64,
+                              c_void_p, c_int64, c_void_p],
+    "sglq_w8a8_fp8_linear": [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64,
+                             c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_bias": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                           c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_grouped_mm": [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p,

@@ -2254,6 +2254,236 @@ __global__ __launch_bounds__(256) void gemm_stream_quant_kernel(const GemmArgs p
   }
 }
 
+// ---------------------------------------------------------------------------
+// gemm_stream_kernel for M <= 8 with the per-token (per-row) activation quantization folded in, for the
+// per-row / per-column scaled kinds: p.a holds the 16-bit activations (row stride p.lda BYTES).  A row's
+// scale needs the whole row, so every block first reads its ROWS rows once (they come from L2 for every
+// block but the first) and forms the rows' abs-max: 256 lanes stride over a row's 16-byte chunks, packed
+// 16-bit integer max on the sign-stripped bit patterns, wave max, the four waves' values meet in LDS.  The
+// first ring stages (weights and raw activations) are issued before that pass, so the weight stream starts
+// with the kernel.  From the row maximum:
+//   FP8  scale = max / 448, inv = scale == 0 ? 0 : 1 / scale, q = e4m3(clamp(x * inv))      (token_quant_kernel,
+//   INT8 scale = max(max, 1e-10) / 127, mul = 127 / max(max, 1e-10), q = clamp(round(x * mul))  quant.hip)
+// with the same expressions as the quantization kernel: bit-identical codes and scales.  The K loop is that
+// of gemm_stream_quant_kernel (raw activations through the wave's ring, quantized into a wave-private
+// 8 x 128-byte tile in the MFMA operand layout) with the accumulation of gemm_stream_kernel<KIND, 1, NIB>
+// in place, and wave 0's epilogue takes the row scale from its register: the output equals
+// quantize-then-multiply through that kernel bit for bit.
+// ---------------------------------------------------------------------------
+template <int KIND, int NIB, int OUT_DT, int IN_DT, int ROWS>
+__global__ __launch_bounds__(256) void gemm_stream_tokenquant_kernel(const GemmArgs p) {
+  static_assert(KIND == KIND_FP8_ROWCOL || KIND == KIND_I8_ROWCOL, "per-row / per-column scaled kinds");
+  constexpr bool IS_FP8 = KIND == KIND_FP8_ROWCOL;
+  constexpr int BN = NIB * 16, XR = 8;
+  constexpr int WC = BN / 8, XC = XR * 256 / 1024;  // one-KiB copies per stage: weights, activations
+  constexpr int CPW = WC + XC;
+  constexpr int W_BYTES = BN * 128, X_BYTES = XR * 256;
+  constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
+  constexpr int NSTAGE = SGLQ_STREAM_NSTAGE;
+  constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+  constexpr int TILE_BYTES = 8 * 128;  // the quantized activations of the current K block
+  constexpr int LPR = 64 / ROWS, EPL = 128 / LPR, WPL = EPL / 2;  // lanes per row, elements and 32-bit words per lane
+  static_assert(ROWS == 1 || ROWS == 2 || ROWS == 4 || ROWS == 8, "rows per wave");
+  static_assert((NSTAGE - 1) * CPW <= 63, "vmcnt holds 6 bits");
+  static_assert(NIB * 1024 <= RING_BYTES, "the partial sums are exchanged through a wave's ring");
+
+  // (one LDS object: rings, the waves' code tiles, then the waves' row maxima)
+  __shared__ __attribute__((aligned(1024))) char smem[4 * (RING_BYTES + TILE_BYTES) + 4 * ROWS * 4];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4, l8 = lane >> 3;
+  const int n0 = blockIdx.x * BN;
+  const int nkb = p.K >> 7;
+  const int nsteps = (nkb - wave + 3) >> 2;  // K blocks wave, wave + 4, ...
+
+  const v4u rx = make_rsrc_sgpr(p.a, p.a_bytes);
+  const v4u rb = make_rsrc_sgpr(p.b, p.b_bytes);
+
+  const int c16_even = (((lane & 7) ^ l8) & 7) * 16, c16_odd = (((lane & 7) ^ l8 ^ 1) & 7) * 16;
+  const uint32_t offw_even = (uint32_t)(n0 + l8) * p.ldb + c16_even, offw_odd = (uint32_t)(n0 + l8) * p.ldb + c16_odd;
+  const uint32_t step_w = 8u * p.ldb;
+  const uint32_t x_piece = (uint32_t)(lane & 15) * 16u;
+  uint32_t offx[XC];
+#pragma unroll
+  for (int j = 0; j < XC; ++j) {
+    const int row = 4 * j + (lane >> 4);
+    offx[j] = row < p.M ? (uint32_t)row * p.lda + x_piece : OOB;
+  }
+
+  const uint32_t ring = lds_addr(smem) + (uint32_t)wave * RING_BYTES;
+  auto issue_group = [&](int t) {  // all copies of this wave's t-th K block into slot t % NSTAGE
+    const uint32_t st = ring + (uint32_t)(t % NSTAGE) * STAGE_BYTES;
+    const uint32_t kb = (uint32_t)(wave + 4 * t);
+    const uint32_t kill = t < nsteps ? 0u : OOB;  // past the end: out of range, the K offset is not bounds-checked
+    const uint32_t k0 = t < nsteps ? kb * 128u : 0u;
+#pragma unroll
+    for (int j = 0; j < WC; ++j)
+      lds_copy16(rb, st + j * 1024, (((j & 1) ? offw_odd : offw_even) + j * step_w) | kill, k0);
+#pragma unroll
+    for (int j = 0; j < XC; ++j) lds_copy16(rx, st + W_BYTES + j * 1024, offx[j] | kill, k0 * 2u);
+  };
+
+  const int sw = (r16 & 7) ^ (r16 >> 3);
+  const int lane_off0 = r16 * 128 + (((2 * g) ^ sw) * 16);
+  const int lane_off1 = lane_off0 ^ 16;
+  auto read_frag = [&](const char* q) -> v8i {
+    v4i lo = *reinterpret_cast<const v4i*>(q + lane_off0);
+    v4i hi = *reinterpret_cast<const v4i*>(q + lane_off1);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  using acc_t = typename std::conditional<IS_FP8, v4f, v4i>::type;
+  acc_t acc[NIB];
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) acc[j] = acc_t{0, 0, 0, 0};
+
+  char* my_ring = smem + wave * RING_BYTES;
+  char* my_tile = smem + 4 * RING_BYTES + wave * TILE_BYTES;
+  uint32_t* red = reinterpret_cast<uint32_t*>(smem + 4 * (RING_BYTES + TILE_BYTES));
+  const int t_row = r16 & (ROWS - 1);
+  const int tile_off0 = t_row * 128 + (((2 * g) ^ t_row) * 16), tile_off1 = tile_off0 ^ 16;
+  const int q_row = lane / LPR, q_first = (lane % LPR) * EPL;
+  const int q_src = q_row * 256 + q_first * 2;
+  const int q_dst = q_row * 128 + ((((q_first >> 4) ^ q_row) & 7) * 16) + (q_first & 15);
+
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t) issue_group(t);
+
+  // ---- the rows' abs-max: every lane of the block strides over the 16-byte chunks of each row (rows past M and
+  // chunks past K are out of range and read as zero)
+  {
+    const __amdgpu_buffer_rsrc_t rxa = make_rsrc(p.a, p.a_bytes);
+    const uint32_t chunks = (uint32_t)p.K >> 3;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      v2us m16 = {0, 0};
+      for (uint32_t c0 = 0; c0 < chunks; c0 += 1024) {
+        v4u raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t c = c0 + (uint32_t)u * 256u + threadIdx.x;
+          raw[u] = __builtin_amdgcn_raw_buffer_load_b128(rxa, c < chunks ? (uint32_t)r * p.lda + c * 16u : OOB, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) m16 = __builtin_elementwise_max(m16, __builtin_bit_cast(v2us, raw[u][i] & 0x7fff7fffu));
+      }
+      const uint32_t hmax = wave_umax(m16.x > m16.y ? (uint32_t)m16.x : (uint32_t)m16.y);
+      if (lane == 0) red[wave * ROWS + r] = hmax;
+    }
+  }
+  __syncthreads();
+  // scale and multiplier of a row, from the same expressions as token_quant_kernel
+  auto row_scale = [&](int r, float& scale, float& mul) {
+    const uint32_t hmax = umax(umax(red[r], red[ROWS + r]), umax(red[2 * ROWS + r], red[3 * ROWS + r]));
+    const float amax_x = to_f32_16<IN_DT>((uint16_t)hmax);
+    if constexpr (IS_FP8) {
+      scale = amax_x / 448.0f;
+      mul = (scale == 0.f) ? 0.f : 1.0f / scale;
+    } else {
+      const float amax = u2f(umax(f2u(amax_x), f2u(1e-10f)));
+      scale = amax / 127.0f;
+      mul = 127.0f / amax;
+    }
+  };
+  float q_scale, q_mul, out_scale, out_mul;
+  row_scale(q_row, q_scale, q_mul);
+  row_scale(t_row, out_scale, out_mul);
+
+  for (int t = 0; t < nsteps; ++t) {
+    issue_group(t + NSTAGE - 1);
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * CPW) : "memory");
+
+    const char* st = my_ring + (t % NSTAGE) * STAGE_BYTES;
+    // ---- quantization of this K block's ROWS x 128 activations with the rows' scales
+    uint32_t w[WPL];
+    {
+      const char* src = st + W_BYTES + q_src;
+      if constexpr (WPL == 8) {
+        const v4u lo = *reinterpret_cast<const v4u*>(src), hi = *reinterpret_cast<const v4u*>(src + 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = lo[i], w[4 + i] = hi[i];
+      } else if constexpr (WPL == 4) {
+        const v4u lo = *reinterpret_cast<const v4u*>(src);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = lo[i];
+      } else if constexpr (WPL == 2) {
+        const v2u lo = *reinterpret_cast<const v2u*>(src);
+        w[0] = lo.x, w[1] = lo.y;
+      } else {
+        w[0] = *reinterpret_cast<const uint32_t*>(src);
+      }
+    }
+    uint32_t codes[(EPL + 3) / 4];
+#pragma unroll
+    for (int i = 0; i < (EPL + 3) / 4; ++i) codes[i] = 0;
+#pragma unroll
+    for (int i = 0; i < WPL; ++i) {
+      float lo = to_f32_16<IN_DT>((uint16_t)(w[i] & 0xffffu)) * q_mul;
+      float hi = to_f32_16<IN_DT>((uint16_t)(w[i] >> 16)) * q_mul;
+      if constexpr (IS_FP8) {
+        lo = clampf(lo, -448.0f, 448.0f);
+        hi = clampf(hi, -448.0f, 448.0f);
+        if (i & 1) codes[i >> 1] = cvt_pk_e4m3<true>(lo, hi, codes[i >> 1]);
+        else codes[i >> 1] = cvt_pk_e4m3<false>(lo, hi, 0);
+      } else {
+        const uint32_t blo = (uint32_t)(int)clampf(__builtin_roundf(lo), -128.0f, 127.0f) & 0xffu;
+        const uint32_t bhi = (uint32_t)(int)clampf(__builtin_roundf(hi), -128.0f, 127.0f) & 0xffu;
+        codes[i >> 1] |= (blo | (bhi << 8)) << ((i & 1) * 16);
+      }
+    }
+    if constexpr (EPL == 16) *reinterpret_cast<v4u*>(my_tile + q_dst) = v4u{codes[0], codes[1], codes[2], codes[3]};
+    else if constexpr (EPL == 8) *reinterpret_cast<v2u*>(my_tile + q_dst) = v2u{codes[0], codes[1]};
+    else if constexpr (EPL == 4) *reinterpret_cast<uint32_t*>(my_tile + q_dst) = codes[0];
+    else *reinterpret_cast<uint16_t*>(my_tile + q_dst) = (uint16_t)codes[0];
+
+    v8i wf[NIB];
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) wf[j] = read_frag(st + j * 16 * 128);
+    const v4i alo = *reinterpret_cast<const v4i*>(my_tile + tile_off0), ahi = *reinterpret_cast<const v4i*>(my_tile + tile_off1);
+    const v8i af = v8i{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) {
+      if constexpr (IS_FP8) {
+        acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[j], af, acc[j], 0, 0, 0, 0, 0, 0);
+      } else {
+        const v4i b0 = {wf[j][0], wf[j][1], wf[j][2], wf[j][3]}, b1 = {wf[j][4], wf[j][5], wf[j][6], wf[j][7]};
+        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, alo, acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, ahi, acc[j], 0, 0, 0);
+      }
+    }
+  }
+
+  // as gemm_stream_kernel: waves 1..3 leave their partial sums in their own ring, wave 0 adds them in wave order
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  if (wave != 0) {
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) *reinterpret_cast<acc_t*>(my_ring + j * 1024 + lane * 16) = acc[j];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+#pragma unroll
+      for (int j = 0; j < NIB; ++j) {
+        const acc_t t = *reinterpret_cast<const acc_t*>(smem + w * RING_BYTES + j * 1024 + lane * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[j][e] += t[e];
+      }
+    int r = r16, gg = g;
+    asm volatile("" : "+v"(r), "+v"(gg));
+    if (r < p.M) {
+#pragma unroll
+      for (int j = 0; j < NIB; ++j) {
+        const int n = n0 + j * 16 + gg * 4;
+        if (n < p.N) finish4<KIND, OUT_DT>(p, r, n, acc[j], out_scale);
+      }
+    }
+  }
+}
+
 // Sum the split-K partials in split order and apply the epilogue; one thread per
 // run of four consecutive n.
 template <int KIND, int OUT_DT>
@@ -3405,6 +3635,124 @@ extern "C" int sglq_w8a8_block_fp8_linear(const void* x, int in_dtype, const voi
   if (rc) return rc;
   return blockwise_entry<KIND_FP8_BLOCK>(name, ws, K, b, ldb, scales, 1, M, sfb, sfb_stride_k, sfb_stride_n, bias, out, ldo, out_dtype,
                                          M, N, K, ws + code_bytes + scale_bytes, workspace_bytes - code_bytes - scale_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------
+// Quantize-and-multiply in one call for the per-token kinds: per-token INT8 quantization + int8_scaled_mm
+// (the pair of calls of W8A8Int8LinearMethod.apply, w8a8_int8.py:387-391) and per-token FP8 quantization +
+// fp8_scaled_mm (apply_fp8_linear's dynamic per-token branch, fp8_utils.py:693,725-732); the fused form is the
+// reference's CPU backend's int8_scaled_mm_with_quant (sgl-kernel/csrc/cpu/gemm_int8.cpp:423-489).  For decode
+// rows on the shapes that the full-K decode kernel takes, one launch does both
+// (gemm_stream_tokenquant_kernel); otherwise the two kernels run one after the other with the codes and the
+// row scales at the head of the workspace.  Either way the output is bit-identical to the two operators
+// called in turn.
+// ---------------------------------------------------------------------------
+template <int KIND, int OUT_DT>
+static void launch_stream_tokenquant(GemmArgs& p, int nib, int in_dtype, hipStream_t st) {
+  p.splits = 1;
+  p.tiles_m = 1;
+  p.tiles_n = (p.N + 16 * nib - 1) / (16 * nib);
+  const dim3 grid((uint32_t)p.tiles_n), block(256);
+  g_last_kernel = nib == 1 ? "gemm_stream_tokenquant_kernel<16 rows>" : "gemm_stream_tokenquant_kernel<32 rows>";
+  auto launch = [&](auto nib_tag, auto in_tag) {
+    constexpr int NIB = decltype(nib_tag)::value, IN_DT = decltype(in_tag)::value;
+    if (p.M <= 1) gemm_stream_tokenquant_kernel<KIND, NIB, OUT_DT, IN_DT, 1><<<grid, block, 0, st>>>(p);
+    else if (p.M <= 2) gemm_stream_tokenquant_kernel<KIND, NIB, OUT_DT, IN_DT, 2><<<grid, block, 0, st>>>(p);
+    else if (p.M <= 4) gemm_stream_tokenquant_kernel<KIND, NIB, OUT_DT, IN_DT, 4><<<grid, block, 0, st>>>(p);
+    else gemm_stream_tokenquant_kernel<KIND, NIB, OUT_DT, IN_DT, 8><<<grid, block, 0, st>>>(p);
+  };
+  using one = std::integral_constant<int, 1>;
+  using two = std::integral_constant<int, 2>;
+  using bf16 = std::integral_constant<int, SGLQ_BF16>;
+  using fp16 = std::integral_constant<int, SGLQ_FP16>;
+  if (in_dtype == SGLQ_BF16) {
+    if (nib == 1) launch(one{}, bf16{});
+    else launch(two{}, bf16{});
+  } else {
+    if (nib == 1) launch(one{}, fp16{});
+    else launch(two{}, fp16{});
+  }
+}
+
+// Rows up to which the single kernel is taken without the test hook (see the measurements in tokenquant_linear_entry)
+#ifndef SGLQ_TOKENQUANT_FUSED_ROWS
+#define SGLQ_TOKENQUANT_FUSED_ROWS 2
+#endif
+
+template <int KIND>
+static int tokenquant_linear_entry(const char* name, const void* x, int in_dtype, const void* b, int64_t ldb,
+                                   const float* scales_b, const void* bias, void* out, int64_t ldo, int out_dtype,
+                                   int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                   void* stream) {
+  constexpr bool IS_FP8 = KIND == KIND_FP8_ROWCOL;
+  if (in_dtype != SGLQ_BF16 && in_dtype != SGLQ_FP16 && in_dtype != SGLQ_FP32) {
+    set_error("%s: activations must be BFloat16, Half or Float", name);
+    return SGLQ_EUNSUPPORTED;
+  }
+  // (x stands in for the codes: same row count, contiguous rows of K elements)
+  int rc = gemm_common_checks(name, x, K, b, ldb, out, ldo, M, N, K, 2);
+  if (rc < 0) return SGLQ_OK;
+  if (rc) return rc;
+  if (!scales_b) {
+    set_error("%s: null scale pointer", name);
+    return SGLQ_EINVAL;
+  }
+  if (reinterpret_cast<uintptr_t>(scales_b) & 15) {
+    set_error("%s: scales_b must be 16-byte aligned", name);
+    return SGLQ_EINVAL;
+  }
+  if (out_dtype != SGLQ_BF16 && out_dtype != SGLQ_FP16) {
+    set_error("%s: out_dtype must be Half or BFloat16", name);
+    return SGLQ_EINVAL;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M <= 8 && in_dtype != SGLQ_FP32 && K % 128 == 0 && M * K * 2 < (1ll << 31)) {
+    GemmArgs p;
+    fill_common(p, x, K, b, ldb, out, ldo, M, N, K);
+    p.sb = scales_b;
+    p.bias = bias;
+    pick_selection(KIND, p);
+    const int nib = stream_choice<KIND>(p);
+    // Every block reads the M rows once more for their maxima (M K 2 bytes from L2 per block) before its first
+    // MFMA; against that stand the quantization launch (2.4-2.8 us) and the codes' round trip.  A forced 16- or
+    // 32-row block (test hook) takes the single kernel for any M <= 8.
+    const bool pays = g_force_tile != 0 || M <= SGLQ_TOKENQUANT_FUSED_ROWS;
+    if (nib > 0 && pays) {
+      p.lda = (uint32_t)(K * 2);  // row stride of the 16-bit activations in bytes
+      p.a_bytes = (uint32_t)(M * K * 2);
+      if (out_dtype == SGLQ_BF16) launch_stream_tokenquant<KIND, SGLQ_BF16>(p, nib, in_dtype, st);
+      else launch_stream_tokenquant<KIND, SGLQ_FP16>(p, nib, in_dtype, st);
+      return finish(name);
+    }
+  }
+  // two launches: codes [M, K] and the row scales [M] at the head of the workspace
+  const int64_t code_bytes = (M * K + 255) / 256 * 256, scale_bytes = (M * 4 + 255) / 256 * 256;
+  if (!workspace || workspace_bytes < code_bytes + scale_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15)) {
+    set_error("%s: a 16-byte aligned workspace of at least %lld bytes is needed for the quantized activations of this shape (%lld given)",
+              name, (long long)(code_bytes + scale_bytes), (long long)workspace_bytes);
+    return SGLQ_EINVAL;
+  }
+  char* ws = static_cast<char*>(workspace);
+  float* scales = reinterpret_cast<float*>(ws + code_bytes);
+  if (IS_FP8) rc = sglq_per_token_quant_fp8(x, in_dtype, ws, scales, M, K, stream);
+  else rc = sglq_per_token_quant_int8(x, in_dtype, ws, scales, nullptr, M, K, stream);
+  if (rc) return rc;
+  return rowcol_entry(name, IS_FP8, ws, K, b, ldb, scales, scales_b, bias, out, ldo, out_dtype, M, N, K, ws + code_bytes + scale_bytes,
+                      workspace_bytes - code_bytes - scale_bytes, stream);
+}
+
+extern "C" int sglq_w8a8_int8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* scales_b,
+                                     const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N,
+                                     int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+  return tokenquant_linear_entry<KIND_I8_ROWCOL>("w8a8_int8_linear", x, in_dtype, b, ldb, scales_b, bias, out, ldo, out_dtype, M, N, K,
+                                                 workspace, workspace_bytes, stream);
+}
+
+extern "C" int sglq_w8a8_fp8_linear(const void* x, int in_dtype, const void* b, int64_t ldb, const float* scales_b,
+                                    const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N,
+                                    int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+  return tokenquant_linear_entry<KIND_FP8_ROWCOL>("w8a8_fp8_linear", x, in_dtype, b, ldb, scales_b, bias, out, ldo, out_dtype, M, N, K,
+                                                  workspace, workspace_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------

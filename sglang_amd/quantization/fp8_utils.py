@@ -9,7 +9,7 @@ from typing import List, Optional
 import torch
 
 from ..sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
-from ..sgl_kernel.gemm import block_fp8_linear, fp8_blockwise_scaled_mm_bias
+from ..sgl_kernel.gemm import block_fp8_linear, fp8_blockwise_scaled_mm_bias, fp8_linear
 from .fp8_kernel import (
     per_token_group_quant_fp8,
     per_token_group_quant_fp8_pow2,
@@ -24,6 +24,9 @@ from .fp8_kernel import (
 # Rows up to which w8a8_block_fp8_linear hands quantization and GEMM to one operator: the single
 # fused decode kernel is chosen for up to 4 rows (measured; beyond that two launches are faster).
 FUSED_QUANT_MAX_ROWS = 4
+# ... and up to which apply_fp8_linear's dynamic per-token branch does (sglq_w8a8_fp8_linear: every block of
+# the fused kernel reads the rows once more for their maxima, which pays for one or two rows)
+FUSED_TOKEN_QUANT_MAX_ROWS = 2
 
 
 def w8a8_block_fp8_linear(
@@ -126,6 +129,13 @@ def apply_fp8_linear(
         assert input_scale.numel() == 1
         qinput, x_scale = static_quant_fp8(input_2d.contiguous(), input_scale, repeat_scale=True)
     else:
+        rows = input_2d.shape[0]
+        if (0 < rows <= FUSED_TOKEN_QUANT_MAX_ROWS and input.is_cuda and input.dtype in (torch.bfloat16, torch.float16)
+                and input_2d.shape[1] % 128 == 0 and weight.stride(0) == 1 and weight_scale.numel() == weight.shape[1] and weight.shape[1] > 1):
+            # decode rows: quantization and GEMM in one operator (a single kernel on the decode kernel's shapes),
+            # bit-identical to the two calls below
+            ws = weight_scale if weight_scale.dtype == torch.float32 and weight_scale.is_contiguous() else weight_scale.to(torch.float32).contiguous()
+            return fp8_linear(input_2d.contiguous(), weight, ws, bias).view(*output_shape)
         qinput, x_scale = sglang_per_token_quant_fp8(input_2d.contiguous())
     m, n = qinput.shape[0], weight.shape[1]
     if x_scale.numel() == 1 and m != 1:

@@ -264,6 +264,49 @@ def block_fp8_linear(input_2d, mat_b, scales_b, bias=None, eps=1e-10):
     return out
 
 
+def _token_quant_linear(fn_name, elem_dtype, elem_name, input_2d, mat_b, scales_b, bias):
+    _check(input_2d.is_cuda and mat_b.is_cuda and scales_b.is_cuda, "tensors must be CUDA tensors")
+    _check(input_2d.dim() == 2 and input_2d.is_contiguous(), "input must be a contiguous 2D tensor")
+    _check(mat_b.dim() == 2 and mat_b.stride(0) == 1 and mat_b.dtype == elem_dtype, f"mat_b must be a column major {elem_name} tensor")
+    _check(input_2d.dtype in (torch.bfloat16, torch.float16), "input must be BFloat16 or Half (the output takes its dtype)")
+    m, k = input_2d.shape
+    n = mat_b.size(1)
+    _check(mat_b.size(0) == k, "input and mat_b shapes cannot be multiplied")
+    _check(k % 16 == 0, "mat_b must be multiple of 16 bytes for memory alignment")
+    _check((n * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    _check(n <= 1 or mat_b.stride(1) % 16 == 0, "mat_b column stride must be a multiple of 16 bytes")
+    _check(scales_b.dtype == torch.float32 and scales_b.is_contiguous() and scales_b.numel() == n, "scales_b must be a contiguous Float32 tensor of N elements")
+    out_dtype = input_2d.dtype
+    if bias is not None:
+        _check(bias.is_cuda and bias.is_contiguous() and bias.numel() == n and bias.dtype == out_dtype,
+               "bias must be a contiguous CUDA tensor of N elements in the output dtype")
+    out = torch.empty((m, n), dtype=out_dtype, device=input_2d.device)
+    if m == 0 or n == 0:
+        return out
+    rc = getattr(_lib.load(), fn_name)(
+        input_2d.data_ptr(), DTYPE_CODE[input_2d.dtype], mat_b.data_ptr(), mat_b.stride(1) if n > 1 else k,
+        scales_b.data_ptr(), None if bias is None else bias.data_ptr(), out.data_ptr(), out.stride(0), DTYPE_CODE[out_dtype],
+        m, n, k, *_lib.workspace(input_2d.device), _lib.stream_ptr(input_2d.device))
+    _lib.check(rc, fn_name[5:])
+    return out
+
+
+def int8_linear(input_2d, mat_b, scales_b, bias=None):
+    """per_token_quant_int8(input_2d) followed by int8_scaled_mm (the pair of calls of
+    W8A8Int8LinearMethod.apply, w8a8_int8.py:387-391) as one operator, the fused form of the reference's
+    CPU backend (int8_scaled_mm_with_quant, sgl-kernel/csrc/cpu/gemm_int8.cpp:423-489).  For decode rows on
+    the shapes of the decode kernel without split-K it is a single launch, otherwise the two kernels run one
+    after the other.  input_2d [M, K] contiguous bfloat16 or half; mat_b [K, N] column-major int8; scales_b
+    [N] or [N, 1] fp32; the output has input_2d's dtype.  Bit-identical to the operators called in turn."""
+    return _token_quant_linear("sglq_w8a8_int8_linear", torch.int8, "Int8", input_2d, mat_b, scales_b, bias)
+
+
+def fp8_linear(input_2d, mat_b, scales_b, bias=None):
+    """sgl_per_token_quant_fp8(input_2d) followed by fp8_scaled_mm (apply_fp8_linear's dynamic per-token
+    branch, fp8_utils.py:693,725-732) as one operator; see int8_linear.  mat_b [K, N] column-major e4m3fn."""
+    return _token_quant_linear("sglq_w8a8_fp8_linear", FP8, "Float8_e4m3fn", input_2d, mat_b, scales_b, bias)
+
+
 def _group_quant_impl(fn_name, q_dtype, input, output_q, output_s, group_size, eps, qmin, qmax):
     check_group_quant(input, output_q, output_s, group_size, q_dtype)
     if input.numel() == 0:
