@@ -146,7 +146,8 @@ int sglq_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int6
  * ceil_to_ue8m0 produces, python/sglang/srt/layers/quantization/fp8_utils.py:485-486).  It stands in for the
  * DeepGEMM call of the reference's w8a8_block_fp8_matmul_deepgemm (fp8_kernel.py; a third-party kernel there),
  * whose caller deepgemm_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:214-258) quantizes with such scales.
- * Same arguments, layouts and checks as sglq_fp8_blockwise_scaled_mm, same result for such scales.  For bf16
+ * Same arguments, layouts and checks as sglq_fp8_blockwise_scaled_mm; for such scales the same sums formed in
+ * another order (within one unit of the 16-bit output of that entry point's result, not bit-identical).  For bf16
  * outputs on the shapes of the 256- and 128-row pipelined kernels (roughly M > 128) the matrix instruction
  * applies the scales itself (v_mfma_scale_f32_16x16x128_f8f6f4 takes one exponent byte per lane and operand)
  * and accumulates in place; only the exponent bits of the scales are read there, so a scale that is not a
@@ -216,8 +217,11 @@ int sglq_w8a8_fp8_linear(const void* x, int in_dtype, const void* b, int64_t ldb
  * forbid it) and therefore have no workspace to pass: the split-K partial sums go through a
  * fixed device array of SGLQ_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held
  * until the process ends) and the call allocates nothing.  Same arguments, checks and results
- * as sglq_fp8_blockwise_scaled_mm called with a workspace of that size.  Problems with
- * M * N > SGLQ_NOALLOC_MAX_OUTPUTS are rejected with SGLQ_EINVAL.  All calls on one GPU share
+ * as sglq_fp8_blockwise_scaled_mm called with a workspace of that size: K is split (and the
+ * array used) only for outputs of up to SGLQ_NOALLOC_MAX_OUTPUTS elements, two fp32 partial sums
+ * each; larger outputs run unsplit without touching the array, and sizes beyond the library's
+ * limits (an operand of 2 GiB or more, 2^30 rows or columns) are rejected with SGLQ_EUNSUPPORTED
+ * and a message, before anything is launched.  All calls on one GPU share
  * that GPU's array: calls that overlap on one GPU (two streams, two threads) race on the
  * partial sums and must be serialised by the caller; calls in sequence on one stream are safe
  * (the array needs no clearing between calls).  The array's address is resolved per device on

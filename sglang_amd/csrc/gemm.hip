@@ -37,7 +37,8 @@ constexpr int KIND_I8_BLOCK = 4;    // block-scaled INT8: sum_kb float(P_kb) * s
 // KIND_FP8_BLOCK whose scales are all powers of two (UE8M0 values held as fp32): the MFMA applies them itself
 // (v_mfma_scale_f32_16x16x128_f8f6f4 takes an exponent byte per lane for each operand) and accumulates in place,
 // so there is no scale-and-accumulate pass behind every MFMA.  Only the 256- and 128-row pipelined kernels are
-// built for it; everywhere else such scales run as KIND_FP8_BLOCK, with the same result.
+// built for it; everywhere else such scales run as KIND_FP8_BLOCK (the same sums folded per K block: equal to the
+// in-place accumulation up to the order of the additions, not bit for bit).
 constexpr int KIND_FP8_BLOCK_POW2 = 5;
 
 constexpr bool is_block(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_I8_BLOCK || kind == KIND_FP8_BLOCK_POW2; }
@@ -3537,9 +3538,11 @@ extern "C" int sglq_int8_mm_i32(const void* a, int64_t lda, const void* b, int64
 // ---------------------------------------------------------------------------
 // Quantize-and-multiply in one call: per-token-group FP8 quantization (groups of 128) of 16-bit
 // activations followed by the block-scaled FP8 GEMM, the pair of calls of
-// cutlass_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:204-209).  For up to 8 rows on the
-// shapes that the full-K decode kernel takes, one launch does both (gemm_stream_quant_kernel);
-// otherwise the two kernels run one after the other with the codes and scales in the workspace.
+// cutlass_w8a8_block_fp8_linear_with_fallback (fp8_utils.py:204-209).  For M <= 4 on the shapes that the
+// full-K decode kernel takes with one to 2.5 blocks per compute unit, one launch does both
+// (gemm_stream_quant_kernel; for M <= 8 on any of that kernel's shapes when a 16- or 32-row block is forced
+// through the test hook); otherwise the two kernels run one after the other with the codes and scales in the
+// workspace.
 // Either way the output is bit-identical to the two operators called in turn.
 // ---------------------------------------------------------------------------
 template <int OUT_DT>
@@ -3804,13 +3807,11 @@ extern "C" int sglq_fp8_blockwise_scaled_mm_noalloc(const void* a, int64_t lda, 
                                                     void* out, int64_t ldo, int out_dtype, int64_t M, int64_t N,
                                                     int64_t K, void* stream) {
   const char* name = "fp8_blockwise_scaled_mm_noalloc";
-  // two fp32 partial sums per output must fit, so that split-K (the reason for the scratch) can apply
-  if (M > 0 && N > 0 && M * N > SGLQ_NOALLOC_MAX_OUTPUTS) {
-    set_error("%s: M * N = %lld exceeds the %lld outputs that the %lld-byte device scratch serves; use "
-              "sglq_fp8_blockwise_scaled_mm with a caller-owned workspace",
-              name, (long long)(M * N), (long long)SGLQ_NOALLOC_MAX_OUTPUTS, (long long)SGLQ_NOALLOC_SCRATCH_BYTES);
-    return SGLQ_EINVAL;
-  }
+  // The scratch holds split-K partial sums: two fp32 per output must fit for K to be split at all, i.e. up to
+  // SGLQ_NOALLOC_MAX_OUTPUTS outputs.  Larger outputs run unsplit and do not touch the scratch (the launchers fall
+  // back to one split when the workspace is too small, exactly as the workspace entry point does with a workspace
+  // of this size), so they are served as well; sizes beyond what the library addresses at all (operands of 2 GiB,
+  // 2^30 rows or columns) are rejected by the common checks with their message.
   void* ws = nullptr;
   const int rc = scratch_of_current_device(name, &ws);
   if (rc) return rc;

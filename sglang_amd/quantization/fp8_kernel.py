@@ -240,6 +240,29 @@ def unpack_ue8m0_scales(x_s: torch.Tensor, num_groups: int) -> torch.Tensor:
     return (e.reshape(x_s.shape[0], -1)[:, :num_groups] << 23).contiguous().view(torch.float32)
 
 
+# weights whose block scales have been checked to be powers of two: (data_ptr, shape, version counter)
+_pow2_checked = set()
+
+
+def check_pow2_scales(Bs: torch.Tensor, what: str = "Bs") -> None:
+    """Raise unless every fp32 scale is a power of two (no mantissa bits, positive): the kernels behind
+    w8a8_block_fp8_matmul_deepgemm read only the exponent of a scale on the shapes where the matrix instruction
+    applies it, so other values would be rounded down there and used in full elsewhere, with no error.  Checked
+    once per tensor (address, shape and version counter; one device round trip), not under stream capture."""
+    key = (Bs.device.type, Bs.data_ptr(), tuple(Bs.shape), Bs._version)
+    if key in _pow2_checked:
+        return
+    if Bs.is_cuda and torch.cuda.is_current_stream_capturing():
+        return
+    bits = Bs.contiguous().view(torch.int32)
+    if bool(((bits & 0x7FFFFF) != 0).any()) or bool((bits <= 0).any()):
+        raise ValueError(f"w8a8_block_fp8_matmul_deepgemm: {what} holds scales that are not powers of two; the weight must go "
+                         "through requant_weight_ue8m0_inplace (or per_block_cast_to_fp8) first")
+    if len(_pow2_checked) > 4096:
+        _pow2_checked.clear()
+    _pow2_checked.add(key)
+
+
 def w8a8_block_fp8_matmul_deepgemm(
     A: torch.Tensor,
     B: torch.Tensor,
@@ -270,6 +293,7 @@ def w8a8_block_fp8_matmul_deepgemm(
     assert -(-N // 128) == Bs.shape[0] and K // 128 == Bs.shape[1]
     if Bs.dtype != torch.float32:
         raise NotImplementedError("w8a8_block_fp8_matmul_deepgemm: Bs must be Float32 powers of two [N/128, K/128]")
+    check_pow2_scales(Bs)
     C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
     if M == 0 or N == 0:
         return C

@@ -233,8 +233,9 @@ def fp8_blockwise_scaled_mm_bias(mat_a, mat_b, scales_a, scales_b, out_dtype, bi
 
 def block_fp8_linear(input_2d, mat_b, scales_b, bias=None, eps=1e-10):
     """per_token_group_quant_fp8(input_2d, 128) followed by fp8_blockwise_scaled_mm and the caller's
-    bias add (fp8_utils.py:204-211) as one operator; for up to 8 rows on the shapes of the decode
-    kernel without split-K it is a single launch.  input_2d [M, K] contiguous, 16- or 32-bit float;
+    bias add (fp8_utils.py:204-211) as one operator; for M <= 4 on the shapes that the decode kernel
+    without split-K takes with one to 2.5 blocks per compute unit it is a single launch (for M <= 8 only
+    when a 16- or 32-row block is forced through the test hook), otherwise the two kernels in turn.  input_2d [M, K] contiguous, 16- or 32-bit float;
     mat_b [K, N] column-major e4m3fn; scales_b [K/128, N/128] fp32; the output has input_2d's dtype
     (bfloat16 or half).  Bit-identical to the operators called in turn."""
     _check(input_2d.is_cuda and mat_b.is_cuda and scales_b.is_cuda, "tensors must be CUDA tensors")

@@ -73,9 +73,11 @@ def test_int8_accumulators_bit_exact(gpu, load_path, tile, mnk):
 @pytest.mark.parametrize("m", [1, 16, 128, 1024])
 def test_int8_scaled_mm_config(gpu, m):
     """A[M,4096] per-token INT8 x B[4096,14336] with per-column scales and bf16 bias."""
+    from sglang_amd import _lib
     from sglang_amd.quantization.int8_kernel import per_token_quant_int8
     from sglang_amd.sgl_kernel import int8_mm_i32, int8_scaled_mm
 
+    lib = _lib.load()
     say("int8_scaled_mm config M", m)
     x = O.gen_activation(m, 4096, seed=1000 + m)
     wt, s_b, bias = O.gen_int8_weight(4096, 14336, seed=1000)
@@ -83,13 +85,26 @@ def test_int8_scaled_mm_config(gpu, m):
     xq, xs = per_token_quant_int8(x.to(gpu))
     assert torch.equal(xq.cpu(), xq_ref) and torch.equal(xs.cpu(), xs_ref)
     wg = wt.t().contiguous().to(gpu).t()  # [K, N] view with stride(0) == 1
-    rows = sample_rows(m, 24)
+    # every INT32 accumulator of the whole output against the oracle (the float64 product is exact here)
     acc = int8_mm_i32(xq, wg).cpu()
-    assert torch.equal(acc[rows], O.int8_mm_i32(xq_ref[rows], wt))
+    acc_ref = O.int8_mm_i32(xq_ref, wt)
+    bad = acc != acc_ref
+    assert not bool(bad.any()), f"{int(bad.sum())} of {acc.numel()} accumulators differ, first {bad.nonzero()[:4].tolist()}"
     for b in (None, bias):
-        out = int8_scaled_mm(xq, wg, xs, s_b.to(gpu), torch.bfloat16, None if b is None else b.to(gpu)).cpu()
-        ref = O.int8_scaled_mm(xq_ref[rows], wt, xs_ref[rows], s_b, torch.bfloat16, b)
-        torch.testing.assert_close(out[rows].float(), ref.float(), rtol=RTOL, atol=ATOL)
+        run = lambda: int8_scaled_mm(xq, wg, xs, s_b.to(gpu), torch.bfloat16, None if b is None else b.to(gpu))
+        out = run()
+        selected = lib.sglq_debug_last_gemm_kernel().decode()
+        # ... and every scaled output: against the oracle's epilogue on those accumulators
+        ref = O.int8_scaled_mm(xq_ref, wt, xs_ref, s_b, torch.bfloat16, b)
+        torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL, msg=lambda s: f"{selected}: {s}")
+        if m >= 512:  # and against the same GEMM on the generic 128 x 128 kernel, as the other configurations' whole-output check
+            lib.sglq_debug_force_tile(128)
+            try:
+                generic = run()
+                assert lib.sglq_debug_last_gemm_kernel().decode().startswith("gemm_kernel")
+            finally:
+                lib.sglq_debug_force_tile(0)
+            torch.testing.assert_close(out.float(), generic.float(), rtol=RTOL, atol=ATOL, msg=lambda s: f"{selected} vs generic kernel: {s}")
 
 
 def make_block_case(m, n, k, seed, outliers=False):

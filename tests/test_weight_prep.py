@@ -1,5 +1,6 @@
 """Load-time helpers of the FP8 / INT8 linear methods (plain torch, CPU): closed forms and brute
 force, no device involved."""
+import pytest
 import torch
 
 from sglang_amd.quantization import fp8_utils as F
@@ -140,3 +141,17 @@ def test_fp8_process_weights_after_loading():
     # block quantization: nothing to do
     ws = torch.ones(1, 1)
     assert P.process_weights_after_loading(q, ws, block_quant=True) == (q, ws, None)
+
+
+def test_pow2_scale_check_rejects_other_scales():
+    """w8a8_block_fp8_matmul_deepgemm reads only the exponents of the weight's block scales where the matrix
+    instruction applies them: scales with mantissa bits (a weight that skipped requant_weight_ue8m0_inplace) must
+    raise instead of being rounded down on some batch sizes and used in full on others."""
+    from sglang_amd.quantization.fp8_kernel import check_pow2_scales
+
+    check_pow2_scales(torch.tensor([[1.0, 0.5], [2.0**-20, 8.0]]))
+    for bad in ([[1.0, 0.75]], [[3e-4, 1.0]], [[0.0, 1.0]], [[-2.0, 1.0]]):
+        with pytest.raises(ValueError, match="powers of two"):
+            check_pow2_scales(torch.tensor(bad))
+    # ceil_to_ue8m0 is what makes a scale pass
+    check_pow2_scales(F.ceil_to_ue8m0(torch.tensor([[3e-4, 0.75]])))
