@@ -241,6 +241,65 @@ def run_launches(args):
     print(json.dumps({"launches": rows, "reps": args.launch_reps, "kind": args.kind}), flush=True)
 
 
+def run_ab(args):
+    """bench.py --ab OTHER.so --launches "M,N,K;...": the block-FP8 GEMM of another build of libsglq.so (for instance
+    one compiled from an earlier commit with the flags of sglang_amd/build.py) against the tree's library in ONE
+    process: the two alternate, four rounds of 60 back-to-back calls each after 60 untimed ones, the shader clock read
+    around every timed block.  One JSON line per (shape, library, round) and whether the outputs are equal bit for bit."""
+    import ctypes
+    from ctypes import c_int, c_int64, c_void_p
+
+    import torch
+
+    dev = torch.device("cuda:0")
+    bk = BenchKernels(dev)
+    sig = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+           c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]
+    libs = []
+    for name, path in (("other", args.ab), ("tree", str(ROOT / "sglang_amd" / "libsglq.so"))):
+        lib = ctypes.CDLL(path)
+        lib.sglq_fp8_blockwise_scaled_mm.argtypes = sig
+        lib.sglq_debug_last_gemm_kernel.restype = ctypes.c_char_p
+        libs.append((name, lib))
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    for i, spec in enumerate(args.launches.split(";")):
+        m, n, k = (int(v) for v in spec.split(","))
+        wq, wsc = make_block_weight(n, k, 7000 + i, dev)
+        g = torch.Generator(device=dev).manual_seed(7100 + i)
+        x = (torch.randn((m, k), generator=g, device=dev) * 2).to(torch.float8_e4m3fn)
+        sa = (torch.rand((k // 128, m), generator=g, device=dev) + 0.5).t()
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        st = torch.cuda.current_stream().cuda_stream
+
+        def call(lib):
+            rc = lib.sglq_fp8_blockwise_scaled_mm(x.data_ptr(), k, wq.data_ptr(), k, sa.data_ptr(), sa.stride(0), sa.stride(1), wsc.data_ptr(),
+                                                  wsc.stride(1), wsc.stride(0), out.data_ptr(), n, 0, m, n, k, ws.data_ptr(), ws.numel(), st)
+            assert rc == 0, rc
+
+        outs = {}
+        for rnd in range(4):
+            for name, lib in libs:
+                for _ in range(60):
+                    call(lib)
+                c0 = bk.clock_sample()
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                for _ in range(60):
+                    call(lib)
+                e.record()
+                c1 = bk.clock_sample()
+                torch.cuda.synchronize()
+                us = s.elapsed_time(e) / 60 * 1e3
+                mhz = bk.clock_mhz(c0, c1)
+                tf = 2.0 * m * n * k / us / 1e6
+                outs[name] = out.clone()
+                print(json.dumps({"library": name, "M": m, "N": n, "K": k, "round": rnd, "kernel": lib.sglq_debug_last_gemm_kernel().decode(),
+                                  "us": round(us, 1), "TFLOPs": round(tf, 1), "clock_mhz": round(mhz),
+                                  "mfma_pipe_utilisation": round(tf * 1e12 / (bk.cus * 8192.0 * max(mhz, 1.0) * 1e6), 3)}), flush=True)
+        print(json.dumps({"M": m, "N": n, "K": k, "outputs_equal": bool(torch.equal(outs["other"], outs["tree"]))}), flush=True)
+        del wq, x, out
+
+
 def run_ceiling(args):
     """bench.py --ceiling: the MFMA pipe's sustained rate under a register-only loop (no memory traffic), for the
     instruction mixes of the two GEMM families and two kinds of operand bytes.  One JSON line."""
@@ -965,6 +1024,8 @@ def main():
     ap.add_argument("--launches", type=str, default=None,
                     help='"M,N,K;M,N,K;...": run these block-FP8 linears as plain launches in this order and exit (for profiler counter runs)')
     ap.add_argument("--launch-reps", type=int, default=5)
+    ap.add_argument("--ab", type=str, default=None, metavar="OTHER.so",
+                    help="with --launches: alternate the block-FP8 GEMM of another build of libsglq.so with the tree's in one process")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="with --launches: rotate the weight over copies of 320 MB and more in total (weights come from HBM every time)")
     ap.add_argument("--kind", type=str, default="block_fp8", choices=("block_fp8", "fp8", "int8"),
@@ -984,7 +1045,9 @@ def main():
               "a tensor-parallel deployment shards N or K per rank and all-reduces outside it). Run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
-    if args.launches:
+    if args.launches and args.ab:
+        run_ab(args)
+    elif args.launches:
         run_launches(args)
     elif args.ceiling:
         run_ceiling(args)
