@@ -99,6 +99,8 @@ class BenchKernels:
         self.lib.sglqb_mfma_ceiling.argtypes = [c.c_int, c.c_int, c.c_void_p, c.c_void_p, c.c_void_p, c.c_int, c.c_void_p]
         self.lib.sglqb_clock_probe.argtypes = [c.c_void_p, c.c_int, c.c_void_p]
         self.lib.sglqb_stream.argtypes = [c.c_int, c.c_void_p, c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_void_p]
+        self.lib.sglqb_lds_fill.argtypes = [c.c_int, c.c_void_p, c.c_int, c.c_int64, c.c_int, c.c_int64, c.c_int, c.c_int, c.c_void_p, c.c_void_p,
+                                            c.c_int, c.c_void_p]
         self.dev = dev
         self.cus = torch.cuda.get_device_properties(dev).multi_processor_count
         self.torch = torch
@@ -298,6 +300,60 @@ def run_ab(args):
                                   "mfma_pipe_utilisation": round(tf * 1e12 / (bk.cus * 8192.0 * max(mhz, 1.0) * 1e6), 3)}), flush=True)
         print(json.dumps({"M": m, "N": n, "K": k, "outputs_equal": bool(torch.equal(outs["other"], outs["tree"]))}), flush=True)
         del wq, x, out
+
+
+def run_fill(args):
+    """bench.py --fill: what the compute units take in through their LDS with the GEMM kernels' global -> LDS copies and
+    nothing else (lds_fill_kernel of libsglq_bench.so: 8 waves per block, one block per CU, every wave keeps stages - 1
+    stages of its own copies in flight, no barrier, no arithmetic), per source of the bytes: windows that stay in the
+    XCDs' L2s, windows shared by four blocks of one XCD, and windows of 2.75 MB per block that come from HBM (the K
+    walk of a 7168-byte row pitch).  One JSON line: per case the median rate per block and the sum over the blocks."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    bk = BenchKernels(dev)
+    cus = bk.cus
+    cases = []
+    for stages in (2, 3):
+        # (label, rows per stage, row pitch, 128-byte steps per row, blocks sharing a window, blocks)
+        cases += [("hbm: a window of 384 rows x 7168 B per block", stages, 384, 7168, 56, 1, cus),
+                  ("hbm, a quarter of the CUs", stages, 384, 7168, 56, 1, cus // 4),
+                  ("four blocks of an XCD share a window of 384 rows x 7168 B (704 MB / 4 in all)", stages, 384, 7168, 56, 4, cus),
+                  ("L2: four blocks share a window of 384 rows x 1024 B (3 MB per XCD)", stages, 384, 1024, 8, 4, cus),
+                  ("L2: a window of 256 rows x 512 B per block (4 MB per XCD)", stages, 256, 512, 4, 1, cus),
+                  ("L2: a window of 128 rows x 512 B per block (2 MB per XCD), 16 KiB stages", stages, 128, 512, 4, 1, cus)]
+    cases += [("L2: a window of 128 rows x 512 B per block (2 MB per XCD), 16 KiB stages", 4, 128, 512, 4, 1, cus),
+              ("hbm: a window of 256 rows x 7168 B per block", 4, 256, 7168, 56, 1, cus)]
+    out = {"what": "global -> LDS copy loop (buffer_load_dwordx4 ... lds, 1 KiB per wave instruction), 8 waves per block, one block per CU, no arithmetic",
+           "cus": cus, "cases": []}
+    for label, stages, rows, pitch, steps, share, blocks in cases:
+        window = ((rows - 1) * pitch + steps * 128 + 4095) // 4096 * 4096
+        windows = -(-blocks // (8 * share)) * 8
+        src = torch.empty(windows * window, dtype=torch.uint8, device=dev)
+        src.random_(0, 255)
+        clocks = torch.zeros(blocks * 2, dtype=torch.int64, device=dev)
+        sink = torch.zeros(blocks, dtype=torch.int32, device=dev)
+        stage_bytes = rows * 128
+        iters = max(steps * 4, 2_000_000_000 // (blocks * stage_bytes) // steps * steps)
+        run = lambda: bk.lib.sglqb_lds_fill(stages, src.data_ptr(), rows, pitch, steps, window, share, iters, clocks.data_ptr(), sink.data_ptr(),
+                                            blocks, bk._stream())
+        rc = run()
+        assert rc == 0, (rc, label)
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        rc = run()
+        e.record()
+        torch.cuda.synchronize()
+        assert rc == 0, (rc, label)
+        ticks = clocks.view(blocks, 2)[:, 1].double().cpu()  # 100 MHz ticks of each block's loop
+        per_block = (iters * stage_bytes) / (ticks * 1e-8) / 1e9
+        out["cases"].append({"source": label, "stages": stages, "stage_KiB": stage_bytes // 1024, "in_flight_KiB_per_CU": (stages - 1) * stage_bytes // 1024,
+                             "blocks": blocks, "bytes_per_block_MB": round(iters * stage_bytes / 1e6, 1), "footprint_MB": round(windows * window / 1e6, 1),
+                             "GBs_per_block_median": round(float(per_block.median()), 1), "GBs_per_block_min": round(float(per_block.min()), 1),
+                             "TBs_all_blocks": round(blocks * iters * stage_bytes / (s.elapsed_time(e) * 1e-3) / 1e12, 2)})
+        del src
+    print(json.dumps(out), flush=True)
 
 
 def run_ceiling(args):
@@ -1032,6 +1088,7 @@ def main():
                     help="with --launches: the block-scaled FP8 linear (default), or the per-token FP8 / INT8 one")
     ap.add_argument("--ue8m0", action="store_true",
                     help="with --launches: power-of-two scales (per_token_group_quant_fp8_pow2 + fp8_blockwise_scaled_mm_ue8m0)")
+    ap.add_argument("--fill", action="store_true", help="only measure what the compute units take in through their LDS (copy loop without arithmetic) and exit")
     ap.add_argument("--ceiling", action="store_true", help="only measure the MFMA pipe's sustained rate (register-only loop) and exit")
     ap.add_argument("--graph", action="store_true", help="also time the K steps replayed as one HIP graph (graph_ms_per_step)")
     ap.add_argument("--prewarm-ms", type=float, default=150.0, help="untimed steps for this long before the warm-up steps")
@@ -1049,6 +1106,8 @@ def main():
         run_ab(args)
     elif args.launches:
         run_launches(args)
+    elif args.fill:
+        run_fill(args)
     elif args.ceiling:
         run_ceiling(args)
     elif args.sweep:

@@ -4,7 +4,9 @@
 //   * a clock probe (shader-clock and constant-rate counters per compute unit), from which a harness
 //     derives the average shader clock over a timed region,
 //   * a plain copy and a read-only / write-only pass of known size, the yardsticks for the
-//     FETCH_SIZE / WRITE_SIZE profiler counters and for the memory system's streaming rate.
+//     FETCH_SIZE / WRITE_SIZE profiler counters and for the memory system's streaming rate,
+//   * a global -> LDS copy loop without arithmetic: what the compute units take in through their LDS from the
+//     L2s, the last-level cache or HBM with the GEMM kernels' copy instruction and tile shapes.
 // C ABI, raw pointers, nothing allocated; every kernel runs a bounded loop.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -185,9 +187,96 @@ __global__ __launch_bounds__(256) void stream_kernel(const v4i* __restrict__ src
   }
 }
 
+// What a compute unit can take in through its LDS: the GEMM kernels' global -> LDS copies and nothing else.
+// 8 waves per block, one block per CU; a "stage" is `rows` rows of 128 bytes (rows a multiple of 64: every wave
+// issues rows / 64 one-KiB copies per stage, lane l bringing 16 bytes of row l / 8 as in the GEMM kernels), the rows
+// `pitch` bytes apart.  Every wave keeps NSTAGE - 1 stages of its own copies in flight (copies retire in order:
+// one vmcnt wait per stage) and nothing synchronises the waves.  Stage t of a block starts at byte
+// (t % steps) * 128 of its window's rows: a block walks its window along the rows like a GEMM block walks K.
+// Blocks b and b + 8, ..., b + 8 (share - 1) read the same window (the dispatcher deals blocks to the eight XCDs
+// round-robin, so they share an L2); windows are `window_bytes` apart.
+typedef unsigned int v4u_b __attribute__((ext_vector_type(4)));
+template <int NSTAGE>
+__global__ __launch_bounds__(512) void lds_fill_kernel(const char* __restrict__ src, int rows, uint32_t pitch, int steps, int64_t window_bytes,
+                                                       int share, int iters, uint64_t* __restrict__ clocks, int* __restrict__ sink) {
+  extern __shared__ __attribute__((aligned(1024))) char fill_smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int cpw = rows / 64;  // copies per wave and stage
+  const int stage_bytes = rows * 128;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int64_t window = (int64_t)((idx / share) * 8 + xcd);
+  const char* base = src + window * window_bytes;
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  const uint32_t extent = (uint32_t)((rows - 1) * (int64_t)pitch + (int64_t)steps * 128);
+  const v4u_b rsrc = {(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a), (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)extent), 0x00020000u};
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)fill_smem);
+  const uint32_t lane_off = (uint32_t)(wave * 8 + (lane >> 3)) * pitch + (uint32_t)(lane & 7) * 16u;
+  auto issue = [&](int t) {
+    const uint32_t st = lds0 + (uint32_t)(t % NSTAGE) * (uint32_t)stage_bytes;
+    const uint32_t k0 = (uint32_t)(t % steps) * 128u;
+    for (int j = 0; j < cpw; ++j) {
+      const uint32_t dst = st + (uint32_t)(wave + 8 * j) * 1024u;
+      const uint32_t voff = lane_off + (uint32_t)(64 * j) * pitch;
+      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(dst), "v"(voff), "s"(rsrc), "s"(k0) : "memory");
+    }
+  };
+  const ClockSample t0 = read_clocks();
+  for (int t = 0; t < NSTAGE - 1; ++t) issue(t);
+  for (int t = 0; t < iters; ++t) {
+    issue(t + NSTAGE - 1);
+    // (stage t has landed: at most the NSTAGE - 1 younger stages' copies are outstanding; cpw is 1, 2, 3, 4 or 6)
+    if (cpw == 1) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * 1) : "memory");
+    else if (cpw == 2) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * 2) : "memory");
+    else if (cpw == 3) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * 3) : "memory");
+    else if (cpw == 4) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * 4) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSTAGE - 1) * 6) : "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  const ClockSample t1 = read_clocks();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    clocks[2 * blockIdx.x] = t1.shader_cycles - t0.shader_cycles;
+    clocks[2 * blockIdx.x + 1] = t1.realtime_ticks - t0.realtime_ticks;
+    if (fill_smem[lane] == 0x5a && fill_smem[1024] == 0x5a) sink[blockIdx.x] = 1;  // keeps the stages observable
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+// The LDS fill loop: `blocks` blocks of 512 lanes, `stages` (2, 3 or 4) stages of rows x 128 bytes in LDS (rows in
+// {64, 128, 192, 256, 384}; stages * rows * 128 <= 160 KiB), `iters` stages per wave.  src must hold
+// ceil(blocks / 8 / share) * 8 windows of window_bytes each, a window at least (rows - 1) * pitch + steps * 128 bytes.
+// clocks: blocks x 2 uint64 (shader cycles, 100 MHz ticks of each block's loop).
+int sglqb_lds_fill(int stages, const void* src, int rows, int64_t pitch, int steps, int64_t window_bytes, int share, int iters,
+                   uint64_t* clocks, int* sink, int blocks, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!src || !clocks || !sink || blocks <= 0 || iters <= 0 || steps <= 0 || share <= 0) return -1;
+  if (rows != 64 && rows != 128 && rows != 192 && rows != 256 && rows != 384) return -1;
+  const int64_t lds = (int64_t)stages * rows * 128;
+  if (lds > 160 * 1024 || pitch < 128 || pitch % 16 != 0 || (rows - 1) * pitch + (int64_t)steps * 128 > window_bytes ||
+      (rows - 1) * pitch + (int64_t)steps * 128 >= (1ll << 31))
+    return -1;
+  const char* s = static_cast<const char*>(src);
+  hipError_t e = hipSuccess;
+  if (stages == 2) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(lds_fill_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) lds_fill_kernel<2><<<blocks, 512, lds, st>>>(s, rows, (uint32_t)pitch, steps, window_bytes, share, iters, clocks, sink);
+  } else if (stages == 3) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(lds_fill_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) lds_fill_kernel<3><<<blocks, 512, lds, st>>>(s, rows, (uint32_t)pitch, steps, window_bytes, share, iters, clocks, sink);
+  } else if (stages == 4) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(lds_fill_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) lds_fill_kernel<4><<<blocks, 512, lds, st>>>(s, rows, (uint32_t)pitch, steps, window_bytes, share, iters, clocks, sink);
+  } else {
+    return -1;
+  }
+  if (e != hipSuccess) return (int)e;
+  return (int)hipGetLastError();
+}
 
 // variant 0..3 (see above); operands: 96 KiB of e4m3 bytes (no NaN codes); sink: blocks * 512 floats;
 // clocks: blocks * 2 uint64 (shader cycles, constant-rate ticks of each block).  8 waves per block,

@@ -4,7 +4,9 @@ reference's benchmark/kernels/quantization/tuning_block_wise_kernel.py for its T
 
     python -m sglang_amd.quantization.tune_block_fp8 --N 4096 --K 7168 [--M 1 8 64 ...] [--out DIR] [--dtype int8_w8a8]
 
-(--dtype int8_w8a8 tunes the block-scaled INT8 GEMM, w8a8_block_int8_matmul, instead.)
+(--dtype int8_w8a8 tunes the block-scaled INT8 GEMM, w8a8_block_int8_matmul, instead; fp8_w8a8_channel / int8_w8a8_channel
+tune fp8_scaled_mm / int8_scaled_mm, whose kernel the reference picks per M bucket in C++, sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:751-791,
+int8_gemm_kernel.cu:585-661.)
 
 Every candidate (kernel code, split-K factor) is timed from HIP-graph replays with the weights
 rotated through more than the last-level cache; an entry is written only where a candidate beats
@@ -60,7 +62,8 @@ class Harness:
     def __init__(self, n: int, k: int, iters: int, dev, dtype: str = "fp8_w8a8"):
         from sglang_amd import _lib
 
-        self.n, self.k, self.dev, self.int8 = n, k, dev, dtype == "int8_w8a8"
+        self.n, self.k, self.dev, self.int8 = n, k, dev, dtype.startswith("int8_w8a8")
+        self.channel = dtype.endswith("_channel")  # per-token / per-channel scales: int8_scaled_mm, fp8_scaled_mm
         self.lib = _lib.load()
         self.g = torch.Generator(device=dev).manual_seed(n + k)
         if self.int8:
@@ -68,6 +71,8 @@ class Harness:
         else:
             w = (torch.randn((n, k), generator=self.g, device=dev) * 0.5).to(torch.float8_e4m3fn)
         self.ws = torch.rand(((n + 127) // 128, (k + 127) // 128), generator=self.g, device=dev) * 1e-2 + 1e-3
+        if self.channel:
+            self.ws = torch.rand((n, 1), generator=self.g, device=dev) * 9e-3 + 1e-3
         # weights in rotation past the 256 MiB last-level cache (320 MB and more), as a model's layers come by in use
         self.copies = max(2, min(48, -(-320_000_000 // (n * k))))
         self.iters = max(iters, self.copies)
@@ -76,7 +81,13 @@ class Harness:
 
     def set_m(self, m: int):
         n, k, g, dev = self.n, self.k, self.g, self.dev
-        if self.int8:
+        if self.channel:
+            if self.int8:
+                self.a = torch.randint(-127, 128, (m, k), generator=g, device=dev, dtype=torch.int32).to(torch.int8)
+            else:
+                self.a = (torch.randn((m, k), generator=g, device=dev) * 2).to(torch.float8_e4m3fn)
+            self.sa = torch.rand((m, 1), generator=g, device=dev) * 1e-2 + 1e-3
+        elif self.int8:
             self.a = torch.randint(-127, 128, (m, k), generator=g, device=dev, dtype=torch.int32).to(torch.int8)
             self.sa = torch.rand((m, k // 128), generator=g, device=dev) * 1e-2 + 1e-3  # row-major, as the INT8 quantizer writes it
         else:
@@ -86,8 +97,10 @@ class Harness:
 
     def run(self, j):
         from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
-        from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+        from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_scaled_mm
 
+        if self.channel:
+            return (int8_scaled_mm if self.int8 else fp8_scaled_mm)(self.a, self.wq[j].t(), self.sa, self.ws, torch.bfloat16, None)
         if self.int8:
             return w8a8_block_int8_matmul(self.a, self.wq[j], self.sa, self.ws, [128, 128], torch.bfloat16)
         return fp8_blockwise_scaled_mm(self.a, self.wq[j].t(), self.sa, self.ws.t(), torch.bfloat16)
@@ -261,7 +274,8 @@ def main():
     ap.add_argument("--iters", type=int, default=8)
     ap.add_argument("--margin", type=float, default=0.04)
     ap.add_argument("--out", type=str, default=None, help="directory for the table (default: the package's configs/)")
-    ap.add_argument("--dtype", choices=["fp8_w8a8", "int8_w8a8"], default="fp8_w8a8", help="block-scaled FP8 or block-scaled INT8 GEMM")
+    ap.add_argument("--dtype", choices=["fp8_w8a8", "int8_w8a8", "fp8_w8a8_channel", "int8_w8a8_channel"], default="fp8_w8a8",
+                    help="block-scaled FP8 or block-scaled INT8 GEMM; with _channel: fp8_scaled_mm / int8_scaled_mm (per-token and per-channel scales)")
     args = ap.parse_args()
     if args.apply:
         apply_verify_log(args.apply, args.dir)

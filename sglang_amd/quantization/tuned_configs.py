@@ -4,7 +4,9 @@ python/sglang/srt/layers/quantization/fp8_kernel.py:738-776; files under
 python/sglang/srt/layers/quantization/configs/).
 
 File name: ``N={N},K={K},device_name={device},dtype={dtype},block_shape=[128, 128].json`` with
-dtype ``fp8_w8a8`` (block-scaled FP8) or ``int8_w8a8`` (block-scaled INT8).  Content: a mapping
+dtype ``fp8_w8a8`` (block-scaled FP8), ``int8_w8a8`` (block-scaled INT8), or ``fp8_w8a8_channel`` /
+``int8_w8a8_channel`` (fp8_scaled_mm / int8_scaled_mm with per-token and per-channel scales, whose kernel the
+reference picks per M bucket in C++: sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:751-791, int8_gemm_kernel.cu:585-661).  Content: a mapping
 from batch sizes M to ``{"tile": code, "splits": s}``, where ``code`` names a kernel as
 ``sglq_debug_force_tile`` does and ``s`` is the split-K factor (0 = leave it to the library).
 As in the reference, a call takes the entry whose M is closest to its own; here that rule is
@@ -22,7 +24,8 @@ from .. import _lib
 
 CONFIG_DIR = Path(__file__).resolve().parent / "configs"
 DEVICE_NAME = "AMD_Instinct_MI355X"
-KIND_OF_DTYPE = {"fp8_w8a8": 0, "int8_w8a8": 4}  # SGLQ_KIND_FP8_BLOCK, SGLQ_KIND_I8_BLOCK
+# SGLQ_KIND_FP8_BLOCK, SGLQ_KIND_I8_BLOCK; per-token / per-channel scales: SGLQ_KIND_FP8_ROWCOL, SGLQ_KIND_I8_ROWCOL
+KIND_OF_DTYPE = {"fp8_w8a8": 0, "int8_w8a8": 4, "fp8_w8a8_channel": 1, "int8_w8a8_channel": 2}
 M_MAX = 1 << 30
 
 
