@@ -159,6 +159,23 @@ int sglq_fp8_blockwise_scaled_mm_ue8m0(const void* a, int64_t lda, const void* b
                                        int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                        int64_t workspace_bytes, void* stream);
 
+/* sglq_fp8_blockwise_scaled_mm_ue8m0 with the activation scales in the packed form that
+ * sgl_per_token_group_quant_fp8 writes with scale_ue8m0 = true (sglq_per_token_group_quant_fp8_ue8m0;
+ * sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:57-64,94) and that the reference hands to DeepGEMM as it is
+ * (fp8_utils.py:240-258, fp8_kernel.py:308-320): int32 words of four UE8M0 codes, byte kb % 4 of word
+ * [m, kb / 4] is K block kb's code, the word at sfa_packed[m * sfa_stride_m + (kb / 4) * sfa_stride_k4] (the
+ * column-major, 4-row-padded tensor of the reference: sfa_stride_m = 1, sfa_stride_k4 = M rounded up to 4).
+ * K must be a multiple of 128.  The kernels whose matrix instruction applies the scales fetch the words and pick
+ * the byte themselves; for every other shape the library first expands them into fp32 at the head of the
+ * workspace, which must therefore hold at least M * K / 128 floats rounded up to 256 bytes (the rest serves
+ * split-K as in the other entry points).  Results: those of sglq_fp8_blockwise_scaled_mm_ue8m0 on the same
+ * scales as fp32, bit for bit.  sfb stays fp32 powers of two [N/128, K/128]. */
+int sglq_fp8_blockwise_scaled_mm_ue8m0_packed(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                              const int32_t* sfa_packed, int64_t sfa_stride_m, int64_t sfa_stride_k4,
+                                              const float* sfb, int64_t sfb_stride_k, int64_t sfb_stride_n, void* out,
+                                              int64_t ldo, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                              void* workspace, int64_t workspace_bytes, void* stream);
+
 /* sglq_fp8_blockwise_scaled_mm fused with the bias add that its caller performs on the
  * result (python/sglang/srt/layers/quantization/fp8_utils.py:207-211: the GEMM, then
  * `output += bias` on the rounded output): out = round(round(gemm) + bias), bias [N] in

@@ -35,6 +35,8 @@ SIGNATURES = {
                                      c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_ue8m0": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                            c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
+    "sglq_fp8_blockwise_scaled_mm_ue8m0_packed": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+                                                  c_int64, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p],
     "sglq_fp8_blockwise_scaled_mm_noalloc": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                              c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
     "sglq_init": [],

@@ -45,6 +45,9 @@ constexpr bool is_block(int kind) { return kind == KIND_FP8_BLOCK || kind == KIN
 constexpr bool fp8_operands(int kind) { return kind == KIND_FP8_BLOCK || kind == KIND_FP8_ROWCOL || kind == KIND_FP8_BLOCK_POW2; }
 // the biased exponent of a positive power of two = its UE8M0 code, in byte 0 as the scaled MFMA reads it
 SGLQ_DEV int ue8m0_of(float pow2) { return (int)(__builtin_bit_cast(uint32_t, pow2) >> 23); }
+// ... of an activation scale as the kernels hold it: the eight bits from `shift` on, 23 for an fp32 power of two, 8 (kb % 4)
+// for a word of four UE8M0 codes (GemmArgs::sa_packed) and K block kb
+SGLQ_DEV int ue8m0_at(float word, int shift) { return (int)((__builtin_bit_cast(uint32_t, word) >> shift) & 0xffu); }
 constexpr bool float_acc(int kind) { return fp8_operands(kind) || kind == KIND_I8_BLOCK; }
 
 constexpr uint32_t OOB = 0x80000000u;  // offset beyond any buffer this library accepts
@@ -70,6 +73,12 @@ struct GemmArgs {
   int num_experts;
   int stream_out;  // the output is larger than the last-level cache: store it with the non-temporal hint
   int pow2_scales;  // block-scaled FP8: every scale is a power of two (KIND_FP8_BLOCK_POW2 where it is built)
+  // ... and the activation scales come as UE8M0 codes, four K blocks to an int32 word: word (m, kb / 4) sits at
+  // sa[m * sa_stride_m + (kb / 4) * sa_stride_k], byte kb % 4 of it is K block kb's code (what
+  // sglq_per_token_group_quant_fp8_ue8m0 writes).  Read as they are by the KIND_FP8_BLOCK_POW2 kernels; every
+  // other kernel gets them expanded to fp32 first (expand_packed_scales).
+  int sa_packed;
+  float* sa_expanded;  // room for [M, K / 128] fp32 scales (sa_packed only)
   float quant_eps;  // fused quantization (gemm_stream_quant_kernel): lower bound of a group's abs-max
 };
 
@@ -1014,7 +1023,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   const int sfb_rd = 2 * STAGE_BYTES + 1024 + (wn >> 1) * 4;
   if constexpr (BLOCK) {
     const int nblocks = (p.N + 127) >> 7;
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb_all - 1) * p.sa_stride_k + 1;
+    const int sa_last = (HW && p.sa_packed) ? (nkb_all - 1) >> 2 : nkb_all - 1;  // (packed: words of four K blocks)
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)sa_last * p.sa_stride_k + 1;
     int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb_all - 1) * p.sb_stride_k + 1;
     if constexpr (MODE == PIPE_GROUPED) sfb_elems += (int64_t)(p.num_experts - 1) * p.sb_expert_stride;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
@@ -1028,9 +1038,15 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     if (wave < 4) return (uint32_t)(m0 * p.sa_stride_m * 4);
     return (uint32_t)(((n0 >> 7) * p.sb_stride_n + expert * p.sb_expert_stride) * 4);
   };
+  // (packed activation scales: this wave's copy of K block kb fetches the word of K blocks 4 (kb / 4) .. + 3)
+  const int sc_kshift = (HW && p.sa_packed && wave < 4) ? 2 : 0;
+  const bool sa_packed = HW && p.sa_packed;
+  auto code_shift = [&](int kb) { return sa_packed ? 8 * (kb & 3) : 23; };
+  int sh_cur = 23;  // where the UE8M0 code of the K block in sfa_cur sits inside its word
   auto copy_scales = [&](int buf, int kb, uint32_t off) {
     char* dst = smem + buf * SCALE_BYTES + sc_dst;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kb * sc_step) + off, 0,
+    const int kw = HW ? kb >> sc_kshift : kb;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kw * sc_step) + off, 0,
                                              0);
   };
   auto read_sfa = [&](int buf, int i) -> float {
@@ -1058,7 +1074,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         sc_prev = sc;
         sc = sfa_cur[i] * sfb_cur;
       }
-      if constexpr (HW) ea = ue8m0_of(sfa_cur[i]);
+      if constexpr (HW) ea = ue8m0_at(sfa_cur[i], sh_cur);
       if (i == 1 && !last) {
         // barrier 1: MFMAs 0..3 have consumed this wave's weight fragments, so its LDS reads
         // of block u's weights are complete; behind the barrier that holds for every wave.
@@ -1153,6 +1169,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         acc[MI - 1][NI - 1][e] = first ? block_value<KIND>(part_prev[e]) * sc
                                        : __builtin_fmaf(block_value<KIND>(part_prev[e]), sc, acc[MI - 1][NI - 1][e]);
     }
+    if constexpr (HW && !last) sh_cur = code_shift(kn);  // sfa_cur now holds block u + 1's words
   };
 
   // ---- persistent walk over the work units blockIdx, blockIdx + gridDim, ...  A unit is an
@@ -1206,6 +1223,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 #pragma unroll
       for (int i = 0; i < MI; ++i) sfa_cur[i] = read_sfa(stage, i);
       sfb_cur = read_sfb(stage);
+      if constexpr (HW) sh_cur = code_shift(kb0);
     }
   };
   read_first(0);
@@ -1384,7 +1402,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   const int sfa_rd = 2 * STAGE_BYTES + (wm * TM + r16) * 4;
   if constexpr (BLOCK) {
     const int nblocks = (p.N + 127) >> 7;
-    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)(nkb - 1) * p.sa_stride_k + 1;
+    const int sa_last = (HW && p.sa_packed) ? (nkb - 1) >> 2 : nkb - 1;  // (packed: words of four K blocks)
+    const int64_t sfa_elems = (int64_t)(p.M - 1) * p.sa_stride_m + (int64_t)sa_last * p.sa_stride_k + 1;
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
@@ -1404,9 +1423,15 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     jsw_nxt = __builtin_amdgcn_readfirstlane(((nb_lo + 1) * 128 - nw) >> 4);
     sfb_rd_nxt = __builtin_amdgcn_readfirstlane(2 * STAGE_BYTES + 1024 + (nb_lo - (n0 >> 7)) * 4);
   };
+  // (packed activation scales: this wave's copy of K block kb fetches the word of K blocks 4 (kb / 4) .. + 3)
+  const int sc_kshift = (HW && p.sa_packed && wave < 4) ? 2 : 0;
+  const bool sa_packed = HW && p.sa_packed;
+  auto code_shift = [&](int kb) { return sa_packed ? 8 * (kb & 3) : 23; };
+  int sh_cur = 23;  // where the UE8M0 code of the K block in sfa_cur sits inside its word
   auto copy_scales = [&](int buf, int kb, uint32_t off) {
     char* dst = smem + buf * SCALE_BYTES + sc_dst;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kb * sc_step) + off, 0,
+    const int kw = HW ? kb >> sc_kshift : kb;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsc, (__attribute__((address_space(3))) void*)dst, 4, lane_s, (uint32_t)(kw * sc_step) + off, 0,
                                              0);
   };
   auto read_sfa = [&](int buf, int i) -> float {
@@ -1445,7 +1470,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const int jsw_now = jsw;
     if constexpr (HW) {
 #pragma unroll
-      for (int i = 0; i < MI; ++i) ea[i] = ue8m0_of(sfa_cur[i]);
+      for (int i = 0; i < MI; ++i) ea[i] = ue8m0_at(sfa_cur[i], sh_cur);
     }
     v4f part_prev = {0.f, 0.f, 0.f, 0.f};
     __builtin_amdgcn_sched_barrier(0);
@@ -1546,6 +1571,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       acc[MI - 1][NI - 1][3] = __builtin_fmaf(block_value<KIND>(part_prev[3]), sc, acc[MI - 1][NI - 1][3]);
     }
     if constexpr (BLOCK) jsw = jsw_nxt;
+    if constexpr (HW) sh_cur = code_shift(kn);  // sfa_cur now holds block u + 1's words (a tile's last step: the next tile's block 0)
   };
 
   // ---- persistent walk over the tiles blockIdx, blockIdx + gridDim, ...
@@ -1578,6 +1604,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     sfb_lo = read_sfb(0, 0);
     sfb_hi = read_sfb(0, 1);
     jsw = jsw_nxt;
+    if constexpr (HW) sh_cur = code_shift(0);
   }
 
   while (true) {
@@ -2539,6 +2566,7 @@ static thread_local bool g_last_hw_scaled = false;   // ... and whether its MFMA
 
 template <int KIND, int OUT_DT>
 static void launch_reduce(GemmArgs& p, hipStream_t st);
+static void expand_packed_scales(GemmArgs& p, hipStream_t st);
 
 // Tile plan of a grouped GEMM, from the experts' row counts and first rows in device memory
 // (problem_sizes[e][0], expert_offsets[e]); one block.  Inconsistent inputs cannot make the
@@ -2602,6 +2630,7 @@ static void launch_grouped_cfg(GemmArgs& p, int max_tiles, hipStream_t st) {
 // CU), K is split across blocks as far as the workspace and the partial sums' traffic allow.
 template <int KIND, int BM, int BN, int WAVES_M, int WAVES_N, int OUT_DT>
 static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  expand_packed_scales(p, st);
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const int tiles = p.tiles_m * p.tiles_n;
@@ -2639,14 +2668,42 @@ static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws
 // Whether this launch takes the kernels whose MFMAs apply the block scales (built for bf16 outputs without a
 // fused bias, what the reference's call of that GEMM produces: fp8_utils.py:225-258).
 template <int KIND, int OUT_DT>
+static bool can_hw_scale(const GemmArgs& p) {
+  return KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16 && p.pow2_scales && !p.bias;
+}
+template <int KIND, int OUT_DT>
 static bool hw_scaled(const GemmArgs& p) {
-  const bool hw = KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16 && p.pow2_scales && !p.bias;
+  const bool hw = can_hw_scale<KIND, OUT_DT>(p);
   if (hw) g_last_hw_scaled = true;
   return hw;
 }
 
+// Packed UE8M0 activation scales (GemmArgs::sa_packed) as fp32 powers of two, column-major [K / 128][M], for the
+// kernels that multiply by the scales instead of handing their exponents to the matrix instruction.
+__global__ __launch_bounds__(256) void expand_ue8m0_kernel(const uint32_t* __restrict__ packed, int64_t stride_m, int64_t stride_k4,
+                                                          float* __restrict__ out, int M, int nkb) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * nkb) return;
+  const int kb = (int)(idx / M), m = (int)(idx % M);
+  const uint32_t word = packed[(int64_t)m * stride_m + (int64_t)(kb >> 2) * stride_k4];
+  out[idx] = __builtin_bit_cast(float, ((word >> (8 * (kb & 3))) & 0xffu) << 23);
+}
+// Called by every launcher whose kernel does not read the packed form, before its launch.
+static void expand_packed_scales(GemmArgs& p, hipStream_t st) {
+  if (!p.sa_packed) return;
+  const int nkb = p.K >> 7;
+  const int64_t n = (int64_t)p.M * nkb;
+  expand_ue8m0_kernel<<<dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, st>>>(reinterpret_cast<const uint32_t*>(p.sa), p.sa_stride_m, p.sa_stride_k,
+                                                                            p.sa_expanded, p.M, nkb);
+  p.sa = p.sa_expanded;
+  p.sa_stride_m = 1;
+  p.sa_stride_k = p.M;
+  p.sa_packed = 0;
+}
+
 template <int KIND, int OUT_DT>
 static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  if (!(t_tile != 256 && p.K >= 384 && can_hw_scale<KIND, OUT_DT>(p))) expand_packed_scales(p, st);
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 255) / 256;
   p.splits = 1;
@@ -2734,6 +2791,7 @@ static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws
 // The pipelined kernel with 128-row tiles: (tile, K range) work units.
 template <int KIND, int OUT_DT>
 static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  if (!can_hw_scale<KIND, OUT_DT>(p)) expand_packed_scales(p, st);
   p.tiles_m = (p.M + 127) / 128;
   p.tiles_n = (p.N + 255) / 256;
   const int tiles = p.tiles_m * p.tiles_n;
@@ -2774,6 +2832,7 @@ static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 
 template <int KIND, int OUT_DT, int NI>
 static void launch_wide(GemmArgs& p, hipStream_t st) {
+  if (!can_hw_scale<KIND, OUT_DT>(p)) expand_packed_scales(p, st);
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 32 * NI - 1) / (32 * NI);
   p.splits = 1;
@@ -2879,6 +2938,7 @@ static int skinny_splits(int M, int N, int K, int bn = 128) {
 
 template <int KIND, int OUT_DT>
 static void launch_skinny(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
+  expand_packed_scales(p, st);
   // Weight rows per block: 128, or 64 where several row tiles share the weight tiles (M > 64) and the model above
   // says that twice as many blocks with two thirds of the bytes each are faster: up to about 200 tiles of 128.
   bool narrow = t_tile == 66 && p.M > 32;
@@ -2966,6 +3026,7 @@ template <int KIND, int OUT_DT>
 static bool launch_stream(GemmArgs& p, hipStream_t st) {
   const int nib = stream_rows<KIND>(p);
   if (nib == 0) return false;
+  expand_packed_scales(p, st);
   p.splits = 1;
   p.tiles_m = 1;
   p.tiles_n = (p.N + 16 * nib - 1) / (16 * nib);
@@ -3018,6 +3079,7 @@ static int stream_tiles_choice(const GemmArgs& p) {  // 0: the split-K kernel; 6
 
 template <int KIND, int OUT_DT>
 static void launch_stream_tiles(GemmArgs& p, hipStream_t st, bool half_rows = false) {
+  expand_packed_scales(p, st);
   p.splits = 1;
   p.tiles_m = half_rows ? (p.M + 31) / 32 : (p.M + 63) / 64;
   p.tiles_n = (p.N + 63) / 64;
@@ -3278,7 +3340,8 @@ template <int KIND>
 static int blockwise_entry(const char* name, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,
                            int64_t sfa_stride_m, int64_t sfa_stride_k, const float* sfb, int64_t sfb_stride_k,
                            int64_t sfb_stride_n, const void* bias, void* out, int64_t ldo, int out_dtype, int64_t M,
-                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream, bool pow2_scales = false) {
+                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream, bool pow2_scales = false,
+                           bool sfa_packed = false) {
   int rc = gemm_common_checks(name, a, lda, b, ldb, out, ldo, M, N, K, 2);
   if (rc < 0) return SGLQ_OK;
   if (rc) return rc;
@@ -3299,6 +3362,23 @@ static int blockwise_entry(const char* name, const void* a, int64_t lda, const v
   p.sa_stride_k = sfa_stride_k;
   p.sb_stride_k = sfb_stride_k;
   p.sb_stride_n = sfb_stride_n;
+  if (sfa_packed) {
+    // The head of the workspace takes the scales as fp32 for the kernels that do not read the packed words
+    // (decode and split-K shapes, outputs other than bf16); split-K partial sums get the rest.
+    if (K % 128 != 0) {
+      set_error("%s: K (%lld) must be a multiple of 128 for packed scales", name, (long long)K);
+      return SGLQ_EINVAL;
+    }
+    const int64_t need = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3)) {
+      set_error("%s: the workspace must hold M * K / 128 floats (%lld bytes) for the expanded scales", name, (long long)need);
+      return SGLQ_EINVAL;
+    }
+    p.sa_packed = 1;
+    p.sa_expanded = static_cast<float*>(workspace);
+    workspace = static_cast<char*>(workspace) + need;
+    workspace_bytes -= need;
+  }
   p.ws = workspace;
   p.pow2_scales = pow2_scales ? 1 : 0;
   g_last_hw_scaled = false;
@@ -3326,6 +3406,16 @@ extern "C" int sglq_fp8_blockwise_scaled_mm_ue8m0(const void* a, int64_t lda, co
   return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm_ue8m0", a, lda, b, ldb, sfa, sfa_stride_m, sfa_stride_k, sfb,
                                          sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N, K, workspace,
                                          workspace_bytes, stream, true);
+}
+
+extern "C" int sglq_fp8_blockwise_scaled_mm_ue8m0_packed(const void* a, int64_t lda, const void* b, int64_t ldb, const int32_t* sfa_packed,
+                                                         int64_t sfa_stride_m, int64_t sfa_stride_k4, const float* sfb,
+                                                         int64_t sfb_stride_k, int64_t sfb_stride_n, void* out, int64_t ldo,
+                                                         int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                                         int64_t workspace_bytes, void* stream) {
+  return blockwise_entry<KIND_FP8_BLOCK>("fp8_blockwise_scaled_mm_ue8m0_packed", a, lda, b, ldb, reinterpret_cast<const float*>(sfa_packed),
+                                         sfa_stride_m, sfa_stride_k4, sfb, sfb_stride_k, sfb_stride_n, nullptr, out, ldo, out_dtype, M, N,
+                                         K, workspace, workspace_bytes, stream, true, true);
 }
 
 extern "C" int sglq_fp8_blockwise_scaled_mm_bias(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sfa,

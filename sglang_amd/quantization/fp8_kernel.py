@@ -275,7 +275,8 @@ def w8a8_block_fp8_matmul_deepgemm(
     gemm_nt_f8f8bf16 in the reference, here sglq_fp8_blockwise_scaled_mm_ue8m0 (the matrix instruction applies
     the scales and accumulates in place).  A e4m3fn [..., K] contiguous; B e4m3fn [N, K] contiguous; As fp32
     powers of two [..., K/128] in any layout (per_token_group_quant_fp8_pow2), or the packed int32 form of
-    sglang_per_token_group_quant_fp8(scale_ue8m0=True), which is unpacked first; Bs fp32 powers of two
+    sglang_per_token_group_quant_fp8(scale_ue8m0=True), which the library reads as it is
+    (sglq_fp8_blockwise_scaled_mm_ue8m0_packed); Bs fp32 powers of two
     [N/128, K/128] (per_block_cast_to_fp8 / requant_weight_ue8m0_inplace).  bf16 output only, as there (:859-860)."""
     assert len(block_size) == 2
     if block_size[0] != 128 or block_size[1] != 128:
@@ -298,7 +299,18 @@ def w8a8_block_fp8_matmul_deepgemm(
     if M == 0 or N == 0:
         return C
     if As.dtype == torch.int32:
-        As2 = unpack_ue8m0_scales(As.reshape(M, As.shape[-1]), K // 128)
+        As2 = As.reshape(M, As.shape[-1]) if As.ndim != 2 else As
+        assert As2.shape == (M, -(-(K // 128) // 4)), "packed scales: one int32 word per row and four K blocks"
+        ws_ptr, ws_bytes = _lib.workspace(A.device)
+        if 4 * M * (K // 128) + 256 > ws_bytes // 2:
+            # (more rows than the cached workspace has room for beside split-K partial sums: expand here)
+            return w8a8_block_fp8_matmul_deepgemm(A, B, unpack_ue8m0_scales(As2, K // 128), Bs, block_size, output_dtype)
+        rc = _lib.load().sglq_fp8_blockwise_scaled_mm_ue8m0_packed(
+            A.data_ptr(), K, B.data_ptr(), K, As2.data_ptr(), As2.stride(0), As2.stride(1),
+            Bs.data_ptr(), Bs.stride(1), Bs.stride(0), C.data_ptr(), N, DTYPE_CODE[output_dtype], M, N, K,
+            ws_ptr, ws_bytes, _lib.stream_ptr(A.device))
+        _lib.check(rc, "w8a8_block_fp8_matmul_deepgemm")
+        return C
     elif As.dtype == torch.float32:
         assert As.shape[-1] == K // 128 and As.numel() == M * (K // 128)
         As2 = As.reshape(M, K // 128) if As.ndim != 2 else As

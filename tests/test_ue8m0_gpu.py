@@ -141,6 +141,103 @@ def test_fp8_blockwise_scaled_mm_ue8m0_fp16_output_runs_the_plain_kernels(gpu):
     torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
 
 
+def pack_codes(exps, gpu):
+    """UE8M0 codes [M, K/128] as the reference's quantization stores them with scale_ue8m0=True (fp8_kernel.py:308-320):
+    int32 words of four codes, column-major with the rows padded to a multiple of four."""
+    m, nkb = exps.shape
+    words = -(-nkb // 4)
+    padded = torch.zeros((m, 4 * words), dtype=torch.int64)
+    padded[:, :nkb] = exps.to(torch.int64)
+    shifts = torch.tensor([0, 8, 16, 24], dtype=torch.int64)
+    packed = (padded.view(m, words, 4) << shifts).sum(dim=-1)
+    packed = torch.where(packed >= 2**31, packed - 2**32, packed).to(torch.int32)
+    store = torch.full((words, -(-m // 4) * 4), 0x7F7F7F7F, dtype=torch.int32, device=gpu)
+    store[:, :m] = packed.t().to(gpu)
+    return store.t()[:m, :]
+
+
+PACKED_CASES = UE8M0_CASES + [
+    ((130, 640, 640), 130, True), ((257, 512, 896), 258, True), ((515, 448, 2176), 224, True), ((2050, 2112, 7168), 0, True),
+    ((33, 1024, 640), 0, False), ((511, 4096, 7168), 0, None), ((96, 7168, 2048), 0, None), ((4096, 256, 256), 0, False),
+]
+
+
+@pytest.mark.parametrize("mnk,tile,hw", PACKED_CASES)
+def test_fp8_blockwise_scaled_mm_ue8m0_packed_scales(gpu, mnk, tile, hw):
+    """The entry point that takes the activation scales as packed UE8M0 words gives the bits of the one that takes
+    them as fp32 powers of two, on the kernels that read the words themselves and on those that get them
+    expanded first (K blocks that do not fill the last word, rows that do not fill the padding)."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul_deepgemm
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_ue8m0
+
+    say("fp8_blockwise ue8m0 packed", mnk, "tile", tile)
+    m, n, k = mnk
+    lib = _lib.load()
+    x = O.gen_activation(m, k, seed=m + n + k, outliers=True)
+    _, xq, xs, wq, ws = pow2_block_case(m, n, k, seed=m + n + k)
+    _, exps, _ = O.per_token_group_quant_fp8_ue8m0(x)
+    packed = pack_codes(exps, gpu)
+    assert packed.stride(0) == 1 and packed.stride(1) % 4 == 0
+    lib.sglq_debug_force_tile(tile)
+    try:
+        want = fp8_blockwise_scaled_mm_ue8m0(xq.to(gpu), wq.to(gpu).t(), xs.t().contiguous().to(gpu).t(), ws.to(gpu).t(), torch.bfloat16)
+        want_kernel, want_hw = lib.sglq_debug_last_gemm_kernel().decode(), bool(lib.sglq_debug_last_gemm_hw_scaled())
+        got = w8a8_block_fp8_matmul_deepgemm(xq.to(gpu), wq.to(gpu), packed, ws.to(gpu), [128, 128], torch.bfloat16)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == want_kernel and bool(lib.sglq_debug_last_gemm_hw_scaled()) == want_hw
+        if hw is not None:
+            assert want_hw == hw, want_kernel
+    finally:
+        lib.sglq_debug_force_tile(0)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16)), want_kernel
+
+
+@pytest.mark.parametrize("splits", [2, 4])
+def test_fp8_blockwise_scaled_mm_ue8m0_packed_scales_split_k(gpu, splits):
+    """Work units that start in the middle of a word of four codes (K ranges of 6 and 3 K blocks)."""
+    from sglang_amd import _lib
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul_deepgemm
+    from sglang_amd.sgl_kernel.gemm import fp8_blockwise_scaled_mm_ue8m0
+
+    lib = _lib.load()
+    for (m, n, k), tile in (((512, 640, 1536), 258), ((300, 384, 1536), 130), ((130, 256, 3072), 130)):
+        say("fp8_blockwise ue8m0 packed split-K", (m, n, k), tile, splits)
+        x = O.gen_activation(m, k, seed=m + n + k + splits, outliers=True)
+        _, xq, xs, wq, ws = pow2_block_case(m, n, k, seed=m + n + k + splits)
+        _, exps, _ = O.per_token_group_quant_fp8_ue8m0(x)
+        lib.sglq_debug_force_tile(tile)
+        lib.sglq_debug_force_splits(splits)
+        try:
+            want = fp8_blockwise_scaled_mm_ue8m0(xq.to(gpu), wq.to(gpu).t(), xs.t().contiguous().to(gpu).t(), ws.to(gpu).t(), torch.bfloat16)
+            assert lib.sglq_debug_last_gemm_hw_scaled() and "splitk" in lib.sglq_debug_last_gemm_kernel().decode()
+            got = w8a8_block_fp8_matmul_deepgemm(xq.to(gpu), wq.to(gpu), pack_codes(exps, gpu), ws.to(gpu), [128, 128], torch.bfloat16)
+            assert lib.sglq_debug_last_gemm_hw_scaled() and "splitk" in lib.sglq_debug_last_gemm_kernel().decode()
+        finally:
+            lib.sglq_debug_force_tile(0)
+            lib.sglq_debug_force_splits(0)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_fp8_blockwise_scaled_mm_ue8m0_packed_checks_the_workspace(gpu):
+    from sglang_amd import _lib
+    from sglang_amd._lib import DTYPE_CODE
+
+    lib = _lib.load()
+    m, n, k = 64, 256, 512
+    a = torch.zeros((m, k), device=gpu, dtype=torch.uint8)
+    b = torch.zeros((n, k), device=gpu, dtype=torch.uint8)
+    sa = torch.zeros((1, m), device=gpu, dtype=torch.int32)
+    sb = torch.ones((2, 4), device=gpu)
+    out = torch.empty((m, n), device=gpu, dtype=torch.bfloat16)
+    small = torch.empty(512, device=gpu, dtype=torch.uint8)
+    rc = lib.sglq_fp8_blockwise_scaled_mm_ue8m0_packed(a.data_ptr(), k, b.data_ptr(), k, sa.data_ptr(), 1, m, sb.data_ptr(), 1, 4,
+                                                       out.data_ptr(), n, DTYPE_CODE[torch.bfloat16], m, n, k, small.data_ptr(), 512, 0)
+    assert rc != 0 and b"workspace" in lib.sglq_last_error()
+    rc = lib.sglq_fp8_blockwise_scaled_mm_ue8m0_packed(a.data_ptr(), k + 64, b.data_ptr(), k + 64, sa.data_ptr(), 1, m, sb.data_ptr(), 1, 4,
+                                                       out.data_ptr(), n, DTYPE_CODE[torch.bfloat16], m, n, k - 64, small.data_ptr(), 512, 0)
+    assert rc != 0
+
+
 @pytest.mark.parametrize("m", [3, 200, 1030])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_deepgemm_linear(gpu, monkeypatch, m, with_bias):
