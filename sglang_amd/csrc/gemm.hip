@@ -303,7 +303,7 @@ SGLQ_DEV void epilogue(const GemmArgs& p, acc_t (&acc)[MI][NI], int m_base, int 
 // convert.  Chunk c (16 bytes) of image row r sits at chunk position c ^ (r & 31).  The other stage buffer is not touched: it is receiving the
 // next tile's first K block.  The caller has made sure nobody reads `img` any more; on
 // return every wave has passed a barrier after its last read of `img`.
-template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, int HALF_ROWS = 128, typename acc_t>
+template <int KIND, int OUT_DT, int MI, int NI, int BN, bool BIAS, int HALF_ROWS = 128, int PASSES = 2, typename acc_t>
 SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* img, float* col_lds, int m0, int n0,
                                int wm, int wn, int r16, int g, int lane, int wave) {
   constexpr int TN = NI * 16;
@@ -350,23 +350,24 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
     }
     col_lds[threadIdx.x] = b;
   }
-  constexpr int HR = MI * 8;  // rows of a wave row in one half
+  constexpr int FR = MI / PASSES;  // fragment rows of a wave in one pass (two passes, the halves; three for 192-row tiles)
+  constexpr int HR = FR * 16;      // rows of a wave row in one pass
   // The tile's part of the output as a buffer: rows m0 .. min(M, m0 + 256) - 1 from column n0
   // on.  Used when every 16-byte chunk of the tile's columns lies inside N and the extent fits
   // the 31-bit offsets (wave-uniform conditions).
   const uint32_t row_bytes = (uint32_t)p.ldo * 2u;
-  const int rows_left = p.M - m0 < 2 * HALF_ROWS ? p.M - m0 : 2 * HALF_ROWS;
+  const int rows_left = p.M - m0 < PASSES * HALF_ROWS ? p.M - m0 : PASSES * HALF_ROWS;
   const bool whole_chunks = n0 + BN <= p.N && p.ldo < (1 << 21);
   const __amdgpu_buffer_rsrc_t r_out =
       make_rsrc(out + ((int64_t)m0 * p.ldo + n0) * 2, whole_chunks ? (uint32_t)rows_left * row_bytes - (uint32_t)n0 * 2u : 0u);
-  static_assert(MI % 2 == 0 && (HR & (HR - 1)) == 0 && HALF_ROWS % HR == 0 && HALF_ROWS % 16 == 0, "the halves are split by fragment row");
+  static_assert(MI % PASSES == 0 && (HR & (HR - 1)) == 0 && HALF_ROWS % HR == 0 && HALF_ROWS % 16 == 0, "the passes are split by fragment row");
   constexpr int RPW = HALF_ROWS / 8;  // image rows per wave in the store phase
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
+  for (int half = 0; half < PASSES; ++half) {
     {
-      float sam[MI / 2];
+      float sam[FR];
 #pragma unroll
-      for (int ii = 0; ii < MI / 2; ++ii) {
+      for (int ii = 0; ii < FR; ++ii) {
         sam[ii] = 1.f;
         if constexpr (ROWCOL) {
           const int m = m0 + wm * MI * 16 + half * HR + ii * 16 + r16;
@@ -382,8 +383,8 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
         }
         const int chunk = wn * (TN / 8) + j * 2 + (g >> 1);
 #pragma unroll
-        for (int ii = 0; ii < MI / 2; ++ii) {
-          const int i = half * (MI / 2) + ii;
+        for (int ii = 0; ii < FR; ++ii) {
+          const int i = half * FR + ii;
           const int ml = wm * HR + ii * 16 + r16;  // row inside the image
           float o[4];
 #pragma unroll
@@ -444,7 +445,7 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
 #pragma unroll
       for (int it = 0; it < RPW / 2; ++it) {
         const int ml = wave * RPW + it * 2 + (lane >> 5);
-        const uint32_t m_rel = (uint32_t)((ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1)));
+        const uint32_t m_rel = (uint32_t)((ml / HR) * (PASSES * HR) + half * HR + (ml & (HR - 1)));
         const uint32_t voff = (c * 8 < BN) ? m_rel * row_bytes + (uint32_t)c * 16u : OOB;
         // (aux bit 1 = nt: a line that will not be read again before it leaves the caches)
         if (p.stream_out) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[it]), r_out, voff, 0, 2);
@@ -454,7 +455,7 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
 #pragma unroll
       for (int it = 0; it < RPW / 2; ++it) {
         const int ml = wave * RPW + it * 2 + (lane >> 5);
-        const int m = m0 + (ml / HR) * (2 * HR) + half * HR + (ml & (HR - 1));
+        const int m = m0 + (ml / HR) * (PASSES * HR) + half * HR + (ml & (HR - 1));
         if (m < p.M && c * 8 < BN) {
           char* row = out + ((int64_t)m * p.ldo + n) * 2;
           if (n + 8 <= p.N) *reinterpret_cast<v4i*>(row) = v[it];  // (N is a multiple of 8: a chunk is in or out as a whole)
@@ -1304,9 +1305,10 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 // four activation fragments are in registers) and is refilled two K blocks ahead; the
 // weight copies of block u + 2 follow behind the last weight fragment's MFMAs.
 // ---------------------------------------------------------------------------
-template <int KIND, int OUT_DT, int NI, bool BIAS>
+template <int KIND, int OUT_DT, int NI, bool BIAS, int MI = 4>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
-  constexpr int BM = 256, NW = 8, WAVES_N = 2, MI = 4;
+  // (MI = 3: tiles of 192 rows, for row counts that 256-row tiles cover with a part-empty round of the CUs)
+  constexpr int BM = 64 * MI, NW = 8, WAVES_N = 2;
   constexpr int TM = MI * 16, TN = NI * 16, BN = WAVES_N * TN;
   constexpr int STAGE_BYTES = 512 * 128;  // stage pitch; only (BM + BN) rows are filled
   constexpr int NB = BN / 8;              // one-KiB weight copies per stage
@@ -1315,7 +1317,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
   constexpr bool BLOCK = is_block(KIND);
   constexpr bool HW = KIND == KIND_FP8_BLOCK_POW2;  // the MFMA applies the block scales
   constexpr bool FOLD = BLOCK && !HW;               // they are applied to each MFMA's result
-  static_assert(NBW <= 4 && NI >= 4, "copy and scale-load slots below assume this");
+  static_assert(NBW <= 4 && NBW <= MI && NI >= 4 && (MI == 4 || MI == 3), "copy and scale-load slots below assume this");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then up to three weight scales
   // (one LDS object per kernel, see gemm_big_kernel: the epilogue's 512 floats sit at the end)
@@ -1407,7 +1409,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const int64_t sfb_elems = (int64_t)(nblocks - 1) * p.sb_stride_n + (int64_t)(nkb - 1) * p.sb_stride_k + 1;
     rsc = wave < 4 ? make_rsrc(p.sa, (uint32_t)(sfa_elems * 4)) : make_rsrc(p.sb, (uint32_t)(sfb_elems * 4));
     sc_step = (int)((wave < 4 ? p.sa_stride_k : p.sb_stride_k) * 4);
-    if (wave < 4) lane_s = (uint32_t)((wave * 64 + lane) * p.sa_stride_m * 4);
+    if (wave < 4) lane_s = wave * 64 < BM ? (uint32_t)((wave * 64 + lane) * p.sa_stride_m * 4) : OOB;
     else lane_s = (wave == 4 && lane < 3) ? (uint32_t)(lane * p.sb_stride_n * 4) : OOB;
   }
   // (SC_NONE: no tile; beyond both scale tensors, and its sum with OOB does not wrap)
@@ -1456,7 +1458,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     const char* st = smem + cur * STAGE_BYTES;
     const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
-    float scv[MI] = {0.f, 0.f, 0.f, 0.f};  // sfa[i] * sfb of the scale block of the fragments being multiplied
+    float scv[MI] = {};  // sfa[i] * sfb of the scale block of the fragments being multiplied
     if constexpr (FOLD) {
 #pragma unroll
       for (int i = 0; i < MI; ++i) scv[i] = sfa_cur[i] * sfb_lo;
@@ -1465,7 +1467,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     // (HW runs one instantiation of the step for every position of the boundary, JSW = NI, and selects per
     // fragment at run time: instantiated per position like the other block kinds, the accumulators change
     // registers between the instantiations and the kernel spills)
-    int ea[MI] = {0, 0, 0, 0};
+    int ea[MI] = {};
     const int eb_lo = HW ? ue8m0_of(sfb_lo) : 0, eb_hi = HW ? ue8m0_of(sfb_hi) : 0;
     const int jsw_now = jsw;
     if constexpr (HW) {
@@ -1497,7 +1499,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
         // block u + 2, which stay in flight.  lgkmcnt(0): this wave's LDS reads of block u's
         // weights and scales are complete.  A bare s_barrier: these waits are all the
         // ordering that is needed.
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(last ? 0 : 4));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(last ? 0 : MI));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1543,12 +1545,12 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
           }
         }
         if constexpr (first) {
-          if (idx >= 4 && idx < 8) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
+          if (idx >= 4 && idx < 4 + MI) copy_a(idx - 4, cur ^ 1, kn * 128, off_a);
           if (idx >= 8 && idx < 8 + NBW) copy_b(idx - 8, cur ^ 1, kn * 128, off_b);
           if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_off);
-          if (idx >= 12 && idx < 16) copy_a(idx - 12, cur, kn2 * 128, off_a2);
+          if (idx >= 12 && idx < 12 + MI) copy_a(idx - 12, cur, kn2 * 128, off_a2);
         } else if constexpr (!last) {
-          if (idx >= 4 && idx < 8) copy_a(idx - 4, cur, kn2 * 128, off_a2);
+          if (idx >= 4 && idx < 4 + MI) copy_a(idx - 4, cur, kn2 * 128, off_a2);
         }
         if constexpr (FOLD) {
           if (idx > 0) {  // scale-and-accumulate the previous MFMA's result while this one runs
@@ -1589,7 +1591,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
     set_scale_split(n0);
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_a(j, 0, 0, off_a);
+  for (int j = 0; j < MI; ++j) copy_a(j, 0, 0, off_a);
 #pragma unroll
   for (int j = 0; j < NBW; ++j) copy_b(j, 0, 0, off_b);
   if constexpr (BLOCK) copy_scales(0, 0, sc_off);
@@ -1670,7 +1672,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmArgs p) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else {
       // (rows of 16-bit outputs are 16-byte aligned: checked on the host)
-      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane, wave);
+      epilogue_via_lds<KIND, OUT_DT, MI, NI, BN, BIAS, MI == 4 ? 128 : 64, MI == 4 ? 2 : 3>(p, acc, smem + last_stage * STAGE_BYTES, col_lds, m0, n0, wm, wn, r16, g, lane, wave);
     }
     if (!has_next) break;
     tile = next_tile;
@@ -2660,6 +2662,7 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 // test hook: 0 = heuristic, 64 = the M <= 64 kernel where it applies, 128 = the 128 x 128 kernel,
 // 256 = the plain 256 x 256 kernel, 258 = the pipelined one (K >= 384, else the plain one),
 // 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258),
+// 193 = that kernel on 192 x 192 tiles (block-scaled FP8 without a bias, K >= 384; else the heuristic),
 // 130 = the pipelined kernel with 128-row tiles (K >= 384, else the 128 x 128 kernel)
 static thread_local int g_force_tile = 0;
 
@@ -2828,6 +2831,20 @@ static void launch_pipe128(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   } else {
     gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN, 128><<<grid, block, 0, st>>>(p);
   }
+}
+
+// 192 x 192 tiles (block-scaled FP8 without a fused bias): the tile for row and column counts that 256-row tiles
+// cover with a part-empty round of the CUs (4096 x 2112: 242 tiles instead of 176 on 256 CUs).
+template <int KIND, int OUT_DT>
+static void launch_wide_192rows(GemmArgs& p, hipStream_t st) {
+  expand_packed_scales(p, st);
+  p.tiles_m = (p.M + 191) / 192;
+  p.tiles_n = (p.N + 191) / 192;
+  p.splits = 1;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int blocks = tiles < num_cus() ? tiles : num_cus();
+  g_last_kernel = "gemm_wide_kernel<6, 192 rows>";
+  if constexpr (KIND == KIND_FP8_BLOCK) gemm_wide_kernel<KIND, OUT_DT, 6, false, 3><<<dim3((uint32_t)blocks), dim3(512), 0, st>>>(p);
 }
 
 template <int KIND, int OUT_DT, int NI>
@@ -3199,6 +3216,10 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     int s128, s256;
     if (model_pipe_splits(p, 128, ws_bytes, s128) < model_pipe_splits(p, 256, ws_bytes, s256)) deep = false;
   }
+  if (KIND == KIND_FP8_BLOCK && t_tile == 193 && (p.K & 127) == 0 && p.K >= 384 && !p.bias) {
+    launch_wide_192rows<KIND, OUT_DT>(p, st);
+    return;
+  }
   const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 192 || t_tile == 224 || t_tile == 257;
   // (up to 128 rows a 256-row tile is half empty: 96 x 36864 x 7168 73.2 us on 192-wide tiles, 65.1 us on 128-row
   // tiles; block-scaled INT8 with one or two K blocks runs 20-35 % faster on the 128 x 128 kernel than on the
@@ -3208,6 +3229,21 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
   if ((p.K & 127) == 0 && (forced_256 || (t_tile == 0 && g_use_dma && rows_256 && (big_tiles >= 140 || deep)))) {
     int width = t_tile == 0 ? (big_tiles >= 140 ? pick_tile_width(p, KIND == KIND_I8_BLOCK && p.K <= 2048 && p.M >= 2048) : 256) : t_tile;
     if (p.K < 384 && width != 256) width = 258;  // the 4 x 2-wave kernel needs three K blocks
+    if (KIND == KIND_FP8_BLOCK && t_tile == 0 && big_tiles >= 140 && p.K >= 384 && !p.bias && !can_hw_scale<KIND, OUT_DT>(p)) {
+      // 192 x 192 tiles where they fill the rounds of the CUs better: rounds x tile area, with 22 % more time per
+      // area for the smaller tile when the chip is full (4096 x 2112 x 7168: 176 tiles of 256 x 192 take 66.2 us,
+      // 242 of 192 x 192 61.4 us; 8192 x 2112 x 7168: 132.9 -> 117 us; 4096 x 4096 x 7168, two rounds of 192 x 192
+      // against one of 256 x 256: 97 -> 116 us)
+      const int cus = num_cus();
+      const int t256 = ((p.M + 255) / 256) * ((p.N + width - 1) / (width == 258 ? 256 : width));
+      const int t192 = ((p.M + 191) / 192) * ((p.N + 191) / 192);
+      const double c256 = (double)((t256 + cus - 1) / cus) * 256.0 * (width == 258 || width == 257 ? 256 : width);
+      const double c192 = (double)((t192 + cus - 1) / cus) * 192.0 * 192.0 * 1.22;
+      if (c192 < c256) {
+        launch_wide_192rows<KIND, OUT_DT>(p, st);
+        return;
+      }
+    }
     if (width == 192) launch_wide<KIND, OUT_DT, 6>(p, st);
     else if (width == 224) launch_wide<KIND, OUT_DT, 7>(p, st);
     else if (width == 257) launch_wide<KIND, OUT_DT, 8>(p, st);
@@ -3314,7 +3350,7 @@ extern "C" int sglq_tuned_clear(void) {
   return SGLQ_OK;
 }
 extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
-  static const int tiles[] = {0, 16, 32, 64, 66, 68, 69, 128, 130, 192, 224, 256, 257, 258};
+  static const int tiles[] = {0, 16, 32, 64, 66, 68, 69, 128, 130, 192, 193, 224, 256, 257, 258};
   bool known = false;
   for (int t : tiles) known = known || t == tile;
   if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {

@@ -51,7 +51,7 @@ def candidates(m: int, n: int, k: int):
         out += [(130, s) for s in (0, 1, 2, 4, 8) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]
         out += [(258, s) for s in (0, 1, 2, 4) if s <= 1 or (nkb % s == 0 and nkb // s >= 3)]
         if m > 256:
-            out += [(192, 0), (224, 0), (257, 0)]
+            out += [(192, 0), (224, 0), (257, 0), (193, 0)]  # (193: 192 x 192 tiles, block FP8 only; elsewhere the rules' choice)
     return out
 
 

@@ -74,17 +74,17 @@ def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
 FP8 = torch.float8_e4m3fn
 
 
-def rows_per_tile(m: int, cap: int = 48, seed: int = 0) -> torch.Tensor:
+def rows_per_tile(m: int, cap: int = 48, seed: int = 0, tile: int = 0) -> torch.Tensor:
     """Rows on which a large GEMM is compared with the oracle, chosen so that every row tile of
     every kernel is read: the first, the last and one random row of each 64-row tile up to
     M = 1024 and of each 256-row tile (the persistent kernels' tile height, which also covers
     their second-round tiles and the hand-over between consecutive tiles of a block) above,
     plus one row for each of the 16 positions inside an MFMA fragment and the rows 1 and M - 2.
-    Up to `cap` rows all rows are taken."""
+    Up to `cap` rows all rows are taken.  `tile`: another tile height (the 192-row kernel)."""
     if m <= cap:
         return torch.arange(m)
     g = torch.Generator().manual_seed(1000003 * seed + m)
-    tile = 64 if m <= 1024 else 256
+    tile = tile or (64 if m <= 1024 else 256)
     rows = [0, 1, m - 2, m - 1]
     for t0 in range(0, m, tile):
         t1 = min(m, t0 + tile)

@@ -135,6 +135,34 @@ def test_fp8_blockwise_scaled_mm(gpu, load_path, tile, mnk, out_dtype):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(192, 192, 384), (193, 200, 512), (500, 2112, 1536), (1000, 640, 7168), (2048, 392, 1024), (4096, 2112, 896)])
+def test_fp8_blockwise_scaled_mm_192_row_tiles(gpu, mnk, out_dtype):
+    """The 4 x 2-wave kernel on 192 x 192 tiles (three fragment rows per wave, an epilogue of three passes): tiles cut by M
+    and by N, the shortest K it takes and a long one; rows of every row tile against the oracle, the whole output against
+    the generic 128 x 128 kernel."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lib = _lib.load()
+    say("fp8_blockwise 192-row tiles", mnk, out_dtype)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = rows_per_tile(m, 64, tile=192)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    args = (xq.to(gpu), wq.to(gpu).t(), xs.t().contiguous().to(gpu).t(), ws.to(gpu).t(), out_dtype)
+    lib.sglq_debug_force_tile(193)
+    try:
+        out = fp8_blockwise_scaled_mm(*args)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_wide_kernel<6, 192 rows>"
+        lib.sglq_debug_force_tile(128)
+        generic = fp8_blockwise_scaled_mm(*args)
+    finally:
+        lib.sglq_debug_force_tile(0)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(out.float(), generic.float(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(3, 14080, 512), (127, 512, 14080), (5, 8192, 16384), (1024, 14080, 4096), (4096, 14080, 14080)])
 def test_fp8_blockwise_scaled_mm_sizes_of_the_reference_test(gpu, mnk, out_dtype):
     """Corner points of the grid of sgl-kernel/tests/test_fp8_blockwise_gemm.py:84-87 (M from 1 to 4096,
@@ -723,7 +751,7 @@ BASELINE_KERNELS = [
     ((4096, 32768, 512), "gemm_pipe_kernel"),
     ((4096, 7168, 16384), "gemm_wide_kernel<7>"),
     ((4096, 4096, 7168), "gemm_pipe_kernel"),
-    ((4096, 2112, 7168), "gemm_wide_kernel<6>"),
+    ((4096, 2112, 7168), "gemm_wide_kernel<6, 192 rows>"),
     # decode launches of the same shapes
     ((1, 7168, 16384), "gemm_stream_kernel<16 rows>"),
     ((8, 7168, 16384), "gemm_stream_kernel<16 rows>"),
