@@ -191,6 +191,9 @@ def run_launches(args):
     dev = torch.device("cuda:0")
     if args.calibrate_copy:
         calibrate_copy(dev)
+    # --force-tile CODE: every GEMM on the kernel that sglq_debug_force_tile(CODE) names (include/sglq.h), to put a
+    # kernel that the selection rules do not pick for a shape under the profiler next to the one they do pick
+    lib.sglq_debug_force_tile(args.force_tile)
     if args.ue8m0:
         quant = lambda x: per_token_group_quant_fp8_pow2(x, 128, column_major_scales=True)
         gemm = fp8_blockwise_scaled_mm_ue8m0
@@ -240,7 +243,8 @@ def run_launches(args):
                      "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "GBs": round(nbytes / us / 1e3, 1),
                      "algorithmic_bytes": nbytes})
         del wq, x, xq
-    print(json.dumps({"launches": rows, "reps": args.launch_reps, "kind": args.kind}), flush=True)
+    lib.sglq_debug_force_tile(0)
+    print(json.dumps({"launches": rows, "reps": args.launch_reps, "kind": args.kind, "force_tile": args.force_tile}), flush=True)
 
 
 def run_ab(args):
@@ -1080,6 +1084,7 @@ def main():
     ap.add_argument("--launches", type=str, default=None,
                     help='"M,N,K;M,N,K;...": run these block-FP8 linears as plain launches in this order and exit (for profiler counter runs)')
     ap.add_argument("--launch-reps", type=int, default=5)
+    ap.add_argument("--force-tile", type=int, default=0, help="with --launches: the kernel code of sglq_debug_force_tile for every GEMM (0 = the selection rules)")
     ap.add_argument("--ab", type=str, default=None, metavar="OTHER.so",
                     help="with --launches: alternate the block-FP8 GEMM of another build of libsglq.so with the tree's in one process")
     ap.add_argument("--rotate-weights", action="store_true",
