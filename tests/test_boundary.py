@@ -176,6 +176,10 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == 1 and b"multiple of 128" in lib.sglq_last_error()
     rc = lib.sglq_per_token_group_quant_fp8_ue8m0(p, 0, p, p, 8, 256, 4, 1e-10, -448.0, 448.0, None)
     assert rc == 1 and b"column stride" in lib.sglq_last_error()
+    # packed UE8M0 activation scales: the workspace must hold the expanded scales; K a multiple of 128
+    packed = lambda k, ws_bytes: lib.sglq_fp8_blockwise_scaled_mm_ue8m0_packed(p, k, p, k, p, 1, 4, p, 1, 4, p, 16, 0, 4, 16, k, p, ws_bytes, None)
+    assert packed(256, 16) == 1 and b"workspace" in lib.sglq_last_error()
+    assert packed(192, 4096) == 1 and b"multiple of 128" in lib.sglq_last_error()
     # grouped GEMM: a [32, 128], 2 experts of [16, 128]; workspace too small, then K not a multiple of 128, then no output type
     grouped = lambda k, ws_bytes, dt: lib.sglq_fp8_blockwise_scaled_grouped_mm(
         p, k, p, k, 16 * k, p, 1, 1, p, 1, 1, 1, p, 16, dt, p, p, 2, 32, 16, k, p, ws_bytes, None)
