@@ -407,7 +407,8 @@ void sglq_debug_set_direct_lds(int on);
  * (M <= 512) with 128 weight rows per block, 66 = with 64 weight rows per block (M > 32);
  * 68 / 69 = the full-K decode kernel on 64 x 64 / 32 x 64 tiles (32 < M <= 1024, K >= 512);
  * 128 = the 128x128 kernel; 256 = the plain 256x256 kernel; 258 = the pipelined 256x256
- * kernel; 130 = the same kernel with 128-row tiles; 192 / 224 / 257 = the pipelined 4x2-wave
+ * kernel (259 = its variant whose waves write their own outputs out and whose copies run on across tile
+ * boundaries: block-scaled FP8 without bias or split-K); 130 = the same kernel with 128-row tiles; 192 / 224 / 257 = the pipelined 4x2-wave
  * kernel with tiles 192 / 224 / 256 wide; 193 = that kernel on 192 x 192 tiles (block-scaled FP8 without a bias).
  * A kernel that does not apply to the shape falls through to the next one that does. */
 void sglq_debug_force_tile(int tile);

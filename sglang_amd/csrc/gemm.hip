@@ -467,6 +467,67 @@ SGLQ_DEV void epilogue_via_lds(const GemmArgs& p, acc_t (&acc)[MI][NI], char* im
   }
 }
 
+// Epilogue of PIPE_DIRECT: every wave turns its own accumulators into whole 128-byte row pieces through 2 KiB of
+// LDS that no other wave touches, one fragment row (16 rows x 64 columns) at a time: four 8-byte writes per lane
+// (the lane's four columns of each fragment), then two 16-byte reads and two stores of 8 rows x 128 bytes.  No
+// block barrier and no stage buffer: LDS operations of a wave execute in order.  Chunk c (16 bytes) of row r sits
+// at chunk position c ^ (r & 7) ^ (r >> 3).  Tiles cut by N (or rows too far apart for 31-bit offsets) take guarded
+// stores and then wait for everything outstanding, so that the caller's count of younger operations stays an upper bound.
+template <int OUT_DT, int MI, int NI, int BM, int BN, typename acc_t>
+SGLQ_DEV void epilogue_direct(const GemmArgs& p, acc_t (&acc)[MI][NI], char* mine, int m0, int n0, int row0, int col0, int r16, int g,
+                              int lane) {
+  static_assert(NI == 4, "a wave's 64 columns are one 128-byte line of 16-bit outputs");
+  asm volatile("" : "+v"(r16), "+v"(g), "+v"(lane));  // (keep the lane arithmetic here, as in epilogue_via_lds)
+  char* out = reinterpret_cast<char*>(p.out);
+  const uint32_t row_bytes = (uint32_t)p.ldo * 2u;
+  const int rows_left = p.M - m0 < BM ? p.M - m0 : BM;
+  const bool whole = n0 + BN <= p.N && p.ldo < (1 << 21);
+  const __amdgpu_buffer_rsrc_t r_out =
+      make_rsrc(out + ((int64_t)m0 * p.ldo + n0) * 2, whole ? (uint32_t)rows_left * row_bytes - (uint32_t)n0 * 2u : 0u);
+  const int swz_w = (r16 & 7) ^ (r16 >> 3);
+  char* const wr = mine + r16 * 128 + (g & 1) * 8;
+  const int c = lane & 7, r8 = lane >> 3;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      char* dst = wr + (((j * 2 + (g >> 1)) ^ swz_w) * 16);
+      if constexpr (OUT_DT == SGLQ_BF16) {
+        typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<bf4*>(dst) = bf4{(__bf16)acc[i][j][0], (__bf16)acc[i][j][1], (__bf16)acc[i][j][2], (__bf16)acc[i][j][3]};
+      } else {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<h4*>(dst) = h4{(_Float16)acc[i][j][0], (_Float16)acc[i][j][1], (_Float16)acc[i][j][2], (_Float16)acc[i][j][3]};
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
+    __builtin_amdgcn_wave_barrier();
+    v4i v[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = h * 8 + r8;
+      v[h] = *reinterpret_cast<const v4i*>(mine + r * 128 + ((c ^ (r & 7) ^ (r >> 3)) * 16));
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
+    __builtin_amdgcn_wave_barrier();
+    if (whole) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t voff = (uint32_t)(row0 + i * 16 + h * 8 + r8) * row_bytes + (uint32_t)(col0 * 2 + c * 16);
+        if (p.stream_out) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[h]), r_out, voff, 0, 2);
+        else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[h]), r_out, voff, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int m = m0 + row0 + i * 16 + h * 8 + r8, n = n0 + col0 + c * 8;
+        if (m < p.M && n + 8 <= p.N) *reinterpret_cast<v4i*>(out + ((int64_t)m * p.ldo + n) * 2) = v[h];
+      }
+    }
+  }
+  if (!whole) __builtin_amdgcn_s_waitcnt(0);
+}
+
 // GROUPED: one launch for a group of problems that share N and K (the experts of an MoE
 // layer).  Row tile t of the grid belongs to expert plan[t].expert and covers rows
 // plan[t].row0 .. of A and C up to the expert's last row; B and its scales are the
@@ -918,7 +979,12 @@ __global__ __launch_bounds__(512) void gemm_big_kernel(const GemmArgs p) {
 // plain one keeps its register allocation: 0 = whole tiles, 1 = split-K work units (raw
 // partial sums to the workspace), 2 = whole tiles of a block-scaled kind with a bias,
 // 3 = grouped GEMM (row tiles and their experts from the plan in the workspace).
-constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2, PIPE_GROUPED = 3;
+constexpr int PIPE_PLAIN = 0, PIPE_SPLITK = 1, PIPE_BIAS = 2, PIPE_GROUPED = 3, PIPE_DIRECT = 4;
+// 4 = whole tiles whose outputs every wave brings into row order by itself (epilogue_direct: 2 KiB of LDS per
+// wave, no block barrier): no stage is needed at a tile's end, so the copies run on across tile boundaries without the deferral,
+// and the next tile's first K blocks are older in the vector-memory queue than the tile's stores: the steps that
+// wait for them do not wait for the stores (vector-memory operations retire in order).  For short K, where
+// the stores of a 256 x 256 tile every four to twelve steps are what the other variants stall on.
 // BM = 128: tiles of 128 rows (a wave owns 64 x 64, 16 MFMAs per step) for problems whose
 // 256-row tiles would leave most of the chip idle; same schedule, half the activation copies.
 template <int KIND, int OUT_DT, int MODE, int BM = 256>
@@ -931,11 +997,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   constexpr bool BLOCK = is_block(KIND);
   constexpr bool HW = KIND == KIND_FP8_BLOCK_POW2;  // the MFMA applies the block scales
   constexpr bool FOLD = BLOCK && !HW;               // they are applied to each MFMA's result
+  constexpr bool DIRECT = MODE == PIPE_DIRECT;      // outputs stored from the accumulators; uniform steps across tile boundaries
   static_assert(NI == 4 && (MI == 8 || MI == 4), "the copy schedule below is written for 4 x 8 or 4 x 4 fragments");
+  static_assert(!DIRECT || (MI == 8 && BLOCK), "PIPE_DIRECT is built for the block-scaled kinds on 256-row tiles");
 
   constexpr int SCALE_BYTES = 2048;  // per K block: 256 activation-row scales, then the tile's two weight scales
   // (one LDS object per kernel, see gemm_big_kernel: the epilogue's 512 floats sit at the end)
-  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES + 2048];
+  // (PIPE_DIRECT: 2 KiB more per wave, the wave's own part of the epilogue)
+  __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE_BYTES + 2 * SCALE_BYTES + 2048 + (MODE == PIPE_DIRECT ? NW * 2048 : 0)];
   float* const col_lds = reinterpret_cast<float*>(smem + 2 * STAGE_BYTES + 2 * SCALE_BYTES);
 
   const int lane = threadIdx.x & 63;
@@ -1058,9 +1127,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
   // One K step: block u sits in stage `cur` and its first fragments are in bf / a_cur.
   // kn: index, inside its tile, of block u + 1 (scales, and the copies deferred to a tile's
   // first step); kn2: that of block u + 2 (off_a2 / off_b2).
-  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag) {
+  // (PIPE_DIRECT: every step copies like a middle step; stores_tag: the tile before this first step has just
+  // issued its 2 MI stores, which are younger than block u + 1's copies)
+  auto k_step = [&](int cur, int kn, int kn2, auto first_tag, auto last_tag, auto stores_tag) {
     constexpr bool first = decltype(first_tag)::value;
     constexpr bool last = decltype(last_tag)::value;
+    constexpr bool after_stores = decltype(stores_tag)::value;
+    constexpr bool refill = !last;             // read block u + 1's first fragments and scales behind their last use
+    constexpr bool copies = !last || DIRECT;   // issue the copies of block u + 2
     const char* st = smem + cur * STAGE_BYTES;
     const char* sn = smem + (cur ^ 1) * STAGE_BYTES;
     float sc = 0.f, sc_prev = 0.f;
@@ -1076,7 +1150,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         sc = sfa_cur[i] * sfb_cur;
       }
       if constexpr (HW) ea = ue8m0_at(sfa_cur[i], sh_cur);
-      if (i == 1 && !last) {
+      if (i == 1 && copies) {
         // barrier 1: MFMAs 0..3 have consumed this wave's weight fragments, so its LDS reads
         // of block u's weights are complete; behind the barrier that holds for every wave.
         __builtin_amdgcn_s_barrier();
@@ -1090,7 +1164,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         // and scales are complete.  A bare s_barrier: these waits are all the ordering needed.
         // (with 16 MFMAs per step the first step's weight copies of block u + 2 come behind
         // this barrier, and what is in flight here are the deferred copies of block u + 1)
-        constexpr int YOUNGER = (last || (first && MI == 4)) ? 0 : 4;
+        constexpr int YOUNGER = DIRECT ? 4 + (after_stores ? 2 * MI : 0) : ((last || (first && MI == 4)) ? 0 : 4);
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(YOUNGER));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -1127,26 +1201,32 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
           // weight fragment j has had its last use in this step: refill it from block u + 1
           // (not in a tile's last step: the next tile's first fragments and scales are read behind
           // the epilogue, which needs the registers)
-          if constexpr (!last) {
+          if constexpr (refill) {
             bf[j] = read_frag(sn + b_base + j * 16 * 128);
             if (j == 0) a_nxt = read_frag(sn + a_base);
+          }
+          if constexpr (copies) {
             if (j < NCOPY_A) copy_a(j, cur, kn2 * 128, off_a2);
-            if constexpr (BLOCK) {
+          }
+          if constexpr (BLOCK) {
+            if constexpr (refill) {
               // scales i < MI - 1 had their last use when the last fragment's scale was formed; its own
               // scale and sfb_cur are dead as well: `sc` holds their product (HW: `ea` and `eb` their exponents)
 #pragma unroll
               for (int q = 0; q < MI / NI; ++q) sfa_cur[(MI / NI) * j + q] = read_sfa(cur ^ 1, (MI / NI) * j + q);
               if (j == 0) sfb_cur = read_sfb(cur ^ 1);
+            }
+            if constexpr (copies) {
               if (j == 0) copy_scales(cur, kn2, sc_off2);
             }
           }
         }
-        if constexpr (first) {
+        if constexpr (first && !DIRECT) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur ^ 1, kn * 128, off_b, false);
           if (idx >= 8 && idx < 8 + NCOPY_A) copy_a(idx - 8, cur ^ 1, kn * 128, off_a);
           if (BLOCK && idx == 11) copy_scales(cur ^ 1, kn, sc_off);
           if (idx >= 12 && idx < 16) copy_b(idx - 12, cur, kn2 * 128, off_b2, true);
-        } else if constexpr (!last) {
+        } else if constexpr (copies) {
           if (idx >= 4 && idx < 8) copy_b(idx - 4, cur, kn2 * 128, off_b2, true);
         }
         if constexpr (FOLD) {
@@ -1170,7 +1250,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
         acc[MI - 1][NI - 1][e] = first ? block_value<KIND>(part_prev[e]) * sc
                                        : __builtin_fmaf(block_value<KIND>(part_prev[e]), sc, acc[MI - 1][NI - 1][e]);
     }
-    if constexpr (HW && !last) sh_cur = code_shift(kn);  // sfa_cur now holds block u + 1's words
+    if constexpr (HW && refill) sh_cur = code_shift(kn);  // sfa_cur now holds block u + 1's words
   };
 
   // ---- persistent walk over the work units blockIdx, blockIdx + gridDim, ...  A unit is an
@@ -1228,6 +1308,14 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     }
   };
   read_first(0);
+  if constexpr (DIRECT) {
+    // the steps of this variant expect block u + 1's copies to be under way when step u starts
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_b(j, 1, (kb0 + 1) * 128, off_b, false);
+#pragma unroll
+    for (int j = 0; j < NCOPY_A; ++j) copy_a(j, 1, (kb0 + 1) * 128, off_a);
+    if constexpr (BLOCK) copy_scales(1, kb0 + 1, sc_off);
+  }
 
   while (true) {
     // The block's next unit; past its last one the prefetches are pointed at rows beyond M
@@ -1247,18 +1335,25 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     const uint32_t off_a_next = a_offset(nm0), off_b_next = b_offset(nn0);
     uint32_t sc_off_next = SC_NONE;
     if constexpr (BLOCK) sc_off_next = scale_offset(nm0, nn0, nexpert);
-    k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{});
+    if constexpr (DIRECT) {
+      if (unit == (int)blockIdx.x) k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{}, std::false_type{});
+      else k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{}, std::true_type{});  // behind the last tile's stores
+    } else {
+      k_step(par, kb0 + 1, kb0 + 2, std::true_type{}, std::false_type{}, std::false_type{});
+    }
     for (int kb = 1; kb + 1 < nkb; ++kb) {
       const bool pen = kb + 2 == nkb;  // the block two ahead is the next unit's first
       off_a2 = pen ? off_a_next : off_a2;
       off_b2 = pen ? off_b_next : off_b2;
       sc_off2 = pen ? sc_off_next : sc_off2;
       if constexpr (MODE == PIPE_GROUPED) b_two = pen ? b_next : b_two;
-      k_step((kb + par) & 1, kb0 + kb + 1, pen ? nkb0 : kb0 + kb + 2, std::false_type{}, std::false_type{});
+      k_step((kb + par) & 1, kb0 + kb + 1, pen ? nkb0 : kb0 + kb + 2, std::false_type{}, std::false_type{}, std::false_type{});
     }
     // last K block: its copies (the next unit's second block) wait for the next unit's first step
+    // (PIPE_DIRECT: they are issued here like any other step's)
     const int last_stage = (nkb - 1 + par) & 1;
-    k_step(last_stage, 0, 0, std::false_type{}, std::true_type{});
+    if constexpr (DIRECT) k_step(last_stage, nkb0, nkb0 + 1, std::false_type{}, std::true_type{}, std::false_type{});
+    else k_step(last_stage, 0, 0, std::false_type{}, std::true_type{}, std::false_type{});
     off_a = off_a2;
     off_b = off_b2;
     sc_off = sc_off2;
@@ -1266,7 +1361,16 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
 
     // Every wave has passed the last step's barrier: nobody reads `last_stage` any more and
     // nothing is being copied into it, so it stages the C tile.
-    if constexpr (MODE == PIPE_SPLITK) {
+    if constexpr (DIRECT) {
+      // (pin the accumulators here: left alone, the compiler sinks the last folds into the epilogue's blocks and
+      // spills their operands across the step's tail)
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) asm volatile("" : "+v"(acc[i][j]));
+      epilogue_direct<OUT_DT, MI, NI, BM, BN>(p, acc, smem + 2 * STAGE_BYTES + 2 * SCALE_BYTES + 2048 + wave * 2048, m0, n0, wm * TM, wn * TN, r16, g,
+                                              lane);
+    } else if constexpr (MODE == PIPE_SPLITK) {
       store_partials_bounded<MI, NI>(p, acc, unit / tiles, m0 + wm * TM, n0 + wn * TN, r16, g);
     } else if constexpr (KIND == KIND_I8_RAW) {
       epilogue<KIND, OUT_DT, MI, NI>(p, acc, m0 + wm * TM, n0 + wn * TN, r16, g);
@@ -1289,6 +1393,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmArgs p) {
     par = last_stage ^ 1;
     read_first(par);  // (landed before the last step's second barrier)
   }
+  // (PIPE_DIRECT: the last step's copies, pointed beyond the operands, still write zeros into LDS)
+  if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0);
 }
 
 // ---------------------------------------------------------------------------
@@ -2663,8 +2769,12 @@ static void launch_cfg(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
 // 256 = the plain 256 x 256 kernel, 258 = the pipelined one (K >= 384, else the plain one),
 // 192 / 224 / 257 = the 4 x 2-wave kernel with tiles 192, 224, 256 wide (K >= 384, else as 258),
 // 193 = that kernel on 192 x 192 tiles (block-scaled FP8 without a bias, K >= 384; else the heuristic),
+// 259 = as 258 with the wave-private epilogue and copies that run on across tile boundaries (block-scaled FP8, no bias, no split),
 // 130 = the pipelined kernel with 128-row tiles (K >= 384, else the 128 x 128 kernel)
 static thread_local int g_force_tile = 0;
+#ifndef SGLQ_DIRECT_MAX_K
+#define SGLQ_DIRECT_MAX_K 4096
+#endif
 
 static double model_pipe_splits(const GemmArgs& p, int rows_per_tile, int64_t ws_bytes, int& splits);
 
@@ -2749,7 +2859,20 @@ static void launch_big(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     } else if (is_block(KIND) && p.bias) {
       if constexpr (is_block(KIND)) gemm_pipe_kernel<KIND, OUT_DT, PIPE_BIAS><<<grid, block, 0, st>>>(p);
     } else if (hw_scaled<KIND, OUT_DT>(p)) {
-      if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
+      if constexpr (KIND == KIND_FP8_BLOCK && OUT_DT == SGLQ_BF16) {
+        if (t_tile == 259 || (t_tile == 0 && p.K <= SGLQ_DIRECT_MAX_K)) {
+          g_last_kernel = "gemm_pipe_kernel<direct stores>";
+          gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_DIRECT><<<grid, block, 0, st>>>(p);
+        } else {
+          gemm_pipe_kernel<KIND_FP8_BLOCK_POW2, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
+        }
+      }
+    } else if (KIND == KIND_FP8_BLOCK && (t_tile == 259 || (t_tile == 0 && p.K <= SGLQ_DIRECT_MAX_K))) {
+      // (measured against the plain variant at M = 4096: K = 1024 76.2 -> 70.4 us, 1536 149.2 -> 140.3, 2048 125.2 -> 117.7,
+      // 3072 177.5 -> 176.2, 4096 222.4 -> 218.6, 7168 95.6 -> 95.1; K = 512 within 1 %: four steps per tile are too few
+      // to keep the stores of one tile out of the way of the next)
+      g_last_kernel = "gemm_pipe_kernel<direct stores>";
+      if constexpr (KIND == KIND_FP8_BLOCK) gemm_pipe_kernel<KIND, OUT_DT, PIPE_DIRECT><<<grid, block, 0, st>>>(p);
     } else {
       gemm_pipe_kernel<KIND, OUT_DT, PIPE_PLAIN><<<grid, block, 0, st>>>(p);
     }
@@ -3220,7 +3343,7 @@ static void launch_kind(GemmArgs& p, int64_t ws_bytes, hipStream_t st) {
     launch_wide_192rows<KIND, OUT_DT>(p, st);
     return;
   }
-  const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 192 || t_tile == 224 || t_tile == 257;
+  const bool forced_256 = t_tile == 256 || t_tile == 258 || t_tile == 259 || t_tile == 192 || t_tile == 224 || t_tile == 257;
   // (up to 128 rows a 256-row tile is half empty: 96 x 36864 x 7168 73.2 us on 192-wide tiles, 65.1 us on 128-row
   // tiles; block-scaled INT8 with one or two K blocks runs 20-35 % faster on the 128 x 128 kernel than on the
   // unpipelined 256 x 256 one: 4096 x 7168 x 128 33.0 -> 27.3 us, 3072 x 7168 x 256 35.7 -> 26.2 us)
@@ -3350,7 +3473,7 @@ extern "C" int sglq_tuned_clear(void) {
   return SGLQ_OK;
 }
 extern "C" int sglq_tuned_add(int kind, int64_t N, int64_t K, int64_t m_lo, int64_t m_hi, int tile, int splits) {
-  static const int tiles[] = {0, 16, 32, 64, 66, 68, 69, 128, 130, 192, 193, 224, 256, 257, 258};
+  static const int tiles[] = {0, 16, 32, 64, 66, 68, 69, 128, 130, 192, 193, 224, 256, 257, 258, 259};
   bool known = false;
   for (int t : tiles) known = known || t == tile;
   if (kind < 0 || kind > 4 || N <= 0 || K <= 0 || m_lo < 0 || m_hi < m_lo || !known || splits < 0 || splits > 64) {

@@ -163,6 +163,37 @@ def test_fp8_blockwise_scaled_mm_192_row_tiles(gpu, mnk, out_dtype):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk", [(256, 256, 384), (300, 520, 512), (1000, 1288, 1536), (2048, 4096, 512), (4096, 16640, 512), (515, 768, 7168)])
+def test_fp8_blockwise_scaled_mm_direct_stores(gpu, mnk, out_dtype):
+    """The pipelined 256 x 256 kernel that stores from the accumulators and copies on across tile boundaries: tiles cut
+    by M, tiles cut by N (guarded stores), the shortest K, one tile per block and several (the first step behind a tile's
+    stores); rows of every row tile against the oracle, the whole output against the generic 128 x 128 kernel."""
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lib = _lib.load()
+    say("fp8_blockwise direct stores", mnk, out_dtype)
+    m, n, k = mnk
+    _, xq, xs, wq, ws = make_block_case(m, n, k, seed=m + n + k, outliers=True)
+    rows = rows_per_tile(m, 48)
+    ref = O.fp8_blockwise_scaled_mm(xq[rows], wq.t(), xs[rows], ws.t(), torch.float32, acc_dtype=torch.float64)
+    args = (xq.to(gpu), wq.to(gpu).t(), xs.t().contiguous().to(gpu).t(), ws.to(gpu).t(), out_dtype)
+    lib.sglq_debug_force_tile(259)
+    lib.sglq_debug_force_splits(1)
+    try:
+        out = fp8_blockwise_scaled_mm(*args)
+        assert lib.sglq_debug_last_gemm_kernel().decode() == "gemm_pipe_kernel<direct stores>"
+        lib.sglq_debug_force_tile(128)
+        lib.sglq_debug_force_splits(0)
+        generic = fp8_blockwise_scaled_mm(*args)
+    finally:
+        lib.sglq_debug_force_tile(0)
+        lib.sglq_debug_force_splits(0)
+    torch.testing.assert_close(out.cpu()[rows].float(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(out.float(), generic.float(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(3, 14080, 512), (127, 512, 14080), (5, 8192, 16384), (1024, 14080, 4096), (4096, 14080, 14080)])
 def test_fp8_blockwise_scaled_mm_sizes_of_the_reference_test(gpu, mnk, out_dtype):
     """Corner points of the grid of sgl-kernel/tests/test_fp8_blockwise_gemm.py:84-87 (M from 1 to 4096,
@@ -747,8 +778,8 @@ def test_narrow_weights_and_few_rows(gpu, mnk, kernel):
 
 BASELINE_KERNELS = [
     # (M, N, K) of the headline step and the kernel the profile summaries under profiles/ name for it
-    ((4096, 24576, 1536), "gemm_pipe_kernel"),
-    ((4096, 32768, 512), "gemm_pipe_kernel"),
+    ((4096, 24576, 1536), "gemm_pipe_kernel<direct stores>"),
+    ((4096, 32768, 512), "gemm_pipe_kernel<direct stores>"),
     ((4096, 7168, 16384), "gemm_wide_kernel<7>"),
     ((4096, 4096, 7168), "gemm_pipe_kernel"),
     ((4096, 2112, 7168), "gemm_wide_kernel<6, 192 rows>"),
