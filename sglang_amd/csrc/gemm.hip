@@ -487,8 +487,10 @@ SGLQ_DEV void epilogue_direct(const GemmArgs& p, acc_t (&acc)[MI][NI], char* min
   const int swz_w = (r16 & 7) ^ (r16 >> 3);
   char* const wr = mine + r16 * 128 + (g & 1) * 8;
   const int c = lane & 7, r8 = lane >> 3;
-#pragma unroll
-  for (int i = 0; i < MI; ++i) {
+  // LDS operations of a wave execute in the order of the program: the reads of fragment row i see its writes and are
+  // done before the writes of row i + 1 land, with no wait in between.  The only waits are the ones for the data of
+  // row i's reads in front of its stores, which are issued behind the LDS operations of row i + 1 (the compiler places them).
+  auto to_lds = [&](int i) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       char* dst = wr + (((j * 2 + (g >> 1)) ^ swz_w) * 16);
@@ -500,16 +502,15 @@ SGLQ_DEV void epilogue_direct(const GemmArgs& p, acc_t (&acc)[MI][NI], char* min
         *reinterpret_cast<h4*>(dst) = h4{(_Float16)acc[i][j][0], (_Float16)acc[i][j][1], (_Float16)acc[i][j][2], (_Float16)acc[i][j][3]};
       }
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
-    __builtin_amdgcn_wave_barrier();
-    v4i v[2];
+  };
+  auto from_lds = [&](v4i (&v)[2]) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int r = h * 8 + r8;
       v[h] = *reinterpret_cast<const v4i*>(mine + r * 128 + ((c ^ (r & 7) ^ (r >> 3)) * 16));
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0_only());
-    __builtin_amdgcn_wave_barrier();
+  };
+  auto to_memory = [&](int i, const v4i (&v)[2]) {
     if (whole) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
@@ -524,7 +525,22 @@ SGLQ_DEV void epilogue_direct(const GemmArgs& p, acc_t (&acc)[MI][NI], char* min
         if (m < p.M && n + 8 <= p.N) *reinterpret_cast<v4i*>(out + ((int64_t)m * p.ldo + n) * 2) = v[h];
       }
     }
+  };
+  v4i v[2][2];
+  to_lds(0);
+  __builtin_amdgcn_wave_barrier();
+  from_lds(v[0]);
+#pragma unroll
+  for (int i = 1; i < MI; ++i) {
+    __builtin_amdgcn_wave_barrier();
+    to_lds(i);
+    __builtin_amdgcn_wave_barrier();
+    from_lds(v[i & 1]);
+    __builtin_amdgcn_sched_barrier(0);
+    to_memory(i - 1, v[(i - 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
   }
+  to_memory(MI - 1, v[(MI - 1) & 1]);
   if (!whole) __builtin_amdgcn_s_waitcnt(0);
 }
 
